@@ -1,0 +1,179 @@
+"""Benchmark of the hot path on one MI355X: fp16 block-64 sparse self-attention, forward + backward.
+
+Workload (the configuration the headline metric is quoted on): batch 8, 16 heads, sequence 4096, head_dim 64,
+block 64, fixed Sparse-Transformer layout (local window of 4 blocks + one global block column per 16 blocks,
+causal), softmax scale 1/8 and an additive key-padding mask hiding the last 0-25% of the keys of each sequence.
+One step = sdd(q, k^T) -> softmax -> dsd(p, v), then the backward pass (softmax backward and four matmuls).
+
+Prints one JSON line.  `value` is the effective matmul throughput of the whole step: the FLOPs of the six
+block-sparse products over their nonzero blocks (2*Z*64*nnz*64^2 each, the reference's formula,
+tests/test_matmul.py:82-84) divided by the wall time of the full step, softmax included.  `kernels` lists every
+launch of the step with its own HIP-event time, effective TFLOP/s or GB/s and roofline fractions; `roofline`
+repeats the entry of the launch that takes the largest share of the step.  `cpu_baseline` is the same chain
+computed by the fp32 dense-masked oracle on the host cores, on a slice of the batch.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, 'torch-blocksparse_amd')):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=30)
+    ap.add_argument('--warmup', type=int, default=5)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--batch', type=int, default=8)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit('bench.py measures one GPU: the path shards over batch and heads without communication, '
+                 'and no multi-GPU run is part of this build (got --gpus %d)' % args.gpus)
+
+    import torch
+    import torch_blocksparse as tb
+    from torch_blocksparse.matmul import _sparse_matmul
+    dev = torch.device('cuda:0')
+    torch.manual_seed(0)
+    B, H, L, dh, block = args.batch, 16, 4096, 64, 64
+    dtype = torch.float16
+    scale = 0.125
+    lay = tb.sparse_transformer_layout(H, L // block, 4, 16, True)
+    nnz = int(lay.sum())
+    q, k, v, do = [torch.randn(B, H, L, dh, dtype=dtype, device=dev) for _ in range(4)]
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    g = torch.Generator().manual_seed(1)
+    kpm = torch.zeros(B, L, dtype=dtype)
+    for z in range(B):
+        pad = int(torch.randint(0, L // 4 + 1, (1,), generator=g))
+        if pad:
+            kpm[z, L - pad:] = float('-inf')
+    kpm = kpm.to(dev)
+    sdd = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=True)
+    dsd = tb.MatMul(lay, block, 'dsd')
+    sm = tb.Softmax(lay, block)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        w = sdd(q, k)
+        p = sm(w, scale=scale, key_padding_mask=kpm)
+        o = dsd(p, v)
+        o.backward(do)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    flops_mm = 2.0 * B * dh * nnz * block * block          # per product (K = N = M = head_dim in all six)
+    es = 2
+    x_bytes = B * nnz * block * block * es
+    dense_bytes = B * H * L * dh * es
+    mm_bytes = x_bytes + 2 * dense_bytes                    # one sparse tensor + two dense tensors, each touched once
+
+    # per-launch timing with HIP events on the launch stream
+    luts = {m: m.make_lut(dtype, dev) for m in (sdd, dsd)}
+    sm_lut, sm_maxlut = sm.make_lut(dev)
+    t = [None]
+    with torch.no_grad():
+        w = sdd(q, k)
+        p = sm(w.clone(), scale=scale, key_padding_mask=kpm)
+        dp = torch.randn_like(p)
+    fn = _sparse_matmul.fn
+    sl, dl = luts[sdd], luts[dsd]
+    spd = lay.shape
+    launches = {
+        # forward
+        'sdd_fwd  q.k^T': (lambda: fn['sdd'](q, k, False, True, False, spd, block, sl[0], sl[1], sl[2], sl[3], False, t), flops_mm, mm_bytes),
+        'softmax_fwd': (lambda: tb.Softmax.sparse_softmax(w, scale, None, kpm, None, 'add', 'add', spd, block, sm_lut, sm_maxlut, False, t), 0.0, 2 * x_bytes + kpm.numel() * es),
+        'dsd_fwd  p.v': (lambda: fn['dsd'](p, v, False, False, False, spd, block, dl[0], dl[1], dl[2], dl[3], False, t), flops_mm, mm_bytes),
+        # backward of dsd: dp = sdd(do, v^T), dv = dsd(p^T, do)
+        'sdd_bwd  do.v^T': (lambda: fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t), flops_mm, mm_bytes),
+        'dsd_bwd  p^T.do': (lambda: fn['dsd'](p, do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t), flops_mm, mm_bytes),
+        'softmax_bwd': (lambda: _bwd_softmax(tb, p, dp, scale, sm_lut, sm_maxlut, spd, block), 0.0, 3 * x_bytes),
+        # backward of sdd: dq = dsd(ds, k), dk = dds(q^T, ds) written transposed
+        'dsd_bwd  ds.k': (lambda: fn['dsd'](dp, k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t), flops_mm, mm_bytes),
+        'dds_bwd  (q^T.ds)^T': (lambda: fn['dds'](q, dp, True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t), flops_mm, mm_bytes),
+    }
+    kernels = {}
+    with torch.no_grad():
+        for name, (f, flops, nbytes) in launches.items():
+            for _ in range(3):
+                f()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            reps = max(args.steps, 10)
+            e0.record()
+            for _ in range(reps):
+                f()
+            e1.record()
+            e1.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
+                   'bytes': nbytes}
+            if flops:
+                ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
+                ent['mfma_frac'] = round(flops / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)
+            kernels[name] = ent
+    dom = max(kernels, key=lambda n: kernels[n]['ms'])
+    roofline = {'kernel': dom, 'bound': 'hbm', 'achieved': kernels[dom]['GB/s'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': kernels[dom]['hbm_frac'], 'traffic': None}
+
+    out = {
+        'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk64',
+        'value': round(6 * flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f16', 'data': 'synthetic',
+        'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block 64, fixed '
+                               'layout (local 4 blocks + 1 global per 16, causal), scale 1/8, additive key-padding mask' % B,
+                   'nnz_blocks': nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
+        'softmax_GB/s': {'fwd': kernels['softmax_fwd']['GB/s'], 'bwd': kernels['softmax_bwd']['GB/s']},
+        'roofline': roofline, 'kernels': kernels,
+    }
+    if not args.no_cpu_baseline:
+        out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, L)
+    print(json.dumps(out))
+
+
+def _bwd_softmax(tb, y, dy, scale, lut, maxlut, spdims, block):
+    import ctypes
+    from torch_blocksparse import _lib
+    rc = _lib.load().bsp_softmax_bwd(_lib.DTYPES[y.dtype], _lib.ptr(y), _lib.ptr(dy), float(scale), _lib.ptr(lut), maxlut,
+                                     y.size(0), spdims[0], spdims[1], block, y.stride(0), dy.stride(0), _lib.stream_ptr(y.device))
+    _lib.check(rc, 'bsp_softmax_bwd')
+
+
+def cpu_baseline(lay, block, dh, scale, L):
+    """The reference's CPU path = its test oracle: dense fp32 matmuls + layout mask + dense softmax, forward and
+    backward (oracle/dense_oracle.py).  Timed on a slice of the workload (1 sequence, all 16 heads)."""
+    import torch
+    from oracle import dense_oracle as D
+    torch.manual_seed(0)
+    Bs, H = 1, lay.shape[0]
+    q, k, v, do = [torch.randn(Bs, H, L, dh) for _ in range(4)]
+    kpm = torch.zeros(Bs, L)
+    kpm[0, L - L // 8:] = float('-inf')
+    D.attention(q[:, :1], k[:, :1], v[:, :1], lay[:1], block, scale, key_padding_mask=kpm, do=do[:, :1])   # warm-up
+    t0 = time.perf_counter()
+    D.attention(q, k, v, lay, block, scale, key_padding_mask=kpm, do=do)
+    dt = time.perf_counter() - t0
+    flops = 6 * 2.0 * Bs * dh * int(lay.sum()) * block * block
+    return {'value': round(flops / dt * 1e-12, 5), 'unit': 'TFLOP/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+            'sample': 'same chain fwd+bwd on 1 of the 8 sequences (16 heads, seq 4096), fp32 dense matmul + mask + softmax, '
+                      '%.1f s; throughput counts only the nonzero-block FLOPs, like the GPU figure' % dt}
+
+
+if __name__ == '__main__':
+    main()

@@ -1,0 +1,128 @@
+/*
+ * bsp.h -- C ABI of the MI355X (gfx950) block-sparse matmul / softmax library.
+ *
+ * Everything here takes plain device pointers, sizes and element strides; no framework types cross the
+ * boundary.  All launches are asynchronous on the given HIP stream (a hipStream_t passed as void*; NULL is
+ * the default stream).  The look-up-table builders additionally copy a few scalars back to the host and
+ * therefore synchronise that stream once before they return.  No function allocates or frees device
+ * memory: outputs, tables and workspaces are provided by the caller.
+ *
+ * Each entry point names the interface of ptillet/torch-blocksparse that it replaces (file:line of the
+ * reference checkout).  Sparse tensors use the reference's storage: [Z, nnz, block, block], block p being
+ * the p-th nonzero of the [H, R, C] layout in row-major (head, block-row, block-col) order.
+ *
+ * Return value: 0 on success, a negative bsp_status otherwise (bsp_strerror gives the text).
+ */
+#ifndef BSP_H
+#define BSP_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum { BSP_F16 = 0, BSP_BF16 = 1, BSP_F32 = 2 } bsp_dtype;
+
+typedef enum {
+  BSP_OK = 0,
+  BSP_ERR_ARG = -1,          /* null pointer, bad size, misaligned operand */
+  BSP_ERR_UNSUPPORTED = -2,  /* block size / dtype / mode not built */
+  BSP_ERR_CAPACITY = -3,     /* caller-provided table or workspace too small */
+  BSP_ERR_EMPTY_HEAD = -4,   /* a head of the layout has no nonzero block (the reference raises here) */
+  BSP_ERR_HIP = -5,          /* a HIP runtime call failed */
+  BSP_ERR_ROW_TOO_LONG = -6, /* softmax row of >= 32768 elements (reference softmax.py:225-227) */
+  BSP_ERR_K_MULTIPLE = -7    /* sdd reduction size not a multiple of 16 (reference matmul.py:318-319) */
+} bsp_status;
+
+int bsp_version(void);
+const char *bsp_strerror(int status);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Look-up-table builders.  d_layout is the layout as int32 [H, R, C] in device memory (0/1 values).
+ * d_ws is scratch of at least bsp_lut_workspace_bytes(H, R, C) bytes.
+ * ------------------------------------------------------------------------------------------------- */
+int64_t bsp_lut_workspace_bytes(int H, int R, int C);
+
+/* Number of nonzero blocks of a layout (host result).  Replaces layout.sum() / layout.nonzero().size(0). */
+int bsp_layout_nnz(const int32_t *d_layout, int H, int R, int C, void *d_ws, int64_t ws_bytes, int64_t *nnz, void *stream);
+
+/* softmax table: replaces _sparse_softmax.make_lut (softmax.py:201-221).
+ * d_lut receives 2*H*R + 4*nnz int32: per block-row (size, offset), then per block (blockid, col, row, head).
+ * *maxlut = largest number of blocks in a block-row. */
+int bsp_softmax_lut_build(const int32_t *d_layout, int H, int R, int C, int32_t *d_lut, int64_t lut_cap,
+                          void *d_ws, int64_t ws_bytes, int64_t *lut_len, int *maxlut, void *stream);
+
+/* dsd/dds table: replaces _sparse_matmul.make_dxx_lut + load_balance (matmul.py:221-267, 372-458).
+ * d_lut receives 6*width header ints (offset, segment length, column, depth, lockid, maxid), then the
+ * 2*nnz*(block/step) interleaved pointer increments and two trailing zeros -- bit-identical to the reference.
+ * d_plan (int32 [2*nnz]) receives, per block in table order, (offset of the block in the dense operand's
+ * reduction dimension, storage index of the block): the absolute positions the increments are differences
+ * of; the matmul launchers below read them instead of re-summing the increments.
+ * lut_cap >= bsp_dxx_lut_cap(...). */
+int64_t bsp_dxx_lut_cap(int H, int R, int C, int64_t nnz, int block, int step, int trans);
+int bsp_dxx_lut_build(const int32_t *d_layout, int H, int R, int C, int block, int step, int trans,
+                      int32_t *d_lut, int64_t lut_cap, int32_t *d_plan, void *d_ws, int64_t ws_bytes,
+                      int64_t *lut_len, int *width, int *num_locks, void *stream);
+
+/* sdd table: replaces _sparse_matmul.make_sdd_lut + torch_blocksparse_cpp_utils.sdd_segment
+ * (matmul.py:281-297, csrc/utils.cpp:11-120).  start_width is 64/block in the reference (matmul.py:283).
+ * d_lut receives rows (head, block-row, block-col, blockid), all pack levels back to back in the order the
+ * reference returns them; level k has pack packs[k] and rows[k] rows (host arrays of >= 8 entries).
+ * d_valid (one byte per row) is 0 for the rows the reference emits for positions that are empty or were
+ * already taken (it does so for some dense layouts at pack 4); the sdd launcher skips them.
+ * cap_rows: capacity of d_lut / d_valid in rows; BSP_ERR_CAPACITY if exceeded (*total_rows = rows needed). */
+int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_width, int32_t *d_lut,
+                      uint8_t *d_valid, int64_t cap_rows, void *d_ws, int64_t ws_bytes, int *n_levels,
+                      int *packs, int64_t *rows, int64_t *total_rows, int *all_valid, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Matmul launchers.  Strides are in elements; the innermost stride of every operand is 1 and rows start on
+ * 16-byte boundaries.  trans_x means the stored matrix is read transposed, as in the reference.
+ * ------------------------------------------------------------------------------------------------- */
+
+/* sparse = dense x dense: replaces _sparse_matmul._sdd_matmul + the SDD branch of the kernel
+ * (matmul.py:299-364, 30-54).  One call per pack level of the sdd table.  For every valid table row
+ * (h, i, j, p):  C[z, p] = op(A)[z, h, i*block:(i+1)*block, 0:K] . op(B)[z, h, 0:K, j*block:(j+1)*block].
+ * lda / ldb: row stride of the stored 2-D matrices.  n_groups = rows / (pack*pack). */
+int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
+                   int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
+                   int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
+                   const uint8_t *d_valid, int64_t n_groups, void *stream);
+
+/* dense = sparse x dense: replaces _sparse_matmul._dsd_matmul + the DSD branch (matmul.py:507-552, 56-82).
+ * C[z, h] = op(A_sparse)[h] . op(B)[z, h], written transposed when trans_c.  N = free dimension of op(B).
+ * a_stride_z = 0 shares one sparse operand over the batch.  d_lut / d_plan / width from bsp_dxx_lut_build
+ * with trans = !trans_a. */
+int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                   int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
+                   int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                   const int32_t *d_plan, int width, void *stream);
+
+/* dense = dense x sparse: replaces _sparse_matmul._dds_matmul + the DDS branch (matmul.py:460-505, 83-99).
+ * C[z, h] = op(A)[z, h] . op(B_sparse)[h], written transposed when trans_c.  M = free dimension of op(A).
+ * Tables from bsp_dxx_lut_build with trans = trans_b. */
+int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                   int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
+                   int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                   const int32_t *d_plan, int width, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Softmax launchers: replace softmax_fwd / softmax_bwd and their dispatch (softmax.py:7-138, 144-194,
+ * 253-326).  x is [Z, nnz, block, block], updated in place.  Optional operands are NULL when absent.
+ *   rpe  : element (z, h, r, c) at rpe[z*rpe_stride_z + h*rpe_stride_h + r*rpe_stride_r + c]
+ *   kpm  : key padding mask, element (z, c) at kpm[z*kpm_stride_z + c]
+ *   attn : attention mask, element (r, c) at attn[r*attn_stride_r + c]
+ * *_mul != 0 selects the reference's 'mul' mode (mask value 0 -> -inf, anything else -> 0).
+ * y = softmax(x*scale + rpe + kpm + attn) over each row's nonzero blocks, computed in fp32. */
+int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int maxlut, const void *rpe,
+                    int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm,
+                    int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r, int attn_mul,
+                    int Z, int H, int R, int block, int64_t x_stride_z, void *stream);
+
+/* dx = y * (dy - sum(y*dy)) * scale per row, written over dy (softmax.py:183-193). */
+int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
+                    int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* BSP_H */

@@ -1,0 +1,68 @@
+"""GPU: the device-built look-up tables are bit-identical to the oracle's (and so to the reference's)."""
+import numpy as np
+import pytest
+import torch
+
+import torch_blocksparse as tb
+from torch_blocksparse.matmul import _sparse_matmul
+from torch_blocksparse.softmax import _sparse_softmax
+from oracle import lut_oracle as O
+from helpers import random_layout
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def check_all_tables(lay, blocks=((16, 16), (16, 8), (32, 16), (64, 16), (128, 8))):
+    lay = torch.as_tensor(lay, dtype=torch.int64)
+    layn = lay.numpy()
+    lut, maxlut = _sparse_softmax.make_lut(lay, 16, DEV)
+    elut, emax = O.make_softmax_lut(layn)
+    assert lut.cpu().tolist() == elut.tolist() and maxlut == emax
+    for block, step in blocks:
+        for trans in (False, True):
+            lut, num_locks, width, _ = _sparse_matmul.make_dxx_lut(lay, block, step, trans, DEV)
+            elut, enl, ewidth = O.make_dxx_lut(layn, block, step, trans)
+            assert lut.cpu().tolist() == elut.tolist(), (block, step, trans)
+            assert (num_locks, width) == (enl, ewidth)
+            # the per-block positions are what the increments are differences of
+            nz = lay.nonzero() if trans else lay.transpose(1, 2).nonzero()
+            assert lut.plan[:len(nz), 0].cpu().tolist() == (nz[:, 2] * block).tolist()
+    for block in (16, 32, 64, 128):
+        luts, _, widths, packs = _sparse_matmul.make_sdd_lut(lay, block, torch.float16, DEV)
+        exp = O.sdd_segment(layn, max(1, 64 // block))
+        assert packs == [p for p, _ in exp]
+        seen = set()
+        for t, w, (p, e) in zip(luts, widths, exp):
+            assert t.cpu().tolist() == e.reshape(-1).tolist(), (block, p)
+            assert w == e.shape[0] // (p * p)
+            valid = [1] * e.shape[0] if t.valid is None else t.valid.cpu().tolist()
+            for (h, i, j, b), v in zip(e.tolist(), valid):      # a row is valid iff it is the first for a real block
+                assert bool(v) == (layn[h, i, j] != 0 and (h, i, j) not in seen)
+                seen.add((h, i, j))
+
+
+def test_golden_layouts(golden):
+    for name, lay in golden['layouts'].items():
+        check_all_tables(lay)
+
+
+@pytest.mark.parametrize('seed', range(6))
+def test_random_layouts(seed):
+    g = torch.Generator().manual_seed(seed)
+    shape = tuple(int(torch.randint(lo, hi, (1,), generator=g)) for lo, hi in ((1, 5), (1, 40), (1, 80)))
+    check_all_tables(random_layout(shape, [0.05, 0.3, 0.5, 0.8, 0.97, 0.15][seed], seed), blocks=((16, 16), (32, 8)))
+
+
+def test_benchmark_config_layouts():
+    check_all_tables(tb.sparse_transformer_layout(16, 64, 4, 16, True), blocks=((64, 16),))          # attention, seq 4096
+    check_all_tables(tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True), blocks=((64, 16),))   # long context
+    check_all_tables(random_layout((1, 32, 32), 0.1, 5), blocks=((128, 16),))                        # sparse linear layer
+    check_all_tables(tb.fixed_layout(4, 64, 'fixed', 4, 'bidirectional', 4, 1), blocks=((16, 16),))
+
+
+def test_empty_head_raises():
+    lay = torch.zeros(2, 4, 4, dtype=torch.int64)
+    lay[0, 1, 2] = 1
+    with pytest.raises(RuntimeError):
+        _sparse_matmul.make_dxx_lut(lay, 16, 16, True, DEV)

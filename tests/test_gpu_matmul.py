@@ -1,0 +1,152 @@
+"""GPU: block-sparse matmul sdd / dsd / dds, forward and backward, against the fp32 dense-masked oracle."""
+import pytest
+import torch
+
+import torch_blocksparse as tb
+from oracle import dense_oracle as D
+from helpers import assert_close, random_layout
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def operand_shapes(mode, trans_a, trans_b, M, N, K):
+    a = (K, M) if trans_a else (M, K)
+    b = (N, K) if trans_b else (K, N)
+    sp = {'sdd': (M, N), 'dsd': a, 'dds': b}[mode]
+    return a, b, sp
+
+
+def run_case(mode, trans_a, trans_b, block, dtype, Z=3, H=2, M=256, N=512, K=384, density=0.5, seed=1, layout=None,
+             dist='rand', scale=1.0, backward=True):
+    """Same protocol as the reference's run_test_mm (tests/test_matmul.py:44-76): y, dx, dw."""
+    torch.manual_seed(seed)
+    ashape, bshape, sp = operand_shapes(mode, trans_a, trans_b, M, N, K)
+    lay = layout if layout is not None else random_layout((H, sp[0] // block, sp[1] // block), density, seed)
+    gen = torch.rand if dist == 'rand' else torch.randn
+    a = (gen((Z, H) + ashape) * scale).to(dtype)
+    b = (gen((Z, H) + bshape) * scale).to(dtype)
+    dc = gen((Z, H, M, N)).to(dtype)
+    if mode == 'dsd':
+        a = D.dense_to_sparse(a, lay, block)
+    if mode == 'dds':
+        b = D.dense_to_sparse(b, lay, block)
+    if mode == 'sdd':
+        dc = D.dense_to_sparse(dc, lay, block)
+    rc, rda, rdb = D.matmul(a, b, mode, trans_a, trans_b, lay, block, dc=dc)
+    op = tb.MatMul(lay, block, mode, trans_a=trans_a, trans_b=trans_b)
+    ag = a.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True)
+    c = op(ag, bg)
+    tag = '%s ta=%d tb=%d block=%d %s' % (mode, trans_a, trans_b, block, dtype)
+    assert_close(c, rc, dtype, tag + ' c')
+    if not backward:
+        return
+    c.backward(dc.to(DEV))
+    assert_close(ag.grad, rda, dtype, tag + ' da')
+    assert_close(bg.grad, rdb, dtype, tag + ' db')
+
+
+# the reference's 21 cases (tests/test_matmul.py:87-103): fp16, Z=3 H=2 M=256 N=512 K=384, half of the blocks kept
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('trans_a', [False, True])
+@pytest.mark.parametrize('trans_b', [False, True])
+def test_reference_trans_cases(mode, trans_a, trans_b):
+    run_case(mode, trans_a, trans_b, 32, torch.float16)
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+def test_reference_block_cases(mode, block):
+    run_case(mode, False, False, block, torch.float16)
+
+
+@pytest.mark.parametrize('mode', ['sdd', 'dsd', 'dds'])
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+@pytest.mark.parametrize('dtype', [torch.float32, torch.bfloat16])
+def test_other_dtypes(mode, block, dtype):
+    run_case(mode, False, True, block, dtype, Z=2, seed=block)
+    run_case(mode, True, False, block, dtype, Z=1, seed=block + 1)
+
+
+def test_readme_configuration():
+    # README of the reference: fp32, Z=4 H=2 M=256 N=512 K=384, block 16, sdd with trans_a, layout randint(0, 2)
+    torch.manual_seed(0)
+    lay = torch.randint(0, 2, (2, 16, 32))
+    run_case('sdd', True, False, 16, torch.float32, Z=4, layout=lay)
+
+
+def test_normal_inputs_with_cancellation():
+    run_case('dsd', False, False, 32, torch.float16, dist='randn', scale=0.05, seed=7)
+    run_case('dds', False, True, 64, torch.float16, dist='randn', scale=0.05, seed=8)
+    run_case('sdd', False, True, 64, torch.float32, dist='randn', scale=1.0, seed=9)
+
+
+def test_degenerate_layouts():
+    # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
+    lay = torch.zeros(2, 4, 6, dtype=torch.int64)
+    lay[0, 1, 2] = 1
+    lay[0, 1, 5] = 1
+    lay[1, 3, 0] = 1
+    run_case('dsd', False, False, 32, torch.float16, M=128, K=192, N=64, layout=lay)
+    run_case('dsd', True, False, 32, torch.float16, M=192, K=128, N=64, layout=lay)
+    run_case('dds', False, False, 32, torch.float16, M=64, K=128, N=192, layout=lay)
+    run_case('sdd', False, False, 32, torch.float16, M=128, N=192, K=64, layout=lay)
+    one = torch.ones(1, 1, 1, dtype=torch.int64)
+    run_case('sdd', False, True, 64, torch.float16, Z=1, H=1, M=64, N=64, K=16, layout=one)
+
+
+def test_dense_layout_with_pack4_rows_outside_the_layout():
+    # at 90% density the reference's packing emits rows for absent / repeated blocks; results must still be right
+    lay = random_layout((1, 24, 24), 0.9, 1234)
+    run_case('sdd', False, False, 16, torch.float16, Z=1, H=1, M=384, N=384, K=64, layout=lay)
+
+
+def test_free_dimension_not_a_multiple_of_the_tile():
+    # multiples of 16 that do not fill a 64-wide tile: forward and backward
+    run_case('dsd', False, False, 32, torch.float16, Z=1, H=2, M=128, K=128, N=80)
+    run_case('dds', False, True, 32, torch.float32, Z=1, H=2, M=48, K=128, N=128)
+    # any size works forward; the backward's sdd keeps the reference's rule (reduction % 16, matmul.py:318-319)
+    run_case('dsd', False, False, 32, torch.float16, Z=1, H=2, M=128, K=128, N=72, backward=False)
+    run_case('dsd', False, False, 32, torch.float32, Z=1, H=2, M=128, K=128, N=20, backward=False)
+    run_case('dds', False, False, 32, torch.float16, Z=1, H=2, M=40, K=128, N=128, backward=False)
+    run_case('dsd', False, True, 16, torch.float16, Z=1, H=1, M=64, K=64, N=10, backward=False)
+    run_case('dsd', False, True, 16, torch.bfloat16, Z=1, H=1, M=64, K=64, N=3, backward=False)
+
+
+def test_sdd_reduction_multiple_of_16():
+    lay = torch.ones(1, 2, 2, dtype=torch.int64)
+    a = torch.zeros(1, 1, 32, 24, dtype=torch.float16, device=DEV)
+    b = torch.zeros(1, 1, 24, 32, dtype=torch.float16, device=DEV)
+    with pytest.raises(ValueError):
+        tb.MatMul(lay, 16, 'sdd')(a, b)
+
+
+def test_dsd_dds_round_trip_config_reduced():
+    # config 2 (fp16, block 32, 2048^3, quarter of the blocks kept), all four transpositions, at Z=1 H=2
+    lay = random_layout((2, 64, 64), 0.25, 2, at_least_one_per_row=True)
+    for ta in (False, True):
+        for tb_ in (False, True):
+            run_case('dsd', ta, tb_, 32, torch.float16, Z=1, H=2, M=2048, N=256, K=2048, layout=lay, dist='randn', scale=2048 ** -0.25)
+            run_case('dds', ta, tb_, 32, torch.float16, Z=1, H=2, M=256, N=2048, K=2048, layout=lay, dist='randn', scale=2048 ** -0.25)
+
+
+def test_sparse_linear_layer_config_reduced():
+    # config 5: dds with trans_b, block 128, tenth of the blocks kept, weight 4096x4096, 1024 tokens; backward dsd + sdd
+    torch.manual_seed(5)
+    lay = random_layout((1, 32, 32), 0.1, 5)
+    run_case('dds', False, True, 128, torch.float16, Z=1, H=1, M=1024, N=4096, K=4096, layout=lay, dist='randn', scale=0.14)
+
+
+def test_linear_module():
+    torch.manual_seed(3)
+    lay = random_layout((1, 4, 6), 0.5, 3)
+    lin = tb.Linear(256, 384, 64, lay).to(DEV).half()
+    x = torch.randn(5, 7, 256, device=DEV, dtype=torch.float16, requires_grad=True)
+    y = lin(x)
+    wd = D.sparse_to_dense(lin.weight.detach().cpu().float()[None], lay, 64)[0, 0]
+    ref = x.detach().cpu().float() @ wd
+    assert_close(y, ref, torch.float16, 'linear y')
+    y.sum().backward()
+    assert lin.weight.grad.shape == lin.weight.shape and x.grad.shape == x.shape
+    assert_close(x.grad, torch.ones(5, 7, 384) @ wd.t(), torch.float16, 'linear dx')

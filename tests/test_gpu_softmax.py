@@ -1,0 +1,110 @@
+"""GPU: block-sparse softmax forward/backward against the fp32 dense-masked oracle (through the C ABI)."""
+import pytest
+import torch
+
+import torch_blocksparse as tb
+from oracle import dense_oracle as D
+from helpers import assert_close, random_layout
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+def run_case(Z, H, R, C, block, dtype, density, seed, scale=0.4, rpe=False, kpm=None, attn=None, layout=None):
+    torch.manual_seed(seed)
+    lay = layout if layout is not None else random_layout((H, R, C), density, seed, at_least_one_per_row=True)
+    nnz = int(lay.sum())
+    M, N = R * block, C * block
+    x = torch.rand((Z, nnz, block, block), dtype=torch.float32).to(dtype)
+    dy = torch.rand((Z, nnz, block, block), dtype=torch.float32).to(dtype)
+    kw = {}
+    if rpe:
+        kw['rpe'] = (0.5 * torch.randn(Z, H, M, N)).to(dtype)
+    if kpm == 'add':            # the reference's test: 0 / -inf, at least one key kept per row is not guaranteed there
+        m = torch.zeros(Z, N)
+        m[torch.rand(Z, N) < 0.3] = float('-inf')
+        m[:, ::block] = 0       # keep one key per block so that no row is fully masked
+        kw['key_padding_mask'] = m.to(dtype)
+        kw['key_padding_mask_mode'] = 'add'
+    elif kpm == 'mul':
+        m = (torch.rand(Z, N) > 0.3).float()
+        m[:, ::block] = 1
+        kw['key_padding_mask'] = m.to(dtype)
+        kw['key_padding_mask_mode'] = 'mul'
+    if attn == 'mul':
+        a = (torch.rand(M, N) > 0.4).float()
+        a[:, 1::block] = 1
+        kw['attn_mask'] = a.to(dtype)
+        kw['attn_mask_mode'] = 'mul'
+    elif attn == 'add':
+        kw['attn_mask'] = torch.randn(M, N).to(dtype)
+        kw['attn_mask_mode'] = 'add'
+    ry, rdx = D.softmax(x, lay, block, scale=scale, dy=dy, **kw)
+    op = tb.Softmax(lay, block)
+    xg = x.to(DEV).requires_grad_(True)
+    gkw = {k: (v.to(DEV) if torch.is_tensor(v) else v) for k, v in kw.items()}
+    y = op(xg * 1.0, scale=scale, **gkw)          # the op works in place: feed it a temporary
+    y.backward(dy.to(DEV))
+    assert_close(y, ry, dtype, 'softmax y')
+    assert_close(xg.grad, rdx, dtype, 'softmax dx')
+
+
+# the reference's own cases (tests/test_softmax.py:80-90): block 16, widths 256 / 576, fp16 / fp32
+@pytest.mark.parametrize('width', [256, 576])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.float32])
+def test_reference_cases(width, dtype):
+    run_case(2, 4, width // 16, width // 16, 16, dtype, 0.6, width, scale=0.4, kpm='add', attn='mul')
+
+
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_blocks_and_dtypes(block, dtype):
+    run_case(2, 2, 6, 5, block, dtype, 0.5, block, scale=0.7)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.float32])
+def test_rpe_and_mask_modes(dtype):
+    run_case(2, 3, 4, 6, 32, dtype, 0.6, 11, scale=0.3, rpe=True, kpm='mul', attn='add')
+    run_case(2, 3, 4, 6, 16, dtype, 0.6, 12, scale=1.0, rpe=True)
+    run_case(1, 2, 3, 3, 64, dtype, 0.7, 13, scale=0.125, kpm='add')
+
+
+@pytest.mark.parametrize('block,cols', [(16, 70), (64, 20), (128, 9), (32, 40)])
+def test_long_rows_streaming_variant(block, cols):
+    # more blocks per row than the register variant holds
+    run_case(1, 1, 2, cols, block, torch.float16, 0.95, cols, scale=0.5, kpm='add')
+    run_case(1, 1, 2, cols, block, torch.float32, 0.95, cols + 1, scale=0.5)
+
+
+def test_rows_without_blocks_and_single_block():
+    lay = torch.zeros(2, 4, 4, dtype=torch.int64)
+    lay[0, 0, 1] = 1
+    lay[0, 2, :] = 1
+    lay[1, 3, 3] = 1
+    run_case(2, 2, 4, 4, 32, torch.float16, 0, 21, layout=lay)
+
+
+def test_attention_config_shape_small_batch():
+    # the benchmark configuration (block 64, seq 4096, fixed layout, additive key padding mask) at batch 1, 2 heads
+    lay = tb.sparse_transformer_layout(2, 64, 4, 16, True)
+    run_case(1, 2, 64, 64, 64, torch.float16, 0, 31, scale=0.125, kpm='add', layout=lay)
+
+
+def test_fully_masked_row_gives_nan_like_the_dense_oracle():
+    lay = torch.ones(1, 2, 2, dtype=torch.int64)
+    x = torch.rand(1, 4, 16, 16, dtype=torch.float16)
+    m = torch.zeros(1, 32, dtype=torch.float16)
+    m[:] = float('-inf')
+    ry = D.softmax(x, lay, 16, key_padding_mask=m)
+    y = tb.Softmax(lay, 16)(x.to(DEV), key_padding_mask=m.to(DEV))
+    assert torch.isnan(ry).all() and torch.isnan(y).all()
+
+
+def test_in_place_and_row_too_long():
+    lay = torch.ones(1, 1, 2, dtype=torch.int64)
+    x = torch.rand(1, 2, 16, 16, dtype=torch.float16, device=DEV)
+    y = tb.Softmax(lay, 16)(x)
+    assert y.data_ptr() == x.data_ptr()
+    big = torch.ones(1, 1, 512, dtype=torch.int64)
+    with pytest.raises(NotImplementedError):
+        tb.Softmax(big, 64)(torch.zeros(1, 512, 64, 64, dtype=torch.float16, device=DEV))

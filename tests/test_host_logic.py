@@ -1,0 +1,106 @@
+"""CPU tests of the host side: the C-ABI library loads and exports every declared symbol, the layout
+generators match the oracle, the dense oracle's converters round-trip, and argument errors are the reference's."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import torch_blocksparse as tb
+from torch_blocksparse import _lib
+from oracle import dense_oracle as D
+from oracle import lut_oracle as O
+from helpers import random_layout
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, 'include', 'bsp.h')).read()
+    declared = set(re.findall(r'\b(bsp_[a-z0-9_]+)\s*\(', header))
+    assert declared == set(_lib.SIGNATURES), declared ^ set(_lib.SIGNATURES)
+    lib = _lib.load()
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.bsp_version() >= 1
+    assert b'multiple of 16' in lib.bsp_strerror(-7)
+
+
+def test_no_cpu_fallback():
+    lay = torch.ones(1, 2, 2, dtype=torch.int64)
+    with pytest.raises(_lib.BlocksparseLibraryError):
+        tb.MatMul(lay, 16, 'sdd')(torch.zeros(1, 1, 32, 16), torch.zeros(1, 1, 16, 32))
+    with pytest.raises(_lib.BlocksparseLibraryError):
+        tb.Softmax(lay, 16)(torch.zeros(1, 4, 16, 16))
+
+
+def test_constructor_errors():
+    lay = torch.ones(1, 2, 2, dtype=torch.int64)
+    with pytest.raises(NotImplementedError):
+        tb.MatMul(lay, 16, 'ssd')
+    with pytest.raises(NotImplementedError):
+        tb.SparsityConfig(mode='bigbird')
+    with pytest.raises(NotImplementedError):
+        tb.SparsityConfig(attention='causal')
+    with pytest.raises(NotImplementedError):
+        tb.MultiheadAttention(32, 2, lay, 16, dropout=0.1)
+    with pytest.raises(ValueError):
+        tb.Softmax(lay, 16)(torch.zeros(1, 4, 16, 16, dtype=torch.float16), attn_mask=torch.zeros(32, 32))
+    with pytest.raises(ValueError):
+        tb.fixed_layout(2, 16, 'fixed', 4, 'unidirectional', 1, 3)
+    with pytest.raises(ValueError):
+        tb.fixed_layout(2, 16, 'fixed', 4, 'unidirectional', 8, 1)
+
+
+def test_layout_generators_match_oracle(golden):
+    for c in golden['make_layout_cpp']:
+        assert tb.make_layout(*c['args']).tolist() == c['layout']
+    for args in [(2, 8, 'fixed', 4, 'unidirectional', 1, 1), (4, 16, 'fixed', 4, 'bidirectional', 2, 2),
+                 (4, 16, 'fixed', 8, 'unidirectional', 4, 2), (3, 32, 'fixed', 8, 'bidirectional', 8, 1),
+                 (2, 8, 'dense', 4, 'unidirectional', 1, 1)]:
+        assert (tb.fixed_layout(*args).numpy() == O.make_layout_py(*args)).all()
+        assert (tb.DeepSpeedSparseSelfAttention._make_layout(*args).numpy() == O.make_layout_py(*args)).all()
+
+
+def test_config3_layout_statistics():
+    lay = tb.sparse_transformer_layout(16, 64, 4, 16, True)
+    assert lay.shape == (16, 64, 64) and int(lay[0].sum()) == 256
+    assert int(lay[0].sum(1).max()) == 7 and int(lay[0].sum(0).max()) == 49
+    assert (lay.triu(1) == 0).all()
+
+
+def test_bigbird_layout():
+    a = tb.bigbird_layout(2, 32, 3, 2, 3, seed=5, causal=True)
+    b = tb.bigbird_layout(2, 32, 3, 2, 3, seed=5, causal=True)
+    assert (a == b).all() and (a.triu(1) == 0).all() and (a[:, :, 0] == 1).all()
+    assert int(a.sum(-1).max()) <= 8
+    c = tb.bigbird_layout(1, 32, 3, 2, 3, seed=5, causal=False)
+    assert (c[0, :2] == 1).all() and (c[0, :, :2] == 1).all()
+
+
+def test_dense_oracle_converters_round_trip():
+    block = 4
+    lay = random_layout((2, 3, 5), 0.5, 3)
+    w = torch.randn(2, 2, 3 * block, 5 * block)
+    sp = D.dense_to_sparse(w, lay, block)
+    # brute force, the reference's loops (tests/utils.py:5-13)
+    nz = lay.nonzero()
+    for z in range(2):
+        for p, (h, i, j) in enumerate(nz.tolist()):
+            assert torch.equal(sp[z, p], w[z, h, i * block:(i + 1) * block, j * block:(j + 1) * block])
+    dn = D.sparse_to_dense(sp, lay, block)
+    assert torch.equal(dn, D.mask_dense(w, lay, block))
+    assert torch.equal(D.dense_to_sparse(dn, lay, block), sp)
+
+
+def test_dense_oracle_softmax_properties():
+    block = 4
+    lay = random_layout((2, 4, 4), 0.6, 9, at_least_one_per_row=True)
+    x = torch.randn(2, int(lay.sum()), block, block)
+    dy = torch.randn_like(x)
+    y, dx = D.softmax(x, lay, block, scale=0.7, dy=dy)
+    rows = D.sparse_to_dense(y, lay, block).sum(-1)
+    assert torch.allclose(rows, torch.ones_like(rows), atol=1e-6)
+    # the gradient of a softmax row sums to zero
+    assert D.sparse_to_dense(dx, lay, block).sum(-1).abs().max() < 1e-5

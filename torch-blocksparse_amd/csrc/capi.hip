@@ -1,0 +1,114 @@
+// C-ABI entry points of the matmul launchers: argument validation and dispatch.  (The table builders and
+// the softmax entry points live next to their kernels in lut.hip / softmax.hip.)
+#include "matmul_generic.h"
+
+using namespace bsp;
+
+namespace {
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+bool block_ok(int block) { return block == 16 || block == 32 || block == 64 || block == 128; }
+int elems16(int dtype) { return dtype == BSP_F32 ? 4 : 8; }   // elements per 16 bytes
+}  // namespace
+
+extern "C" int bsp_version(void) { return 1; }
+
+extern "C" const char *bsp_strerror(int status) {
+  switch (status) {
+    case BSP_OK: return "ok";
+    case BSP_ERR_ARG: return "invalid argument (null pointer, bad size or operand not 16-byte aligned)";
+    case BSP_ERR_UNSUPPORTED: return "unsupported block size, dtype or problem size";
+    case BSP_ERR_CAPACITY: return "caller-provided table or workspace too small";
+    case BSP_ERR_EMPTY_HEAD: return "a head of the layout has no nonzero block";
+    case BSP_ERR_HIP: return "HIP runtime error";
+    case BSP_ERR_ROW_TOO_LONG: return "Reductions larger than 32768 elements are not yet implemented";
+    case BSP_ERR_K_MULTIPLE: return "Reduction size for SDD must be a multiple of 16";
+    default: return "unknown status";
+  }
+}
+
+extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
+                              int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
+                              int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
+                              const uint8_t *d_valid, int64_t n_groups, void *stream) {
+  if (!a || !b || !c || !d_lut || Z <= 0 || K <= 0 || n_groups < 0) return BSP_ERR_ARG;
+  if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
+  if (K % 16) return BSP_ERR_K_MULTIPLE;   // reference matmul.py:318-319
+  const int u = elems16(dtype);
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
+  if (a_stride_z % u || a_stride_h % u || lda % u || b_stride_z % u || b_stride_h % u || ldb % u || c_stride_z % u) return BSP_ERR_ARG;
+  SddArgs g;
+  g.a = a; g.b = b; g.c = c; g.Z = Z; g.K = K;
+  g.a_sz = a_stride_z; g.a_sh = a_stride_h; g.lda = lda;
+  g.b_sz = b_stride_z; g.b_sh = b_stride_h; g.ldb = ldb; g.c_sz = c_stride_z;
+  g.lut = d_lut; g.valid = d_valid; g.n_groups = n_groups;
+  // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
+  const bool a_kc = !trans_a, b_kc = trans_b != 0;
+  hipStream_t st = as_stream(stream);
+  int rc;
+  switch (dtype) {
+    case BSP_F16: rc = sdd_generic_f16(g, block, pack, a_kc, b_kc, st); break;
+    case BSP_BF16: rc = sdd_generic_bf16(g, block, pack, a_kc, b_kc, st); break;
+    case BSP_F32: rc = sdd_generic_f32(g, block, pack, a_kc, b_kc, st); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
+static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, void *stream) {
+  hipStream_t st = as_stream(stream);
+  int rc;
+  switch (dtype) {
+    case BSP_F16: rc = xsd_generic_f16(g, block, sp_trans, dn_kc, out_nc, st); break;
+    case BSP_BF16: rc = xsd_generic_bf16(g, block, sp_trans, dn_kc, out_nc, st); break;
+    case BSP_F32: rc = xsd_generic_f32(g, block, sp_trans, dn_kc, out_nc, st); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
+extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                              int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
+                              int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                              const int32_t *d_plan, int width, void *stream) {
+  if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || N <= 0 || width < 0) return BSP_ERR_ARG;
+  if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
+  const int u = elems16(dtype);
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
+  if (N % u || a_stride_z % u || b_stride_z % u || b_stride_h % u || ldb % u || c_stride_z % u || c_stride_h % u || ldc % u) return BSP_ERR_ARG;
+  XsdArgs g;
+  g.sp = a; g.dn = b; g.out = c; g.Z = Z; g.NF = N;
+  g.sp_sz = a_stride_z; g.dn_sz = b_stride_z; g.dn_sh = b_stride_h; g.ldd = ldb;
+  g.out_sz = c_stride_z; g.out_sh = c_stride_h; g.ldo = ldc;
+  g.lut = d_lut; g.plan = d_plan; g.width = width;
+  g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));   // step of the table: 8 for fp32, 16 otherwise (matmul.py:617)
+  g.n_tiles = (N + 63) / 64;
+  // rows of the kernel = rows of op(A); op(A)(m,k) is stored [k][m] when trans_a.  Dense (n,k) = op(B)[k][n]:
+  // reduction contiguous when B is read transposed.  C[m][n] has n contiguous unless written transposed.
+  return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, stream);
+}
+
+extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                              int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
+                              int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                              const int32_t *d_plan, int width, void *stream) {
+  if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || M <= 0 || width < 0) return BSP_ERR_ARG;
+  if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
+  const int u = elems16(dtype);
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
+  if (M % u || a_stride_z % u || a_stride_h % u || lda % u || b_stride_z % u || c_stride_z % u || c_stride_h % u || ldc % u) return BSP_ERR_ARG;
+  XsdArgs g;
+  g.sp = b; g.dn = a; g.out = c; g.Z = Z; g.NF = M;
+  g.sp_sz = b_stride_z; g.dn_sz = a_stride_z; g.dn_sh = a_stride_h; g.ldd = lda;
+  g.out_sz = c_stride_z; g.out_sh = c_stride_h; g.ldo = ldc;
+  g.lut = d_lut; g.plan = d_plan; g.width = width;
+  g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));
+  g.n_tiles = (M + 63) / 64;
+  // dds is dsd on the transposed problem: kernel rows = columns of op(B) (stored [k][col] unless trans_b), dense
+  // rows = rows of op(A) (reduction contiguous unless trans_a), and C[row][col] has the kernel's m index contiguous
+  // unless written transposed.
+  return xsd_dispatch(dtype, g, block, !trans_b, !trans_a, trans_c != 0, stream);
+}

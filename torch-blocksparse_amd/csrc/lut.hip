@@ -1,0 +1,507 @@
+// Device builders for the three look-up tables (softmax, dsd/dds, sdd).
+//
+// The reference builds these tables on the host with Python loops and a small OpenMP C++ helper
+// (matmul.py:221-297,372-458; softmax.py:201-221; csrc/utils.cpp:11-120).  Here the layout is copied
+// to the GPU once and the tables are produced there: counts -> prefix sums -> one thread per block-row /
+// block-column writes its part.  Only the greedy super-block packing of the sdd table is sequential by
+// nature (every decision depends on the blocks retained before it); it runs one wavefront per head.
+// All tables are bit-identical to the reference's.
+#include "bsp_common.h"
+
+namespace bsp {
+namespace {
+
+// ---------------------------------------------------------------------------------------------------------
+// workspace carving (int32 units)
+// ---------------------------------------------------------------------------------------------------------
+struct Ws {
+  int64_t rowcnt, rowstart, colcnt, colstart, linepacks, segstart, headmax, rank, lay, tmp, top, counts, offsets, scal, end;
+  __host__ Ws(int H, int R, int C) {
+    int64_t hr = (int64_t)H * R, hc = (int64_t)H * C, cells = (int64_t)H * R * C, hl = hr > hc ? hr : hc;
+    int64_t o = 0;
+    auto take = [&](int64_t n) { int64_t at = o; o += (n + 3) & ~(int64_t)3; return at; };
+    rowcnt = take(hr); rowstart = take(hr + 1); colcnt = take(hc); colstart = take(hc + 1);
+    linepacks = take(hl); segstart = take(hl + 1); headmax = take(H);
+    rank = take(cells); lay = take(cells); tmp = take(cells); top = take((int64_t)H * 4 * C);
+    counts = take(2 * 8 * (int64_t)H);   // int64 [8 levels][H]
+    offsets = take(2 * 8 * (int64_t)H);  // int64 [8 levels][H]
+    scal = take(16);
+    end = o;
+  }
+};
+
+enum { S_MAXLUT = 0, S_TOTAL = 1, S_WIDTH = 2, S_NNZ = 3, S_ERR = 4, S_INVALID = 5 };
+
+// ---------------------------------------------------------------------------------------------------------
+// small generic kernels
+// ---------------------------------------------------------------------------------------------------------
+__global__ void k_fill(int32_t *p, int64_t n, int32_t v) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// nonzeros per block-row and per block-column of every head
+__global__ void k_row_counts(const int32_t *lay, int H, int R, int C, int32_t *rowcnt) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * R) return;
+  const int32_t *p = lay + i * C;
+  int n = 0;
+  for (int c = 0; c < C; c++) n += p[c] != 0;
+  rowcnt[i] = n;
+}
+__global__ void k_col_counts(const int32_t *lay, int H, int R, int C, int32_t *colcnt) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * C) return;
+  int h = (int)(i / C), c = (int)(i % C);
+  const int32_t *p = lay + (int64_t)h * R * C + c;
+  int n = 0;
+  for (int r = 0; r < R; r++) n += p[(int64_t)r * C] != 0;
+  colcnt[i] = n;
+}
+
+// Exclusive prefix sum of n int32 by one workgroup of 1024 threads; out has n+1 entries (out[n] = total).
+// Optionally also reduces the maximum into *maxout.
+__global__ void __launch_bounds__(1024) k_exclusive_scan(const int32_t *in, int32_t *out, int64_t n, int32_t *maxout) {
+  __shared__ int32_t buf[1024];
+  __shared__ int32_t carry_s;
+  __shared__ int32_t max_s;
+  const int t = threadIdx.x;
+  if (t == 0) { carry_s = 0; max_s = 0; }
+  __syncthreads();
+  for (int64_t base = 0; base < n; base += 1024) {
+    int32_t v = (base + t < n) ? in[base + t] : 0;
+    buf[t] = v;
+    __syncthreads();
+    for (int d = 1; d < 1024; d <<= 1) {
+      int32_t add = (t >= d) ? buf[t - d] : 0;
+      __syncthreads();
+      buf[t] += add;
+      __syncthreads();
+    }
+    int32_t carry = carry_s;
+    if (base + t < n) out[base + t] = carry + buf[t] - v;
+    if (maxout) atomicMax(&max_s, v);
+    __syncthreads();
+    if (t == 1023) carry_s = carry + buf[1023];
+    __syncthreads();
+  }
+  if (t == 0) { out[n] = carry_s; if (maxout) *maxout = max_s; }
+}
+
+// rank[h,r,c] = position of block (h,r,c) among the nonzeros in (h,r,c) order; 0 where the layout is empty
+// (the reference's `idx` tensor starts as zeros, utils.cpp:99-112).
+__global__ void k_rank(const int32_t *lay, int H, int R, int C, const int32_t *rowstart, int32_t *rank) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * R) return;
+  int32_t t = rowstart[i];
+  for (int c = 0; c < C; c++) {
+    bool nz = lay[i * C + c] != 0;
+    rank[i * C + c] = nz ? t : 0;
+    t += nz;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// softmax table (reference softmax.py:201-221)
+// ---------------------------------------------------------------------------------------------------------
+__global__ void k_softmax_lut(const int32_t *lay, int H, int R, int C, const int32_t *rowcnt, const int32_t *rowstart,
+                              int32_t *lut) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  const int64_t nrows = (int64_t)H * R;
+  if (i >= nrows) return;
+  const int h = (int)(i / R), r = (int)(i % R);
+  int64_t t = rowstart[i];
+  lut[2 * i + 0] = rowcnt[i];                          // sizes            (:206-207)
+  lut[2 * i + 1] = (int32_t)(t * 4 + 2 * nrows);       // offsets*4 + 2*sizes.numel()   (:218)
+  for (int c = 0; c < C; c++)
+    if (lay[i * C + c] != 0) {                         // core = (idx, columns, rows, head)  (:212-216)
+      int32_t *e = lut + 2 * nrows + 4 * t;
+      e[0] = (int32_t)t; e[1] = c; e[2] = r; e[3] = h;
+      t++;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dsd/dds table (reference matmul.py:221-267 load_balance, :372-458 make_dxx_lut)
+// A "line" is a block-row (trans) or a block-column (not trans) of one head: one reduction.
+// ---------------------------------------------------------------------------------------------------------
+__global__ void k_head_max(const int32_t *sizes, int H, int L, int32_t *headmax, int32_t *scal) {
+  int h = blockIdx.x * blockDim.x + threadIdx.x;
+  if (h >= H) return;
+  int mx = 0;
+  for (int i = 0; i < L; i++) mx = max(mx, sizes[(int64_t)h * L + i]);
+  headmax[h] = mx;
+  if (mx == 0) scal[S_ERR] = BSP_ERR_EMPTY_HEAD;  // the reference raises on a head without blocks (:226-227)
+}
+
+// load_balance with seg_max = max_size (matmul.py:232).  Then div = size // seg_max is 0 or 1 and rem is 0
+// whenever div is 1, so the lock condition `d > 1 or (d == 1 and r >= seg_min)` (:253) never holds and
+// lockid / maxid stay 0 for every segment; the general segment formula is kept literally.
+struct LineSplit { int d, r, isempty, n; };
+__device__ __forceinline__ LineSplit split_line(int size, int seg_max) {
+  int seg_min = max((seg_max + 3) / 4, 4);                 // :233
+  LineSplit s;
+  s.d = size / seg_max; s.r = size % seg_max;              // :235-236
+  s.isempty = size < seg_min;                              // :248
+  s.n = s.d + (s.r >= seg_min) + s.isempty;                // :237 / :249
+  return s;
+}
+// length (in blocks) of the j-th segment of a line (:258-262)
+__device__ __forceinline__ int segment_len(const LineSplit &s, int size, int seg_max, int j) {
+  int seg_min = max((seg_max + 3) / 4, 4);
+  int len = j < s.d ? seg_max : 0;
+  if (s.r < seg_min && !s.isempty && j == s.d - 1) len += s.r;
+  if ((s.r >= seg_min || s.isempty) && j == s.d) len = s.r;
+  (void)size;
+  return len;
+}
+
+__global__ void k_line_packs(const int32_t *sizes, const int32_t *headmax, int H, int L, int32_t *linepacks) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * L) return;
+  int mx = headmax[i / L];
+  linepacks[i] = mx > 0 ? split_line(sizes[i], mx).n : 0;
+}
+
+__global__ void k_dxx_header(const int32_t *sizes, const int32_t *headmax, const int32_t *segstart, const int32_t *blkstart,
+                             int H, int L, int block, int step, int32_t *lut) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * L) return;
+  const int h = (int)(i / L), line = (int)(i % L);
+  const int mx = headmax[h];
+  if (mx <= 0) return;
+  const int64_t width = segstart[(int64_t)H * L];
+  const int64_t nnz = blkstart[(int64_t)H * L];
+  const int div = block / step;                                       // :413
+  const int size = sizes[i];
+  LineSplit s = split_line(size, mx);
+  int64_t off = blkstart[i];                                          // cumsum of segments + blocks of earlier heads (:266, :398)
+  for (int j = 0; j < s.n; j++) {
+    int len = segment_len(s, size, mx, j);
+    int64_t o = off < nnz - 1 ? off : nnz - 1;                        // :408
+    int32_t *e = lut + 6 * ((int64_t)segstart[i] + j);
+    e[0] = (int32_t)(o * 2 * div + 6 * width);                        // :445, :449
+    e[1] = (int32_t)((int64_t)len * step * div);                      // :401, :446
+    e[2] = line;                                                      // column (:251)
+    e[3] = h;                                                         // depth (:390)
+    e[4] = 0;                                                         // lockid
+    e[5] = 0;                                                         // maxid
+    off += len;
+  }
+}
+
+// plan[2t] = offset of block t in the dense operand's reduction dimension, plan[2t+1] = storage index (:403-432)
+__global__ void k_dxx_plan(const int32_t *lay, const int32_t *rank, const int32_t *blkstart, int H, int R, int C, int block,
+                           int trans, int32_t *plan) {
+  const int L = trans ? R : C;
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * L) return;
+  const int h = (int)(i / L), line = (int)(i % L);
+  int64_t t = blkstart[i];
+  if (trans) {
+    for (int c = 0; c < C; c++) {
+      int64_t p = ((int64_t)h * R + line) * C + c;
+      if (lay[p] != 0) { plan[2 * t] = c * block; plan[2 * t + 1] = (int32_t)t; t++; }   // nnz[:,2]*block ; arange
+    }
+  } else {
+    for (int r = 0; r < R; r++) {
+      int64_t p = ((int64_t)h * R + r) * C + line;
+      if (lay[p] != 0) { plan[2 * t] = r * block; plan[2 * t + 1] = rank[p]; t++; }     // transposed nonzero(); widx (:426-431)
+    }
+  }
+}
+
+__global__ void k_dxx_incs(const int32_t *plan, int64_t nnz, int block, int step, int trans, int64_t width, int32_t *lut) {
+  int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (t >= nnz) return;
+  const int div = block / step;
+  const int64_t bb = (int64_t)block * block;
+  const int64_t wstep = trans ? step : (int64_t)step * block;        // :436-441
+  int64_t dx = (int64_t)plan[2 * t] - (t ? (int64_t)plan[2 * t - 2] : 0);                 // :410-411
+  int64_t dw = (int64_t)plan[2 * t + 1] * bb - (t ? (int64_t)plan[2 * t - 1] * bb : 0);   // :433-434
+  int32_t *inc = lut + 6 * width + 2 * t * div;
+  for (int j = 0; j < div; j++) {
+    inc[2 * j + 0] = (int32_t)(j ? step : dx - (int64_t)(div - 1) * step);                // :414-416
+    inc[2 * j + 1] = (int32_t)(j ? wstep : dw - (int64_t)(div - 1) * wstep);
+  }
+  if (t == nnz - 1) { inc[2 * div] = 0; inc[2 * div + 1] = 0; }                           // :452
+}
+
+// first increment of every non-empty segment is the absolute position (:418, :442)
+__global__ void k_dxx_fix(const int32_t *sizes, const int32_t *headmax, const int32_t *segstart, const int32_t *blkstart,
+                          const int32_t *plan, int H, int L, int block, int step, int32_t *lut) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * L) return;
+  const int mx = headmax[i / L];
+  if (mx <= 0) return;
+  const int64_t width = segstart[(int64_t)H * L];
+  const int div = block / step;
+  const int size = sizes[i];
+  LineSplit s = split_line(size, mx);
+  int64_t off = blkstart[i];
+  for (int j = 0; j < s.n; j++) {
+    int len = segment_len(s, size, mx, j);
+    if (len > 0) {
+      int32_t *inc = lut + 6 * width + 2 * off * div;
+      inc[0] = plan[2 * off];
+      inc[1] = plan[2 * off + 1];
+    }
+    off += len;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// sdd table: greedy packing of nonzero blocks into w x w super-blocks, w = start_width, /2, ..., 1
+// (reference csrc/utils.cpp:11-120).  One wavefront per head; the 64 lanes scan 64 layout cells at a time
+// and cooperate on the "anything in between" test, every decision itself is taken in reference order.
+// The kernel runs twice: a counting pass (write = 0) that fixes where each (level, head) slice starts,
+// and a writing pass on a fresh copy of the layout.
+// ---------------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(64) k_sdd_segment(int32_t *lay, const int32_t *rank, int32_t *tmp, int32_t *top, int H, int R,
+                                                    int C, int start_width, int write, int64_t *counts,
+                                                    const int64_t *offsets, int32_t *out, uint8_t *valid, int64_t cap_rows,
+                                                    int32_t *scal) {
+  const int h = blockIdx.x, lane = threadIdx.x;
+  int32_t *L = lay + (int64_t)h * R * C;
+  const int32_t *K = rank + (int64_t)h * R * C;
+  int32_t *T = tmp + (int64_t)h * R * C;
+  int32_t *P = top + (int64_t)h * 4 * C;
+  int lev = 0;
+  for (int w = start_width; w > 0; w >>= 1, lev++) {
+    for (int64_t i = lane; i < (int64_t)R * C; i += 64) T[i] = 0;        // tmp = zeros_like(layout), utils.cpp:15
+    for (int i = lane; i < w * C; i += 64) P[i] = -1;                    // ii_top, :32
+    __syncthreads();
+    int left[4] = {-1, -1, -1, -1};                                      // ii_left, :31 (ring index k lives in left[k + 4 - w])
+    int64_t nrows = 0;
+    const int64_t base = write ? offsets[lev * H + h] : 0;
+    int32_t *Plast = P + (int64_t)(w - 1) * C;
+    for (int m = 0; m < R; m++) {
+      for (int n0 = 0; n0 < C; n0 += 64) {
+        int v = (n0 + lane < C) ? L[(int64_t)m * C + n0 + lane] : 0;
+        unsigned long long mask = __ballot(v != 0);
+        while (mask) {
+          const int n = n0 + __ffsll((long long)mask) - 1;
+          mask &= mask - 1;
+          const int n_left = left[3];                                                    // :39
+          const int m_top = Plast[n];                                                    // :40
+          const int tp = (m_top >= 0) ? T[(int64_t)m_top * C + n] : 0;                   // :41
+          const int lf = (n_left >= 0) ? T[(int64_t)m * C + n_left] : 0;                 // :42
+          const int tl = (m_top >= 0 && n_left >= 0) ? T[(int64_t)m_top * C + n_left] : 0; // :43
+          int width = min(lf, min(tp, tl)) + 1;                                          // :44
+          bool between = false;                                                          // :48-50, 64 columns per step
+          for (int nn = n_left + 1 + lane; nn < n; nn += 64) between |= Plast[nn] > m_top;
+          if (__ballot(between)) width = 1;
+          T[(int64_t)m * C + n] = width;                                                 // :51
+          left[0] = left[1]; left[1] = left[2]; left[2] = left[3]; left[3] = n;          // :54-56
+          for (int k = 0; k < w - 1; k++) P[(int64_t)k * C + n] = P[(int64_t)(k + 1) * C + n]; // :59-60
+          Plast[n] = m;                                                                  // :61
+          if (width != w) continue;                                                      // :64-65
+          for (int km = 0; km < w; km++)
+            for (int kn = 0; kn < w; kn++) {                                             // :68-82
+              const int mm = P[(int64_t)km * C + n];
+              const int nn = left[kn + 4 - w];
+              if (mm < 0 || nn < 0) continue;
+              const int64_t p = (int64_t)mm * C + nn;
+              const int was = L[p];
+              L[p] = 0;
+              T[p] = 0;
+              if (write) {
+                const int64_t row = base + nrows;
+                if (row < cap_rows && lane == 0) {
+                  out[row * 4 + 0] = h; out[row * 4 + 1] = mm; out[row * 4 + 2] = nn; out[row * 4 + 3] = K[p];
+                  valid[row] = was != 0;
+                }
+              }
+              if (was == 0) scal[S_INVALID] = 1;   // a row for a block that is empty or already taken
+              // a cell of this row still pending in `mask` may just have been retained: the reference reads the
+              // layout live (:36), so drop it
+              if (mm == m && nn > n && nn < n0 + 64) mask &= ~(1ull << (nn - n0));
+              nrows++;
+            }
+        }
+      }
+    }
+    if (!write && lane == 0) counts[lev * H + h] = nrows;
+    __syncthreads();
+  }
+}
+
+// offsets[lev][h] = rows emitted before slice (lev, h) in (level, head) order
+__global__ void k_sdd_offsets(const int64_t *counts, int64_t *offsets, int nlev, int H, int32_t *scal) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int64_t run = 0;
+  for (int i = 0; i < nlev * H; i++) { offsets[i] = run; run += counts[i]; }
+  (void)scal;
+}
+
+int prepare_counts(const int32_t *d_layout, int H, int R, int C, int32_t *ws, const Ws &o, hipStream_t st) {
+  const int T = 256;
+  hipLaunchKernelGGL(k_fill, dim3(1), dim3(64), 0, st, ws + o.scal, (int64_t)16, 0);
+  hipLaunchKernelGGL(k_row_counts, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowcnt);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.rowcnt, ws + o.rowstart, (int64_t)H * R, ws + o.scal + S_MAXLUT);
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
+int check_args(const void *d_layout, int H, int R, int C, void *d_ws, int64_t ws_bytes) {
+  if (!d_layout || !d_ws || H <= 0 || R <= 0 || C <= 0) return BSP_ERR_ARG;
+  if ((int64_t)H * R * C >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (ws_bytes < bsp_lut_workspace_bytes(H, R, C)) return BSP_ERR_CAPACITY;
+  return BSP_OK;
+}
+
+}  // namespace
+}  // namespace bsp
+
+using namespace bsp;
+
+extern "C" int64_t bsp_lut_workspace_bytes(int H, int R, int C) {
+  if (H <= 0 || R <= 0 || C <= 0) return 0;
+  return Ws(H, R, C).end * (int64_t)sizeof(int32_t);
+}
+
+extern "C" int bsp_layout_nnz(const int32_t *d_layout, int H, int R, int C, void *d_ws, int64_t ws_bytes, int64_t *nnz,
+                              void *stream) {
+  int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
+  if (rc != BSP_OK || !nnz) return rc != BSP_OK ? rc : BSP_ERR_ARG;
+  hipStream_t st = as_stream(stream);
+  Ws o(H, R, C);
+  int32_t *ws = (int32_t *)d_ws;
+  rc = prepare_counts(d_layout, H, R, C, ws, o, st);
+  if (rc != BSP_OK) return rc;
+  int32_t total = 0;
+  BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.rowstart + (int64_t)H * R, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  *nnz = total;
+  return BSP_OK;
+}
+
+extern "C" int bsp_softmax_lut_build(const int32_t *d_layout, int H, int R, int C, int32_t *d_lut, int64_t lut_cap, void *d_ws,
+                                     int64_t ws_bytes, int64_t *lut_len, int *maxlut, void *stream) {
+  int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
+  if (rc != BSP_OK) return rc;
+  if (!d_lut || !lut_len || !maxlut) return BSP_ERR_ARG;
+  hipStream_t st = as_stream(stream);
+  Ws o(H, R, C);
+  int32_t *ws = (int32_t *)d_ws;
+  rc = prepare_counts(d_layout, H, R, C, ws, o, st);
+  if (rc != BSP_OK) return rc;
+  int32_t host[2];
+  BSP_HIP_CHECK(hipMemcpyAsync(&host[0], ws + o.rowstart + (int64_t)H * R, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipMemcpyAsync(&host[1], ws + o.scal + S_MAXLUT, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  const int64_t need = 2 * (int64_t)H * R + 4 * (int64_t)host[0];
+  *lut_len = need;
+  *maxlut = host[1];
+  if (need > lut_cap) return BSP_ERR_CAPACITY;
+  hipLaunchKernelGGL(k_softmax_lut, dim3(cdiv((int64_t)H * R, 256)), dim3(256), 0, st, d_layout, H, R, C, ws + o.rowcnt,
+                     ws + o.rowstart, d_lut);
+  BSP_LAUNCH_CHECK();
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  return BSP_OK;
+}
+
+extern "C" int64_t bsp_dxx_lut_cap(int H, int R, int C, int64_t nnz, int block, int step, int trans) {
+  if (step <= 0 || block < step) return 0;
+  int64_t lines = (int64_t)H * (trans ? R : C);
+  return 6 * 2 * lines + 2 * nnz * (block / step) + 2;   // every line yields at most two segments
+}
+
+extern "C" int bsp_dxx_lut_build(const int32_t *d_layout, int H, int R, int C, int block, int step, int trans, int32_t *d_lut,
+                                 int64_t lut_cap, int32_t *d_plan, void *d_ws, int64_t ws_bytes, int64_t *lut_len, int *width,
+                                 int *num_locks, void *stream) {
+  int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
+  if (rc != BSP_OK) return rc;
+  if (!d_lut || !d_plan || !lut_len || !width || !num_locks || step <= 0 || block < step || block % step) return BSP_ERR_ARG;
+  hipStream_t st = as_stream(stream);
+  Ws o(H, R, C);
+  int32_t *ws = (int32_t *)d_ws;
+  const int T = 256;
+  const int L = trans ? R : C;
+  const int64_t lines = (int64_t)H * L;
+  rc = prepare_counts(d_layout, H, R, C, ws, o, st);
+  if (rc != BSP_OK) return rc;
+  hipLaunchKernelGGL(k_rank, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowstart, ws + o.rank);
+  const int32_t *sizes, *blkstart;
+  if (trans) {
+    sizes = ws + o.rowcnt; blkstart = ws + o.rowstart;
+  } else {
+    hipLaunchKernelGGL(k_col_counts, dim3(cdiv((int64_t)H * C, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.colcnt);
+    hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.colcnt, ws + o.colstart, (int64_t)H * C, (int32_t *)nullptr);
+    sizes = ws + o.colcnt; blkstart = ws + o.colstart;
+  }
+  hipLaunchKernelGGL(k_head_max, dim3(cdiv(H, 64)), dim3(64), 0, st, sizes, H, L, ws + o.headmax, ws + o.scal);
+  hipLaunchKernelGGL(k_line_packs, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, H, L, ws + o.linepacks);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.linepacks, ws + o.segstart, lines, (int32_t *)nullptr);
+  BSP_LAUNCH_CHECK();
+  int32_t host[3];
+  BSP_HIP_CHECK(hipMemcpyAsync(&host[0], ws + o.segstart + lines, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipMemcpyAsync(&host[1], blkstart + lines, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipMemcpyAsync(&host[2], ws + o.scal + S_ERR, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  if (host[2] != 0) return host[2];
+  const int64_t w = host[0], nnz = host[1];
+  if (nnz <= 0) return BSP_ERR_EMPTY_HEAD;
+  const int64_t need = 6 * w + 2 * nnz * (block / step) + 2;
+  *lut_len = need; *width = (int)w; *num_locks = 1;   // max(1, lockid.max()) with lockid == 0 everywhere (matmul.py:457)
+  if (need > lut_cap) return BSP_ERR_CAPACITY;
+  hipLaunchKernelGGL(k_dxx_header, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, ws + o.segstart, blkstart, H, L, block, step, d_lut);
+  hipLaunchKernelGGL(k_dxx_plan, dim3(cdiv(lines, T)), dim3(T), 0, st, d_layout, ws + o.rank, blkstart, H, R, C, block, trans, d_plan);
+  hipLaunchKernelGGL(k_dxx_incs, dim3(cdiv(nnz, T)), dim3(T), 0, st, d_plan, nnz, block, step, trans, w, d_lut);
+  hipLaunchKernelGGL(k_dxx_fix, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, ws + o.segstart, blkstart, d_plan, H, L, block, step, d_lut);
+  BSP_LAUNCH_CHECK();
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  return BSP_OK;
+}
+
+extern "C" int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_width, int32_t *d_lut, uint8_t *d_valid,
+                                 int64_t cap_rows, void *d_ws, int64_t ws_bytes, int *n_levels, int *packs, int64_t *rows,
+                                 int64_t *total_rows, int *all_valid, void *stream) {
+  int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
+  if (rc != BSP_OK) return rc;
+  if (!d_lut || !d_valid || !n_levels || !packs || !rows || !total_rows || !all_valid) return BSP_ERR_ARG;
+  if (start_width != 1 && start_width != 2 && start_width != 4) return BSP_ERR_UNSUPPORTED;
+  hipStream_t st = as_stream(stream);
+  Ws o(H, R, C);
+  int32_t *ws = (int32_t *)d_ws;
+  const int T = 256;
+  const int64_t cells = (int64_t)H * R * C;
+  int nlev = 0;
+  for (int w = start_width; w > 0; w >>= 1) nlev++;
+  rc = prepare_counts(d_layout, H, R, C, ws, o, st);
+  if (rc != BSP_OK) return rc;
+  hipLaunchKernelGGL(k_rank, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowstart, ws + o.rank);
+  int64_t *counts = (int64_t *)(ws + o.counts), *offsets = (int64_t *)(ws + o.offsets);
+  // counting pass
+  BSP_HIP_CHECK(hipMemcpyAsync(ws + o.lay, d_layout, cells * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+  hipLaunchKernelGGL(k_sdd_segment, dim3(H), dim3(64), 0, st, ws + o.lay, ws + o.rank, ws + o.tmp, ws + o.top, H, R, C, start_width, 0,
+                     counts, offsets, d_lut, d_valid, cap_rows, ws + o.scal);
+  hipLaunchKernelGGL(k_sdd_offsets, dim3(1), dim3(64), 0, st, counts, offsets, nlev, H, ws + o.scal);
+  BSP_LAUNCH_CHECK();
+  int64_t hcounts[8 * 64];
+  int64_t *hc = hcounts;
+  int64_t *heap = nullptr;
+  if ((int64_t)nlev * H > 8 * 64) { heap = new int64_t[(size_t)nlev * H]; hc = heap; }
+  hipError_t e = hipMemcpyAsync(hc, counts, sizeof(int64_t) * nlev * H, hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) { delete[] heap; return BSP_ERR_HIP; }
+  int levels = 0; int64_t total = 0; int lev = 0;
+  for (int w = start_width; w > 0; w >>= 1, lev++) {
+    int64_t r = 0;
+    for (int h = 0; h < H; h++) r += hc[lev * H + h];
+    if (r > 0) { packs[levels] = w; rows[levels] = r; levels++; total += r; }   // empty levels are not returned (utils.cpp:90-91)
+  }
+  delete[] heap;
+  *n_levels = levels; *total_rows = total;
+  if (total > cap_rows) return BSP_ERR_CAPACITY;
+  // writing pass on a fresh copy
+  BSP_HIP_CHECK(hipMemcpyAsync(ws + o.lay, d_layout, cells * sizeof(int32_t), hipMemcpyDeviceToDevice, st));
+  hipLaunchKernelGGL(k_sdd_segment, dim3(H), dim3(64), 0, st, ws + o.lay, ws + o.rank, ws + o.tmp, ws + o.top, H, R, C, start_width, 1,
+                     counts, offsets, d_lut, d_valid, cap_rows, ws + o.scal);
+  BSP_LAUNCH_CHECK();
+  int32_t inval = 0;
+  BSP_HIP_CHECK(hipMemcpyAsync(&inval, ws + o.scal + S_INVALID, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  *all_valid = inval ? 0 : 1;
+  return BSP_OK;
+}

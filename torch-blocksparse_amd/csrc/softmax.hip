@@ -1,0 +1,408 @@
+// Block-sparse softmax, forward and backward, for gfx950.
+//
+// Replaces the reference's softmax_fwd / softmax_bwd (softmax.py:7-138, 144-194).  The reference runs one
+// program per matrix row; here one 64-lane wavefront owns 16 consecutive rows of one block-row: 4 lanes
+// share a row, every lane keeps BLOCK/4 columns of each of the row's nonzero blocks in registers, and the
+// row maximum / sum are two xor-shuffles.  Each block is read and written exactly once with 16-byte
+// accesses, so the kernel moves the algorithmic 2 (forward) or 3 (backward) passes over x and nothing more.
+// Rows with more blocks than fit in registers take a streaming variant that re-reads x.
+#include "bsp_common.h"
+
+namespace bsp {
+namespace {
+
+constexpr int kRowsPerWave = 16;
+constexpr int kLanesPerRow = 4;
+constexpr int kWavesPerGroup = 4;
+
+template <typename T, int EV> struct RawVec;
+template <> struct RawVec<f16, 8> { typedef u32x4 type; };
+template <> struct RawVec<bf16, 8> { typedef u32x4 type; };
+template <> struct RawVec<f16, 4> { typedef u32x2 type; };
+template <> struct RawVec<bf16, 4> { typedef u32x2 type; };
+template <> struct RawVec<float, 4> { typedef u32x4 type; };
+
+template <typename T, int EV> struct Pack {
+  typedef typename RawVec<T, EV>::type raw_t;
+  union { raw_t raw; T e[EV]; };
+  __device__ __forceinline__ void load(const T *p) { raw = *reinterpret_cast<const raw_t *>(p); }
+  __device__ __forceinline__ void store(T *p) const { *reinterpret_cast<raw_t *>(p) = raw; }
+};
+
+__device__ __forceinline__ float row_max(float v) {
+  v = fmaxf(v, __shfl_xor(v, 1));
+  v = fmaxf(v, __shfl_xor(v, 2));
+  return v;
+}
+__device__ __forceinline__ float row_sum(float v) {
+  v += __shfl_xor(v, 1);
+  v += __shfl_xor(v, 2);
+  return v;
+}
+
+template <typename T> __device__ __forceinline__ float exp_sub(float x, float mx) {
+  if constexpr (sizeof(T) == 4) return expf(x - mx);
+  else return __builtin_amdgcn_exp2f((x - mx) * 1.44269504088896340736f);
+}
+
+struct FwdArgs {
+  void *x; float scale; const int32_t *lut;
+  const void *rpe; int64_t rpe_sz, rpe_sh, rpe_sr;
+  const void *kpm; int64_t kpm_sz; int kpm_mul;
+  const void *attn; int64_t attn_sr; int attn_mul;
+  int Z, H, R; int64_t x_sz; int64_t n_units;
+};
+
+// where does this wavefront work?  unit = ((z * H*R) + block-row) * (BLOCK/16) + 16-row group
+template <int BLOCK> struct Unit {
+  int z, hr, rxm, q;   // batch, head*R + block-row, row inside the block, lane's position inside the row
+  bool ok;
+  __device__ __forceinline__ Unit(int64_t n_units, int HR) {
+    constexpr int G = BLOCK / kRowsPerWave;
+    const int64_t n_wg = (n_units + kWavesPerGroup - 1) / kWavesPerGroup;
+    const int64_t wg = xcd_remap(blockIdx.x, n_wg);
+    const int64_t u = wg * kWavesPerGroup + (threadIdx.x >> 6);
+    ok = u < n_units;
+    const int lane = threadIdx.x & 63;
+    const int g = (int)(u % G);
+    const int64_t t = u / G;
+    hr = (int)(t % HR);
+    z = (int)(t / HR);
+    rxm = g * kRowsPerWave + lane / kLanesPerRow;
+    q = lane % kLanesPerRow;
+  }
+};
+
+// The lane's columns inside a block: chunk j (of NJ) starts at (j*4 + q)*EV, so that the four lanes of a row
+// cover 4*EV consecutive elements per load instruction.
+template <typename T, int BLOCK> struct Cols {
+  static constexpr int VEC = BLOCK / kLanesPerRow;
+  static constexpr int EV = VEC < (int)(16 / sizeof(T)) ? VEC : (int)(16 / sizeof(T));
+  static constexpr int NJ = VEC / EV;
+  __device__ static __forceinline__ int col(int j, int q) { return (j * kLanesPerRow + q) * EV; }
+};
+
+template <typename T, int BLOCK>
+__device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
+                                           float (&fx)[Cols<T, BLOCK>::VEC]) {
+  typedef Cols<T, BLOCK> CL;
+  const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK;
+  const int64_t grow = (int64_t)brow * BLOCK + u.rxm;   // row in the dense matrix
+  const int64_t gcol = (int64_t)bcol * BLOCK;           // first column of the block in the dense matrix
+#pragma unroll
+  for (int j = 0; j < CL::NJ; j++) {
+    const int c = CL::col(j, u.q);
+    Pack<T, CL::EV> px;
+    px.load(x + c);
+#pragma unroll
+    for (int e = 0; e < CL::EV; e++) fx[j * CL::EV + e] = to_float(px.e[e]) * a.scale;          // softmax.py:112-116
+    if (a.rpe) {                                                                                // :118-120, address :50-55
+      Pack<T, CL::EV> p;
+      p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol + c);
+#pragma unroll
+      for (int e = 0; e < CL::EV; e++) fx[j * CL::EV + e] += to_float(p.e[e]);
+    }
+    if (a.kpm) {                                                                                // :122-124, address :60-62
+      Pack<T, CL::EV> p;
+      p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol + c);
+#pragma unroll
+      for (int e = 0; e < CL::EV; e++) {
+        float m = to_float(p.e[e]);
+        if (a.kpm_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                        // :104-106
+        fx[j * CL::EV + e] += m;
+      }
+    }
+    if (a.attn) {                                                                               // :126-128, address :67-70
+      Pack<T, CL::EV> p;
+      p.load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol + c);
+#pragma unroll
+      for (int e = 0; e < CL::EV; e++) {
+        float m = to_float(p.e[e]);
+        if (a.attn_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                       // :108-110
+        fx[j * CL::EV + e] += m;
+      }
+    }
+  }
+}
+
+template <typename T, int BLOCK>
+__device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<BLOCK> &u, int64_t blockid, const float (&y)[Cols<T, BLOCK>::VEC]) {
+  typedef Cols<T, BLOCK> CL;
+  T *x = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK;
+#pragma unroll
+  for (int j = 0; j < CL::NJ; j++) {
+    Pack<T, CL::EV> p;
+#pragma unroll
+    for (int e = 0; e < CL::EV; e++) p.e[e] = from_float<T>(y[j * CL::EV + e]);
+    p.store(x + CL::col(j, u.q));
+  }
+}
+
+// NB = number of blocks of a row kept in registers; NB == 0 selects the streaming variant.
+template <typename T, int BLOCK, int NB>
+__global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
+  typedef Cols<T, BLOCK> CL;
+  const int HR = a.H * a.R;
+  Unit<BLOCK> u(a.n_units, HR);
+  if (!u.ok) return;
+  const int size = a.lut[2 * u.hr + 0];                 // header (size, offset), softmax.py:30-32
+  const int offset = a.lut[2 * u.hr + 1];
+  const int head = u.hr / a.R, brow = u.hr % a.R;       // = the table's (row, head) fields of every block of this row
+  if (size <= 0) return;
+  const int32_t *core = a.lut + offset;
+  if constexpr (NB > 0) {
+    float fx[NB][CL::VEC];
+    int32_t bid[NB];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+        bid[b] = core[4 * b + 0];
+        fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], bid[b], fx[b]);
+#pragma unroll
+        for (int e = 0; e < CL::VEC; e++) mx = fmaxf(mx, fx[b][e]);
+      }
+    mx = row_max(mx);                                   // :130
+    float sum = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int e = 0; e < CL::VEC; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
+      }
+    sum = row_sum(sum);
+    const float inv = 1.f / sum;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int e = 0; e < CL::VEC; e++) fx[b][e] *= inv;                                            // :137
+        fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
+      }
+  } else {
+    float fx[CL::VEC];
+    float mx = -INFINITY;
+    for (int b = 0; b < size; b++) {
+      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+#pragma unroll
+      for (int e = 0; e < CL::VEC; e++) mx = fmaxf(mx, fx[e]);
+    }
+    mx = row_max(mx);
+    float sum = 0.f;
+    for (int b = 0; b < size; b++) {
+      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+#pragma unroll
+      for (int e = 0; e < CL::VEC; e++) sum += exp_sub<T>(fx[e], mx);
+    }
+    sum = row_sum(sum);
+    const float inv = 1.f / sum;
+    for (int b = 0; b < size; b++) {
+      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+#pragma unroll
+      for (int e = 0; e < CL::VEC; e++) fx[e] = exp_sub<T>(fx[e], mx) * inv;
+      fwd_store<T, BLOCK>(a, u, core[4 * b + 0], fx);
+    }
+  }
+}
+
+struct BwdArgs {
+  const void *y; void *dy; float scale; const int32_t *lut;
+  int Z, H, R; int64_t y_sz, dy_sz; int64_t n_units;
+};
+
+template <typename T, int BLOCK, int NB>
+__global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
+  typedef Cols<T, BLOCK> CL;
+  typedef Pack<T, CL::EV> P;
+  const int HR = a.H * a.R;
+  Unit<BLOCK> u(a.n_units, HR);
+  if (!u.ok) return;
+  const int size = a.lut[2 * u.hr + 0];
+  const int offset = a.lut[2 * u.hr + 1];
+  if (size <= 0) return;
+  const int32_t *core = a.lut + offset;
+  const T *yb = reinterpret_cast<const T *>(a.y) + (int64_t)u.z * a.y_sz + u.rxm * BLOCK;
+  T *db = reinterpret_cast<T *>(a.dy) + (int64_t)u.z * a.dy_sz + u.rxm * BLOCK;
+  if constexpr (NB > 0) {
+    P py[NB][CL::NJ], pd[NB][CL::NJ];
+    int32_t bid[NB];
+    float dot = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+        bid[b] = core[4 * b];
+        const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
+#pragma unroll
+        for (int j = 0; j < CL::NJ; j++) {
+          py[b][j].load(yb + o + CL::col(j, u.q));
+          pd[b][j].load(db + o + CL::col(j, u.q));
+        }
+      }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int j = 0; j < CL::NJ; j++)
+#pragma unroll
+          for (int e = 0; e < CL::EV; e++) dot += to_float(py[b][j].e[e]) * to_float(pd[b][j].e[e]);   // softmax.py:187-188
+      }
+    dot = row_sum(dot);
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+        const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
+#pragma unroll
+        for (int j = 0; j < CL::NJ; j++) {
+          P out;
+#pragma unroll
+          for (int e = 0; e < CL::EV; e++)
+            out.e[e] = from_float<T>(to_float(py[b][j].e[e]) * (to_float(pd[b][j].e[e]) - dot) * a.scale);   // :189
+          out.store(db + o + CL::col(j, u.q));
+        }
+      }
+  } else {
+    float dot = 0.f;
+    for (int b = 0; b < size; b++) {
+      const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
+#pragma unroll
+      for (int j = 0; j < CL::NJ; j++) {
+        P py, pd;
+        py.load(yb + o + CL::col(j, u.q));
+        pd.load(db + o + CL::col(j, u.q));
+#pragma unroll
+        for (int e = 0; e < CL::EV; e++) dot += to_float(py.e[e]) * to_float(pd.e[e]);
+      }
+    }
+    dot = row_sum(dot);
+    for (int b = 0; b < size; b++) {
+      const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
+#pragma unroll
+      for (int j = 0; j < CL::NJ; j++) {
+        P py, pd, out;
+        py.load(yb + o + CL::col(j, u.q));
+        pd.load(db + o + CL::col(j, u.q));
+#pragma unroll
+        for (int e = 0; e < CL::EV; e++) out.e[e] = from_float<T>(to_float(py.e[e]) * (to_float(pd.e[e]) - dot) * a.scale);
+        out.store(db + o + CL::col(j, u.q));
+      }
+    }
+  }
+}
+
+// Register budget: a lane keeps NB * BLOCK/4 values (forward, fp32) or twice that many raw elements (backward).
+template <typename T, int BLOCK> constexpr int max_nb_fwd() { return 128 / (BLOCK / 4); }
+template <typename T, int BLOCK> constexpr int max_nb_bwd() { return (int)(128 * 4 / (2 * (BLOCK / 4) * sizeof(T))) > 32 ? 32 : (int)(128 * 4 / (2 * (BLOCK / 4) * sizeof(T))); }
+
+template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
+  const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
+  hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+}
+template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hipStream_t st) {
+  const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
+  hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+}
+
+template <typename T, int BLOCK> void launch_fwd(const FwdArgs &a, int maxlut, hipStream_t st) {
+  constexpr int MX = max_nb_fwd<T, BLOCK>();
+  if (maxlut <= 1 && 1 <= MX) launch_fwd_nb<T, BLOCK, 1>(a, st);
+  else if (maxlut <= 2 && 2 <= MX) launch_fwd_nb<T, BLOCK, 2>(a, st);
+  else if (maxlut <= 4 && 4 <= MX) launch_fwd_nb<T, BLOCK, 4>(a, st);
+  else if (maxlut <= 8 && 8 <= MX) launch_fwd_nb<T, BLOCK, (8 <= MX ? 8 : 0)>(a, st);
+  else if (maxlut <= 16 && 16 <= MX) launch_fwd_nb<T, BLOCK, (16 <= MX ? 16 : 0)>(a, st);
+  else if (maxlut <= 32 && 32 <= MX) launch_fwd_nb<T, BLOCK, (32 <= MX ? 32 : 0)>(a, st);
+  else launch_fwd_nb<T, BLOCK, 0>(a, st);
+}
+template <typename T, int BLOCK> void launch_bwd(const BwdArgs &a, int maxlut, hipStream_t st) {
+  constexpr int MX = max_nb_bwd<T, BLOCK>();
+  if (maxlut <= 1 && 1 <= MX) launch_bwd_nb<T, BLOCK, 1>(a, st);
+  else if (maxlut <= 2 && 2 <= MX) launch_bwd_nb<T, BLOCK, (2 <= MX ? 2 : 0)>(a, st);
+  else if (maxlut <= 4 && 4 <= MX) launch_bwd_nb<T, BLOCK, (4 <= MX ? 4 : 0)>(a, st);
+  else if (maxlut <= 8 && 8 <= MX) launch_bwd_nb<T, BLOCK, (8 <= MX ? 8 : 0)>(a, st);
+  else if (maxlut <= 16 && 16 <= MX) launch_bwd_nb<T, BLOCK, (16 <= MX ? 16 : 0)>(a, st);
+  else if (maxlut <= 32 && 32 <= MX) launch_bwd_nb<T, BLOCK, (32 <= MX ? 32 : 0)>(a, st);
+  else launch_bwd_nb<T, BLOCK, 0>(a, st);
+}
+
+template <typename T> int dispatch_fwd(const FwdArgs &a, int block, int maxlut, hipStream_t st) {
+  switch (block) {
+    case 16: launch_fwd<T, 16>(a, maxlut, st); break;
+    case 32: launch_fwd<T, 32>(a, maxlut, st); break;
+    case 64: launch_fwd<T, 64>(a, maxlut, st); break;
+    case 128: launch_fwd<T, 128>(a, maxlut, st); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  return BSP_OK;
+}
+template <typename T> int dispatch_bwd(const BwdArgs &a, int block, int maxlut, hipStream_t st) {
+  switch (block) {
+    case 16: launch_bwd<T, 16>(a, maxlut, st); break;
+    case 32: launch_bwd<T, 32>(a, maxlut, st); break;
+    case 64: launch_bwd<T, 64>(a, maxlut, st); break;
+    case 128: launch_bwd<T, 128>(a, maxlut, st); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  return BSP_OK;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+}  // namespace
+}  // namespace bsp
+
+using namespace bsp;
+
+extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int maxlut, const void *rpe,
+                               int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm,
+                               int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r, int attn_mul, int Z,
+                               int H, int R, int block, int64_t x_stride_z, void *stream) {
+  if (!x || !d_lut || Z <= 0 || H <= 0 || R <= 0 || maxlut < 0) return BSP_ERR_ARG;
+  if ((int64_t)maxlut * block >= 32768) return BSP_ERR_ROW_TOO_LONG;   // softmax.py:225-227
+  const int64_t es = dtype == BSP_F32 ? 4 : 2;
+  // vector accesses: every row segment a lane touches must start on a 16-byte boundary
+  const int64_t unit = 16 / es;
+  if (!aligned16(x) || !aligned16(rpe) || !aligned16(kpm) || !aligned16(attn)) return BSP_ERR_ARG;
+  if (x_stride_z % unit || rpe_stride_z % unit || rpe_stride_h % unit || rpe_stride_r % unit || kpm_stride_z % unit ||
+      attn_stride_r % unit)
+    return BSP_ERR_ARG;
+  FwdArgs a;
+  a.x = x; a.scale = scale; a.lut = d_lut;
+  a.rpe = rpe; a.rpe_sz = rpe_stride_z; a.rpe_sh = rpe_stride_h; a.rpe_sr = rpe_stride_r;
+  a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
+  a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
+  a.Z = Z; a.H = H; a.R = R; a.x_sz = x_stride_z;
+  a.n_units = (int64_t)Z * H * R * (block / 16);
+  if (a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  int rc;
+  switch (dtype) {
+    case BSP_F16: rc = dispatch_fwd<f16>(a, block, maxlut, as_stream(stream)); break;
+    case BSP_BF16: rc = dispatch_fwd<bf16>(a, block, maxlut, as_stream(stream)); break;
+    case BSP_F32: rc = dispatch_fwd<float>(a, block, maxlut, as_stream(stream)); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
+extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
+                               int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream) {
+  if (!y || !dy || !d_lut || Z <= 0 || H <= 0 || R <= 0 || maxlut < 0) return BSP_ERR_ARG;
+  if ((int64_t)maxlut * block >= 32768) return BSP_ERR_ROW_TOO_LONG;
+  const int64_t unit = dtype == BSP_F32 ? 4 : 8;
+  if (!aligned16(y) || !aligned16(dy) || y_stride_z % unit || dy_stride_z % unit) return BSP_ERR_ARG;
+  BwdArgs a;
+  a.y = y; a.dy = dy; a.scale = scale; a.lut = d_lut;
+  a.Z = Z; a.H = H; a.R = R; a.y_sz = y_stride_z; a.dy_sz = dy_stride_z;
+  a.n_units = (int64_t)Z * H * R * (block / 16);
+  if (a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  int rc;
+  switch (dtype) {
+    case BSP_F16: rc = dispatch_bwd<f16>(a, block, maxlut, as_stream(stream)); break;
+    case BSP_BF16: rc = dispatch_bwd<bf16>(a, block, maxlut, as_stream(stream)); break;
+    case BSP_F32: rc = dispatch_bwd<float>(a, block, maxlut, as_stream(stream)); break;
+    default: return BSP_ERR_UNSUPPORTED;
+  }
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}

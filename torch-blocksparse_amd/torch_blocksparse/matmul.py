@@ -1,0 +1,344 @@
+"""Block-sparse matrix multiplication (sdd / dsd / dds) on MI355X.
+
+Drop-in for the reference's torch_blocksparse/matmul.py: same `MatMul(layout, block, mode, trans_a, trans_b,
+bench)` object, same sparse storage ([Z, nnz, block, block], blocks in layout.nonzero() order), same
+look-up tables (built on the GPU, bit-identical to matmul.py:221-297 and :372-458), same autograd wiring
+(matmul.py:558-606).  The kernels are HIP/MFMA kernels reached through the C ABI in include/bsp.h.
+"""
+import ctypes
+import math
+
+import torch
+
+from . import _lib
+
+
+def _vec(dtype):
+    return 4 if dtype == torch.float32 else 8
+
+
+def _prep(x):
+    """Operands are read with 16-byte vector loads along a unit inner stride."""
+    v = _vec(x.dtype)
+    ok = x.stride(-1) == 1 and x.data_ptr() % 16 == 0 and all(s % v == 0 for s in x.stride()[:-1])
+    return x if ok else x.contiguous()
+
+
+class _Timer:
+    """Event timing of one launch when bench=True (milliseconds); the reference stores the JIT's own timing."""
+
+    def __init__(self, bench, device):
+        self.bench = bench
+        if bench:
+            self.start = torch.cuda.Event(enable_timing=True)
+            self.stop = torch.cuda.Event(enable_timing=True)
+            self.start.record(torch.cuda.current_stream(device))
+        self.device = device
+
+    def done(self):
+        if not self.bench:
+            return None
+        self.stop.record(torch.cuda.current_stream(self.device))
+        self.stop.synchronize()
+        return self.start.elapsed_time(self.stop)
+
+
+class SddTables(list):
+    """The per-pack sdd tables, in the reference's order; `nnz` is the number of blocks of the output."""
+    nnz = 0
+
+
+class _sparse_matmul(torch.autograd.Function):
+
+    ##########################
+    # SPARSE = DENSE x DENSE #
+    ##########################
+    @staticmethod
+    def make_sdd_lut(layout, block, dtype, device):
+        """-> (luts, None, widths, packs) as the reference (matmul.py:281-297); built on `device`.
+
+        start_width is 64 // block in the reference, which is 0 for block 128 and leaves the table empty
+        (matmul.py:283, csrc/utils.cpp:117); max(1, .) gives block 128 the single-block table it needs.
+        Each table tensor carries `.valid` (None, or a uint8 tensor marking the rows that really are blocks).
+        """
+        lib = _lib.load()
+        dev = torch.device(device)
+        lay = _lib.layout_to_device(layout, dev)
+        H, R, C = lay.shape
+        ws, ws_bytes = _lib.workspace(lay, dev)
+        start_width = max(1, 64 // block)
+        nnz = int((layout != 0).sum())
+        cap = nnz + nnz // 8 + 64
+        n_levels = ctypes.c_int(0)
+        packs = (ctypes.c_int * 8)()
+        rows = (ctypes.c_int64 * 8)()
+        total = ctypes.c_int64(0)
+        all_valid = ctypes.c_int(1)
+        for attempt in range(2):
+            lut = torch.empty((cap, 4), dtype=torch.int32, device=dev)
+            valid = torch.empty((cap,), dtype=torch.uint8, device=dev)
+            rc = lib.bsp_sdd_lut_build(_lib.ptr(lay), H, R, C, start_width, _lib.ptr(lut), _lib.ptr(valid), cap, _lib.ptr(ws),
+                                       ws_bytes, ctypes.byref(n_levels), packs, rows, ctypes.byref(total),
+                                       ctypes.byref(all_valid), _lib.stream_ptr(dev))
+            if rc == _lib.ERR_CAPACITY and attempt == 0:
+                cap = int(total.value)
+                continue
+            _lib.check(rc, 'bsp_sdd_lut_build')
+            break
+        luts, widths, out_packs = SddTables(), [], []
+        luts.nnz = nnz
+        done = 0
+        for k in range(n_levels.value):
+            p, r = int(packs[k]), int(rows[k])
+            t = lut[done:done + r].reshape(-1)
+            t.valid = None if all_valid.value else valid[done:done + r]
+            luts.append(t)
+            widths.append(r // (p * p))
+            out_packs.append(p)
+            done += r
+        return luts, None, widths, out_packs
+
+    @staticmethod
+    def _sdd_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, luts, num_locks, widths, packs, bench, time):
+        if trans_c:                                   # matmul.py:303-305
+            a, b = b, a
+            trans_a, trans_b = not trans_b, not trans_a
+        a, b = _prep(a), _prep(b)
+        AS0 = a.size(0)
+        AS3 = a.size(2 if trans_a else 3)
+        if AS3 % 16 != 0:
+            raise ValueError('Reduction size for SDD must be a multiple of 16')
+        if b.size(0) != AS0 or b.size(1) != a.size(1) or b.size(3 if trans_b else 2) != AS3:
+            raise ValueError('incompatible operand shapes for sdd: %s and %s' % (tuple(a.shape), tuple(b.shape)))
+        lib = _lib.load()
+        total_width = luts.nnz if isinstance(luts, SddTables) else sum(w * p * p for w, p in zip(widths, packs))
+        c = torch.empty((AS0, total_width, block, block), dtype=a.dtype, device=a.device)
+        timer = _Timer(bench, a.device)
+        for lut, width, pack in zip(luts, widths, packs):
+            rc = lib.bsp_sdd_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
+                                    AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
+                                    c.stride(0), block, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
+                                    _lib.stream_ptr(a.device))
+            _lib.check(rc, 'bsp_sdd_matmul')
+        time[0] = timer.done()
+        return c
+
+    ##########################
+    # DENSE = DENSE x SPARSE #
+    ##########################
+    @staticmethod
+    def make_dxx_lut(layout, block, step, trans, device, transform=lambda idx: idx):
+        """-> (lut, num_locks, width, None) as the reference (matmul.py:372-458); built on `device`.
+
+        The table tensor carries `.plan`: per block, in table order, (position in the dense operand's reduction
+        dimension, storage index) -- the absolute values the table's increments are differences of.
+        """
+        lib = _lib.load()
+        dev = torch.device(device)
+        lay = _lib.layout_to_device(layout, dev)
+        H, R, C = lay.shape
+        ws, ws_bytes = _lib.workspace(lay, dev)
+        nnz = int((layout != 0).sum())
+        cap = lib.bsp_dxx_lut_cap(H, R, C, nnz, block, step, int(bool(trans)))
+        lut = torch.empty((cap,), dtype=torch.int32, device=dev)
+        plan = torch.empty((max(nnz, 1), 2), dtype=torch.int32, device=dev)
+        n = ctypes.c_int64(0)
+        width = ctypes.c_int(0)
+        num_locks = ctypes.c_int(0)
+        rc = lib.bsp_dxx_lut_build(_lib.ptr(lay), H, R, C, block, step, int(bool(trans)), _lib.ptr(lut), cap, _lib.ptr(plan),
+                                   _lib.ptr(ws), ws_bytes, ctypes.byref(n), ctypes.byref(width), ctypes.byref(num_locks),
+                                   _lib.stream_ptr(dev))
+        if rc == _lib.ERR_EMPTY_HEAD:
+            raise RuntimeError('block-sparse layout has a head without any nonzero block')
+        _lib.check(rc, 'bsp_dxx_lut_build')
+        lut = lut[:n.value]
+        lut.plan = plan
+        return lut, num_locks.value, width.value, None
+
+    @staticmethod
+    def _pad_free_dim(x, dim, v):
+        pad = (-x.size(dim)) % v
+        if pad == 0:
+            return x
+        shape = list(x.shape)
+        shape[dim] = pad
+        return torch.cat((x, x.new_zeros(shape)), dim=dim)
+
+    @staticmethod
+    def _dds_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, lut, num_locks, width, packs, bench, time):
+        v = _vec(a.dtype)
+        AS2 = a.size(3 if trans_a else 2)                     # free dimension M (matmul.py:467)
+        a = _prep(_sparse_matmul._pad_free_dim(a, 3 if trans_a else 2, v))
+        M = a.size(3 if trans_a else 2)
+        b = b if b.is_contiguous() else b.contiguous()
+        BS2 = block * spdims[1 if trans_b else 2]             # matmul.py:471
+        CS2, CS3 = (BS2, M) if trans_c else (M, BS2)
+        c = torch.empty((a.size(0), a.size(1), CS2, CS3), dtype=a.dtype, device=a.device)
+        b_sz = b.stride(0) if (b.dim() == 4 and b.size(0) > 1) else 0   # a 3-D (or batch-1) sparse operand is shared by the batch
+        timer = _Timer(bench, a.device)
+        rc = _lib.load().bsp_dds_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
+                                        int(trans_c), a.size(0), M, a.stride(0), a.stride(1), a.stride(2), b_sz, c.stride(0),
+                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
+                                        _lib.stream_ptr(a.device))
+        _lib.check(rc, 'bsp_dds_matmul')
+        time[0] = timer.done()
+        if M != AS2:
+            c = c[:, :, :, :AS2] if trans_c else c[:, :, :AS2, :]
+        return c
+
+    @staticmethod
+    def _dsd_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, lut, num_locks, width, packs, bench, time):
+        v = _vec(b.dtype)
+        BS3 = b.size(2 if trans_b else 3)                     # free dimension N (matmul.py:518)
+        b = _prep(_sparse_matmul._pad_free_dim(b, 2 if trans_b else 3, v))
+        N = b.size(2 if trans_b else 3)
+        a = a if a.is_contiguous() else a.contiguous()
+        AS1 = block * spdims[2 if trans_a else 1]             # matmul.py:513
+        CS2, CS3 = (N, AS1) if trans_c else (AS1, N)
+        c = torch.empty((b.size(0), b.size(1), CS2, CS3), dtype=b.dtype, device=b.device)
+        a_sz = a.stride(0) if (a.dim() == 4 and a.size(0) > 1) else 0
+        timer = _Timer(bench, b.device)
+        rc = _lib.load().bsp_dsd_matmul(_lib.DTYPES[b.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
+                                        int(trans_c), b.size(0), N, a_sz, b.stride(0), b.stride(1), b.stride(2), c.stride(0),
+                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
+                                        _lib.stream_ptr(b.device))
+        _lib.check(rc, 'bsp_dsd_matmul')
+        time[0] = timer.done()
+        if N != BS3:
+            c = c[:, :, :BS3, :] if trans_c else c[:, :, :, :BS3]
+        return c
+
+    fn = {'sdd': _sdd_matmul.__get__(object),
+          'dsd': _dsd_matmul.__get__(object),
+          'dds': _dds_matmul.__get__(object)}
+
+    @staticmethod
+    def forward(ctx, a, b, trans_a, trans_b, trans_c, mode, spdims, block,
+                c_lut, c_num_locks, c_width, c_packs, c_bench, c_time,
+                da_lut, da_num_locks, da_width, da_packs, da_bench, da_time,
+                db_lut, db_num_locks, db_width, db_packs, db_bench, db_time):
+        _lib.require_gpu_tensor(a, 'matmul operand a')
+        _lib.require_gpu_tensor(b, 'matmul operand b')
+        if a.dtype != b.dtype or a.dtype not in _lib.DTYPES:
+            raise ValueError('matmul operands must both be float16, bfloat16 or float32 (got %s, %s)' % (a.dtype, b.dtype))
+        c = _sparse_matmul.fn[mode](a, b, trans_a, trans_b, trans_c, spdims, block,
+                                    c_lut, c_num_locks, c_width, c_packs, c_bench, c_time)
+        ctx.save_for_backward(a, b)
+        ctx.da = (da_lut, da_num_locks, da_width, da_packs, da_bench, da_time)
+        ctx.db = (db_lut, db_num_locks, db_width, db_packs, db_bench, db_time)
+        ctx.mode, ctx.spdims, ctx.block = mode, spdims, block
+        ctx.trans_a, ctx.trans_b = trans_a, trans_b
+        return c
+
+    @staticmethod
+    def backward(ctx, dc):
+        a, b = ctx.saved_tensors
+        mode = ctx.mode
+        da = db = None
+        if ctx.needs_input_grad[0]:                           # matmul.py:593-596
+            mode_da = mode[1] + mode[0] + mode[2]
+            da = _sparse_matmul.fn[mode_da](dc, b, False, not ctx.trans_b, ctx.trans_a, ctx.spdims, ctx.block, *ctx.da)
+            if da.shape != a.shape:
+                da = da.reshape(a.shape) if da.numel() == a.numel() else da.sum(0).reshape(a.shape)
+        if ctx.needs_input_grad[1]:                           # matmul.py:598-601
+            mode_db = mode[2] + mode[1] + mode[0]
+            db = _sparse_matmul.fn[mode_db](a, dc, not ctx.trans_a, False, ctx.trans_b, ctx.spdims, ctx.block, *ctx.db)
+            if db.shape != b.shape:
+                db = db.reshape(b.shape) if db.numel() == b.numel() else db.sum(0).reshape(b.shape)
+        return (da, db) + (None,) * 24
+
+
+class MatMul:
+    """C = op(A) @ op(B) with one block-sparse participant.
+
+    mode 'sdd': C sparse, A and B dense; 'dsd': A sparse; 'dds': B sparse.  `layout` ([H, R, C], 0/1, on the CPU)
+    always describes the sparse tensor as stored.
+    """
+
+    def make_lut(self, dtype, device):
+        key = (dtype, device)
+        if key in self.lut_cache:
+            return self.lut_cache[key]
+        layout, block = self.layout, self.block
+        step = 8 if dtype == torch.float32 else 16             # matmul.py:617
+        sdd = lambda: _sparse_matmul.make_sdd_lut(layout, block, dtype, device)
+        dxx = lambda trans: _sparse_matmul.make_dxx_lut(layout, block, step, trans, device)
+        if self.mode == 'sdd':                                 # matmul.py:618-637
+            c, da, db = sdd(), dxx(True), dxx(False)
+        elif self.mode == 'dsd':
+            c, da, db = dxx(not self.trans_a), sdd(), dxx(self.trans_a)
+        else:
+            c, da, db = dxx(self.trans_b), dxx(not self.trans_b), sdd()
+        self.lut_cache[key] = c + da + db
+        return self.lut_cache[key]
+
+    def __init__(self, layout, block, mode, trans_a=False, trans_b=False, bench=False):
+        if mode not in ['sdd', 'dsd', 'dds']:
+            raise NotImplementedError('Supported modes are: sdd, dsd, dds')
+        if block not in (16, 32, 64, 128):
+            raise ValueError('block must be 16, 32, 64 or 128')
+        self.lut_cache = dict()
+        self.trans_a = trans_a
+        self.trans_b = trans_b
+        self.mode = mode
+        self.spdims = layout.shape
+        self.block = block
+        self.layout = layout
+        self.bench = bench
+        self.time_c = None
+        self.time_da = None
+        self.time_db = None
+
+    @staticmethod
+    def _pad_shape(x, is_sparse):
+        max_dim = 3 if is_sparse else 4                        # matmul.py:663-668
+        for _ in range(max_dim - x.dim()):
+            x = x.unsqueeze(0)
+        return x
+
+    def __call__(self, a, b):
+        _lib.require_gpu_tensor(a, 'matmul operand a')
+        luts = self.make_lut(a.dtype, a.device)
+        time_c, time_da, time_db = [None], [None], [None]
+        a = MatMul._pad_shape(a, self.mode == 'dsd')
+        b = MatMul._pad_shape(b, self.mode == 'dds')
+        c = _sparse_matmul.apply(a, b, self.trans_a, self.trans_b, False, self.mode, self.spdims, self.block,
+                                 luts[0], luts[1], luts[2], luts[3], self.bench, time_c,
+                                 luts[4], luts[5], luts[6], luts[7], self.bench, time_da,
+                                 luts[8], luts[9], luts[10], luts[11], self.bench, time_db)
+        self.time_c, self.time_da, self.time_db = time_c[0], time_da[0], time_db[0]
+        return c
+
+
+class Linear(torch.nn.Module):
+    """y = x @ W with a block-sparse W of shape [in_features, out_features] (blocks [nnz, block, block]).
+
+    The reference's constructor passes its arguments to MatMul in the wrong order (matmul.py:702) and cannot be
+    instantiated; this one builds the dds product it meant.
+    """
+
+    def __init__(self, in_features, out_features, block, layout, bench=False):
+        super(Linear, self).__init__()
+        if layout.dim() == 2:
+            layout = layout[None]
+        if layout.shape[0] != 1 or layout.shape[1] * block != in_features or layout.shape[2] * block != out_features:
+            raise ValueError('layout must be [1, in_features/block, out_features/block]')
+        self.in_features = in_features
+        self.out_features = out_features
+        self.block = block
+        self.weight = torch.nn.Parameter(torch.empty(int(layout.sum()), block, block))
+        self.reset_parameters()
+        self.matmul = MatMul(layout, block, 'dds', False, False, bench)
+
+    def reset_parameters(self):
+        torch.nn.init.kaiming_uniform_(self.weight, a=math.sqrt(5))
+
+    def forward(self, input):
+        shape = input.shape
+        x = input.reshape(1, 1, -1, shape[-1])
+        tokens = x.size(2)
+        pad = (-tokens) % 16     # the weight gradient is an sdd product reducing over the tokens (multiple of 16)
+        if pad:
+            x = torch.cat((x, x.new_zeros(1, 1, pad, shape[-1])), dim=2)
+        y = self.matmul(x, self.weight)[:, :, :tokens]
+        return y.reshape(shape[:-1] + (self.out_features,))

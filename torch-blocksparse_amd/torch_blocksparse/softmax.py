@@ -1,0 +1,136 @@
+"""Block-sparse softmax (forward + backward) on MI355X.
+
+Drop-in for the reference's torch_blocksparse/softmax.py: `Softmax(layout, block, bench)` and
+`softmax(x, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode)`, in place on x,
+same look-up table (softmax.py:201-221, built on the GPU), same autograd behaviour (softmax.py:253-326).
+"""
+import ctypes
+
+import torch
+
+from . import _lib
+from .matmul import _Timer
+
+
+class _sparse_softmax(torch.autograd.Function):
+
+    @staticmethod
+    def make_lut(layout, block, device):
+        """-> (lut int32 on device, maxlut) as the reference (softmax.py:201-221)."""
+        lib = _lib.load()
+        dev = torch.device(device)
+        lay = _lib.layout_to_device(layout, dev)
+        H, R, C = lay.shape
+        ws, ws_bytes = _lib.workspace(lay, dev)
+        cap = 2 * H * R + 4 * int((layout != 0).sum())
+        lut = torch.empty((max(cap, 1),), dtype=torch.int32, device=dev)
+        n = ctypes.c_int64(0)
+        maxlut = ctypes.c_int(0)
+        rc = lib.bsp_softmax_lut_build(_lib.ptr(lay), H, R, C, _lib.ptr(lut), cap, _lib.ptr(ws), ws_bytes, ctypes.byref(n),
+                                       ctypes.byref(maxlut), _lib.stream_ptr(dev))
+        _lib.check(rc, 'bsp_softmax_lut_build')
+        return lut[:n.value], int(maxlut.value)
+
+    @staticmethod
+    def _check_rows(maxlut, block):
+        if maxlut * block >= 32768:                        # softmax.py:225-227
+            raise NotImplementedError('Reductions larger than 32768 elements are not yet implemented')
+
+    @staticmethod
+    def _strided16(t, what):
+        """Masks are read with vector loads: unit inner stride, 16-byte aligned rows."""
+        v = 4 if t.dtype == torch.float32 else 8
+        if t.stride(-1) != 1 and t.size(-1) != 1:
+            t = t.contiguous()
+        if t.data_ptr() % 16 != 0 or any(s % v for s in t.stride()[:-1]):
+            t = t.contiguous()
+            if t.data_ptr() % 16 != 0:
+                t = t.clone()
+        return t
+
+    @staticmethod
+    def forward(ctx, x, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode,
+                spdims, block, lut, maxlut, bench, time):
+        _lib.require_gpu_tensor(x, 'softmax input')
+        if x.dtype not in _lib.DTYPES:
+            raise ValueError('softmax input must be float16, bfloat16 or float32')
+        if not x.is_contiguous():
+            raise ValueError('softmax works in place on a contiguous [Z, nnz, block, block] tensor')
+        _sparse_softmax._check_rows(maxlut, block)
+        null = ctypes.c_void_p(0)
+        rpe_args = (null, 0, 0, 0)
+        if rpe is not None:                                # element (z, h, r, c), softmax.py:50-55, 265
+            while rpe.dim() < 4:
+                rpe = rpe.unsqueeze(0)
+            rpe = _sparse_softmax._strided16(rpe.expand(x.size(0), spdims[0], rpe.size(2), rpe.size(3)), 'rpe')
+            rpe_args = (_lib.ptr(rpe), rpe.stride(0), rpe.stride(1), rpe.stride(2))
+        kpm_args = (null, 0)
+        if key_padding_mask is not None:                   # element (z, c), softmax.py:60-62, 274
+            key_padding_mask = _sparse_softmax._strided16(key_padding_mask, 'key_padding_mask')
+            kpm_args = (_lib.ptr(key_padding_mask), key_padding_mask.stride(0) if key_padding_mask.size(0) > 1 else 0)
+        attn_args = (null, 0)
+        if attn_mask is not None:                          # element (r, c), softmax.py:67-70, 283
+            attn_mask = _sparse_softmax._strided16(attn_mask, 'attn_mask')
+            attn_args = (_lib.ptr(attn_mask), attn_mask.stride(0))
+        timer = _Timer(bench, x.device)
+        rc = _lib.load().bsp_softmax_fwd(_lib.DTYPES[x.dtype], _lib.ptr(x), float(scale), _lib.ptr(lut), maxlut,
+                                         rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3],
+                                         kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
+                                         attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'),
+                                         x.size(0), spdims[0], spdims[1], block, x.stride(0), _lib.stream_ptr(x.device))
+        _lib.check(rc, 'bsp_softmax_fwd')
+        time[0] = timer.done()
+        ctx.mark_dirty(x)
+        ctx.save_for_backward(x, lut)
+        ctx.spdims, ctx.block, ctx.maxlut, ctx.scale = spdims, block, maxlut, scale
+        return x
+
+    @staticmethod
+    def backward(ctx, dx):
+        x, lut = ctx.saved_tensors
+        dx = dx.contiguous()
+        if dx.data_ptr() % 16 != 0:
+            dx = dx.clone()
+        rc = _lib.load().bsp_softmax_bwd(_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(dx), float(ctx.scale), _lib.ptr(lut),
+                                         ctx.maxlut, x.size(0), ctx.spdims[0], ctx.spdims[1], ctx.block, x.stride(0),
+                                         dx.stride(0), _lib.stream_ptr(x.device))
+        _lib.check(rc, 'bsp_softmax_bwd')
+        return (dx,) + (None,) * 12
+
+
+class Softmax:
+    """softmax over each row of a block-sparse matrix, restricted to the row's nonzero blocks."""
+
+    sparse_softmax = _sparse_softmax.apply
+
+    def make_lut(self, device):
+        key = (device,)
+        if key not in self.lut_cache:
+            self.lut_cache[key] = _sparse_softmax.make_lut(self.layout, self.block, device)
+        return self.lut_cache[key]
+
+    def __init__(self, layout, block, bench=False):
+        if block not in (16, 32, 64, 128):
+            raise ValueError('block must be 16, 32, 64 or 128')
+        self.spdims = layout.shape
+        self.layout = layout
+        self.block = block
+        self.bench = bench
+        self.lut_cache = dict()
+        self.time_y = None
+
+    def __call__(self, x, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
+                 key_padding_mask_mode='add', attn_mask_mode='add'):
+        time_y = [None]
+        if rpe is not None and rpe.dtype != x.dtype:
+            raise ValueError('relative position embedding must be %s' % x.dtype)
+        if attn_mask is not None and attn_mask.dtype != x.dtype:
+            raise ValueError('Attention mask must be %s' % x.dtype)
+        if key_padding_mask is not None and key_padding_mask.dtype != x.dtype:
+            raise ValueError('Key padding mask must be %s' % x.dtype)
+        _lib.require_gpu_tensor(x, 'softmax input')
+        lut, maxlut = self.make_lut(x.device)
+        x = Softmax.sparse_softmax(x, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode,
+                                   self.spdims, self.block, lut, maxlut, self.bench, time_y)
+        self.time_y = time_y[0]
+        return x
