@@ -1,10 +1,16 @@
 // C-ABI entry points of the matmul launchers: argument validation and dispatch.  (The table builders and
 // the softmax entry points live next to their kernels in lut.hip / softmax.hip.)
 #include "matmul_generic.h"
+#include <cstdlib>
 
 using namespace bsp;
 
 namespace {
+// BSP_GENERIC_ONLY=1 in the environment routes every launch to the general kernels (used to test both paths).
+bool generic_only() {
+  const char *e = std::getenv("BSP_GENERIC_ONLY");
+  return e && e[0] == '1';
+}
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool block_ok(int block) { return block == 16 || block == 32 || block == 64 || block == 128; }
 int elems16(int dtype) { return dtype == BSP_F32 ? 4 : 8; }   // elements per 16 bytes
@@ -44,7 +50,9 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);
-  int rc;
+  int rc = generic_only() ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
+  if (rc < 0) return rc;
+  if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
   switch (dtype) {
     case BSP_F16: rc = sdd_generic_f16(g, block, pack, a_kc, b_kc, st); break;
     case BSP_BF16: rc = sdd_generic_bf16(g, block, pack, a_kc, b_kc, st); break;
@@ -58,7 +66,9 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
 
 static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, void *stream) {
   hipStream_t st = as_stream(stream);
-  int rc;
+  int rc = generic_only() ? 0 : xsd_fast64(dtype, g, block, sp_trans, dn_kc, out_nc, st);
+  if (rc < 0) return rc;
+  if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
   switch (dtype) {
     case BSP_F16: rc = xsd_generic_f16(g, block, sp_trans, dn_kc, out_nc, st); break;
     case BSP_BF16: rc = xsd_generic_bf16(g, block, sp_trans, dn_kc, out_nc, st); break;

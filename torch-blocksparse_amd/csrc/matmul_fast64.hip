@@ -1,0 +1,255 @@
+// Bandwidth-oriented kernels for the attention shapes: block 64, fp16 / bf16, dense operands with a unit stride
+// along the head dimension.  At head_dim 64 every product of the sdd -> softmax -> dsd chain moves ~400 MB for
+// 17 GFLOP (43 flop/byte), i.e. it is bound by HBM, not by the matrix cores; these kernels are organised
+// around keeping many 16-byte loads in flight and touching every byte once.
+//
+//   k_sdd64_nt : C_blk = A[i-rows, :K] . B[j-rows, :K]^T.  One wavefront per output block.  Both operands
+//                have the reduction dimension contiguous, which is exactly the MFMA operand layout (a lane
+//                owns one row and 8 consecutive reduction indices), so they go from global memory straight
+//                into the operand registers: no LDS, no barrier.
+//   k_xsd64    : out[64 rows of one table segment, 64 columns] = sum over the segment's blocks
+//                S_t . D[pos_t : pos_t + 64, n0 : n0 + 64].  D is stored with the reduction dimension strided,
+//                and so is S when it is read transposed (the dV / dK products); those tiles are staged in LDS
+//                as they lie in memory and read back with the transposing LDS load of gfx950
+//                (ds_read_b64_tr_b16), which hands each lane 4 reduction-consecutive values of its column.
+//                Four wavefronts per workgroup, each owning 16 output rows; global loads run four blocks
+//                ahead of the MFMAs in a register ring.
+#include "matmul_generic.h"
+
+namespace bsp {
+namespace {
+
+template <typename T> struct Mma32;   // 32x32x16: lane l supplies row l % 32, reduction indices 8 * (l / 32) + j
+template <> struct Mma32<f16> {
+  typedef f16x8 frag_t;
+  static __device__ __forceinline__ f32x16 run(frag_t a, frag_t b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mma32<bf16> {
+  typedef bf16x8 frag_t;
+  static __device__ __forceinline__ f32x16 run(frag_t a, frag_t b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+
+template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  union { T h[2]; uint32_t u; } p;
+  p.h[0] = from_float<T>(lo);
+  p.h[1] = from_float<T>(hi);
+  return p.u;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// sdd, block 64, A and B both with the reduction dimension contiguous ("NT"), K a multiple of 64
+// ---------------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) k_sdd64_nt(SddArgs g) {
+  typedef Mma32<T> M;
+  typedef typename M::frag_t frag_t;
+  const int64_t n_items = g.n_groups * g.Z;
+  const int64_t n_wg = (n_items + 3) >> 2;
+  const int64_t item = xcd_remap(blockIdx.x, n_wg) * 4 + (threadIdx.x >> 6);
+  if (item >= n_items) return;
+  const int lane = threadIdx.x & 63;
+  const int z = (int)(item / g.n_groups);
+  const int64_t grp = item % g.n_groups;
+  if (g.valid && !g.valid[grp]) return;
+  const int32_t *e = g.lut + grp * 4;
+  const int h = e[0], bi = e[1], bj = e[2];
+  const int64_t bk = e[3];
+  // lane's operand rows: r and r + 32 of the block-row (A) / block-column (B); its reduction offset inside a step
+  const int r = lane & 31, kq = (lane >> 5) * 8;
+  const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh + ((int64_t)bi * 64 + r) * g.lda + kq;
+  const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh + ((int64_t)bj * 64 + r) * g.ldb + kq;
+  const int64_t a32 = 32 * g.lda, b32 = 32 * g.ldb;
+  f32x16 acc[2][2];   // [tn][tm]: rows n of the 32x32 result come from B, columns m from A
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+#pragma unroll
+    for (int j = 0; j < 2; j++)
+#pragma unroll
+      for (int v = 0; v < 16; v++) acc[i][j][v] = 0.f;
+  for (int k0 = 0; k0 < g.K; k0 += 64) {
+    frag_t fa[2][4], fb[2][4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+      fa[0][s] = *reinterpret_cast<const frag_t *>(pa + k0 + 16 * s);
+      fa[1][s] = *reinterpret_cast<const frag_t *>(pa + a32 + k0 + 16 * s);
+      fb[0][s] = *reinterpret_cast<const frag_t *>(pb + k0 + 16 * s);
+      fb[1][s] = *reinterpret_cast<const frag_t *>(pb + b32 + k0 + 16 * s);
+    }
+#pragma unroll
+    for (int s = 0; s < 4; s++)
+#pragma unroll
+      for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+        for (int tm = 0; tm < 2; tm++) acc[tn][tm] = M::run(fb[tn][s], fa[tm][s], acc[tn][tm]);
+  }
+  // Result element v = 4*gq + e of tile (tn, tm) is C[m = 32*tm + r][n = 32*tn + 8*gq + 4*(lane/32) + e].
+  // Exchanging the upper half-wave's values of group gq = 2a with the lower half-wave's of gq = 2a+1 leaves every
+  // lane with 8 consecutive n: one 16-byte store.
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz + bk * 4096 + (lane >> 5) * 8;
+#pragma unroll
+  for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+    for (int tm = 0; tm < 2; tm++)
+#pragma unroll
+      for (int a = 0; a < 2; a++) {
+        const f32x16 &c = acc[tn][tm];
+        uint32_t p0 = pack2<T>(c[8 * a + 0], c[8 * a + 1]), p1 = pack2<T>(c[8 * a + 2], c[8 * a + 3]);
+        uint32_t q0 = pack2<T>(c[8 * a + 4], c[8 * a + 5]), q1 = pack2<T>(c[8 * a + 6], c[8 * a + 7]);
+        auto x = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
+        auto y = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
+        u32x4 out = {x[0], y[0], x[1], y[1]};
+        *reinterpret_cast<u32x4 *>(pc + (32 * tm + r) * 64 + 32 * tn + 16 * a) = out;
+      }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// xsd, block 64, dense operand and output with the free dimension contiguous
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kLdsRow = 72;     // elements per LDS tile row: 64 + 8 (144 bytes, keeps 16-byte alignment)
+constexpr int kRing = 4;        // blocks in flight per workgroup
+
+template <typename T> __device__ __forceinline__ typename Mma16<T>::frag_t tr_frag(const T *p_lo, const T *p_hi) {
+  // two transposing reads: reduction indices 0..3 and 4..7 of this lane's column
+  typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+  s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p_lo);
+  s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p_hi);
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+  return __builtin_bit_cast(typename Mma16<T>::frag_t, v);
+}
+
+template <typename T, bool SP_TRANS>
+__global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int TILE = 64 * kLdsRow;
+  __shared__ __attribute__((aligned(16))) T Ys[2][TILE];
+  __shared__ __attribute__((aligned(16))) T Xs[SP_TRANS ? 2 : 1][SP_TRANS ? TILE : 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t per_z = (int64_t)g.width * g.n_tiles;
+  const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
+  const int z = (int)(w / per_z);
+  const int seg = (int)((w % per_z) / g.n_tiles);
+  const int n0 = (int)(w % g.n_tiles) * 64;
+  const int32_t *hd = g.lut + 6 * (int64_t)seg;
+  const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];
+  const int nblk = seglen >> 6;
+  if (nblk == 0 && seg > 0 && hd[-4] == column && hd[-3] == depth) return;   // see k_xsd: empty twin of a real segment
+  const int32_t *plan = g.plan + 2 * (int64_t)((offset - 6 * g.width) / g.div2);
+  const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
+  const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
+  const int64_t ldd = g.ldd;
+
+  // cooperative tile loads: thread handles 16-byte chunks (row tid/8, column-chunk tid%8) and the same 32 rows below
+  const int ck = tid >> 3, cc = (tid & 7) * 8;
+  // direct X operand (not transposed): lane owns row 16*wave + lane%16 of the block, reduction offset 8*(lane/16)
+  const int xr = wave * 16 + (lane & 15), xq = (lane >> 4) * 8;
+
+  struct Stage { u32x4 y[2]; u32x4 x[2]; };
+  Stage ring[kRing];
+  auto issue = [&](Stage &st, int b) {
+    const int64_t pos = plan[2 * b];
+    const T *blk = sp + (int64_t)plan[2 * b + 1] * 4096;
+    const T *py = dn + (pos + ck) * ldd + cc;
+    st.y[0] = *reinterpret_cast<const u32x4 *>(py);
+    st.y[1] = *reinterpret_cast<const u32x4 *>(py + 32 * ldd);
+    if constexpr (SP_TRANS) {
+      st.x[0] = *reinterpret_cast<const u32x4 *>(blk + ck * 64 + cc);
+      st.x[1] = *reinterpret_cast<const u32x4 *>(blk + (ck + 32) * 64 + cc);
+    } else {
+      st.x[0] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + xq);
+      st.x[1] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + 32 + xq);
+    }
+  };
+
+  f32x4 acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+#pragma unroll
+  for (int u = 0; u < kRing; u++)
+    if (u < nblk) issue(ring[u], u);
+
+  // transposing-read addresses: within a 16-lane group, lane t points at row (t / 4), 4-element piece (t % 4);
+  // the group then receives, per lane i, the 4 rows' values of column i.
+  const int tr_row = (lane >> 4) * 8 + ((lane & 15) >> 2), tr_col = (lane & 3) * 4;
+
+  for (int b0 = 0; b0 < nblk; b0 += kRing) {
+#pragma unroll
+    for (int u = 0; u < kRing; u++) {
+      const int b = b0 + u;
+      if (b < nblk) {
+        const int buf = b & 1;
+        Stage &st = ring[u];
+        *reinterpret_cast<u32x4 *>(&Ys[buf][ck * kLdsRow + cc]) = st.y[0];
+        *reinterpret_cast<u32x4 *>(&Ys[buf][(ck + 32) * kLdsRow + cc]) = st.y[1];
+        frag_t xf[2];
+        if constexpr (SP_TRANS) {
+          *reinterpret_cast<u32x4 *>(&Xs[buf][ck * kLdsRow + cc]) = st.x[0];
+          *reinterpret_cast<u32x4 *>(&Xs[buf][(ck + 32) * kLdsRow + cc]) = st.x[1];
+        } else {
+          xf[0] = __builtin_bit_cast(frag_t, st.x[0]);
+          xf[1] = __builtin_bit_cast(frag_t, st.x[1]);
+        }
+        if (b + kRing < nblk) issue(st, b + kRing);
+        __syncthreads();
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const T *yrow = &Ys[buf][(32 * s + tr_row) * kLdsRow + tr_col];
+          if constexpr (SP_TRANS) {
+            const T *xrow = &Xs[buf][(32 * s + tr_row) * kLdsRow + 16 * wave + tr_col];
+            xf[s] = tr_frag<T>(xrow, xrow + 4 * kLdsRow);
+          }
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            frag_t yf = tr_frag<T>(yrow + 16 * j, yrow + 16 * j + 4 * kLdsRow);
+            acc[j] = M::run(yf, xf[s], acc[j]);   // result rows = n (16*j + 4*(lane/16) + e), column = m (lane%16)
+          }
+        }
+      }
+    }
+  }
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + ((int64_t)column * 64 + wave * 16 + (lane & 15)) * g.ldo +
+          n0 + 4 * (lane >> 4);
+#pragma unroll
+  for (int j = 0; j < 4; j++) store4<T>(po + 16 * j, acc[j]);
+}
+
+bool fast_ok_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc) {
+  return block == 64 && pack == 1 && a_kc && b_kc && g.K % 64 == 0;
+}
+bool fast_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
+  return block == 64 && !dn_kc && out_nc && g.NF % 64 == 0;
+}
+
+template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
+  const int64_t n_wg = (g.n_groups * g.Z + 3) / 4;
+  if (n_wg <= 0) return BSP_OK;
+  if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(k_sdd64_nt<T>, dim3((unsigned)n_wg), dim3(256), 0, st, g);
+  return BSP_OK;
+}
+template <typename T> int xsd_fast_t(const XsdArgs &g, bool sp_trans, hipStream_t st) {
+  const int64_t n_wg = (int64_t)g.width * g.n_tiles * g.Z;
+  if (n_wg <= 0) return BSP_OK;
+  if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (sp_trans) hipLaunchKernelGGL((k_xsd64<T, true>), dim3((unsigned)n_wg), dim3(256), 0, st, g);
+  else hipLaunchKernelGGL((k_xsd64<T, false>), dim3((unsigned)n_wg), dim3(256), 0, st, g);
+  return BSP_OK;
+}
+
+}  // namespace
+
+// Returns 1 if a specialised kernel took the launch, 0 if the caller should use the general kernel, < 0 on error.
+int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st) {
+  if (dtype == BSP_F32 || !fast_ok_sdd(g, block, pack, a_kc, b_kc)) return 0;
+  int rc = dtype == BSP_F16 ? sdd_fast_t<f16>(g, st) : sdd_fast_t<bf16>(g, st);
+  return rc == BSP_OK ? 1 : rc;
+}
+int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+  if (dtype == BSP_F32 || !fast_ok_xsd(g, block, dn_kc, out_nc)) return 0;
+  int rc = dtype == BSP_F16 ? xsd_fast_t<f16>(g, sp_trans, st) : xsd_fast_t<bf16>(g, sp_trans, st);
+  return rc == BSP_OK ? 1 : rc;
+}
+
+}  // namespace bsp

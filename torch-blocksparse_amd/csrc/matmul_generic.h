@@ -385,4 +385,9 @@ int xsd_generic_f16(const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool
 int xsd_generic_bf16(const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
 int xsd_generic_f32(const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
 
+
+// specialised block-64 16-bit kernels (matmul_fast64.hip): 1 = launched, 0 = not applicable, < 0 = error
+int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st);
+int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
+
 }  // namespace bsp
