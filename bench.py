@@ -26,6 +26,16 @@ for p in (ROOT, os.path.join(ROOT, 'torch-blocksparse_amd')):
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 
+# HBM bytes per launch at batch 8, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what
+# the same counter reads for the calibration copy of known size (profiles/traffic_attention_seq4096.txt).  None = not
+# measured for this build of the kernel.
+TRAFFIC_BYTES = {
+    'sdd_fwd  q.k^T': 134815882 + 268435456, 'sdd_bwd  do.v^T': 134815882 + 268435456,
+    'dsd_fwd  p.v': 336633312 + 67108864, 'dsd_bwd  ds.k': 336633312 + 67108864,
+    'dsd_bwd  p^T.do': 402584314 + 67108864, 'dds_bwd  (q^T.ds)^T': 402584314 + 67108864,
+    'softmax_fwd': 269257126 + 268435456, 'softmax_bwd': 537486370 + 268435456,
+}
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -84,52 +94,79 @@ def main():
     dense_bytes = B * H * L * dh * es
     mm_bytes = x_bytes + 2 * dense_bytes                    # one sparse tensor + two dense tensors, each touched once
 
-    # per-launch timing with HIP events on the launch stream
+    # Per-launch timing with HIP events on the launch stream, the eight launches of a step issued back to back in
+    # step order (so each kernel sees the cache state its predecessor leaves), K steps, one synchronisation at the end.
     luts = {m: m.make_lut(dtype, dev) for m in (sdd, dsd)}
     sm_lut, sm_maxlut = sm.make_lut(dev)
     t = [None]
-    with torch.no_grad():
-        w = sdd(q, k)
-        p = sm(w.clone(), scale=scale, key_padding_mask=kpm)
-        dp = torch.randn_like(p)
     fn = _sparse_matmul.fn
     sl, dl = luts[sdd], luts[dsd]
     spd = lay.shape
-    launches = {
-        # forward
-        'sdd_fwd  q.k^T': (lambda: fn['sdd'](q, k, False, True, False, spd, block, sl[0], sl[1], sl[2], sl[3], False, t), flops_mm, mm_bytes),
-        'softmax_fwd': (lambda: tb.Softmax.sparse_softmax(w, scale, None, kpm, None, 'add', 'add', spd, block, sm_lut, sm_maxlut, False, t), 0.0, 2 * x_bytes + kpm.numel() * es),
-        'dsd_fwd  p.v': (lambda: fn['dsd'](p, v, False, False, False, spd, block, dl[0], dl[1], dl[2], dl[3], False, t), flops_mm, mm_bytes),
-        # backward of dsd: dp = sdd(do, v^T), dv = dsd(p^T, do)
-        'sdd_bwd  do.v^T': (lambda: fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t), flops_mm, mm_bytes),
-        'dsd_bwd  p^T.do': (lambda: fn['dsd'](p, do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t), flops_mm, mm_bytes),
-        'softmax_bwd': (lambda: _bwd_softmax(tb, p, dp, scale, sm_lut, sm_maxlut, spd, block), 0.0, 3 * x_bytes),
-        # backward of sdd: dq = dsd(ds, k), dk = dds(q^T, ds) written transposed
-        'dsd_bwd  ds.k': (lambda: fn['dsd'](dp, k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t), flops_mm, mm_bytes),
-        'dds_bwd  (q^T.ds)^T': (lambda: fn['dds'](q, dp, True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t), flops_mm, mm_bytes),
-    }
-    kernels = {}
+    st = {}
+
+    def k_sdd_fwd():
+        st['w'] = fn['sdd'](q, k, False, True, False, spd, block, sl[0], sl[1], sl[2], sl[3], False, t)
+
+    def k_softmax_fwd():
+        st['p'] = tb.Softmax.sparse_softmax(st['w'], scale, None, kpm, None, 'add', 'add', spd, block, sm_lut, sm_maxlut, False, t)
+
+    def k_dsd_fwd():
+        st['o'] = fn['dsd'](st['p'], v, False, False, False, spd, block, dl[0], dl[1], dl[2], dl[3], False, t)
+
+    def k_sdd_bwd():     # dp = do . v^T restricted to the layout
+        st['dp'] = fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t)
+
+    def k_dsd_bwd_t():   # dv = p^T . do
+        st['dv'] = fn['dsd'](st['p'], do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t)
+
+    def k_softmax_bwd():
+        _bwd_softmax(tb, st['p'], st['dp'], scale, sm_lut, sm_maxlut, spd, block)
+
+    def k_dsd_bwd():     # dq = ds . k
+        st['dq'] = fn['dsd'](st['dp'], k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t)
+
+    def k_dds_bwd():     # dk = (q^T . ds)^T
+        st['dk'] = fn['dds'](q, st['dp'], True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t)
+
+    def k_copy():        # plain copy of |x| bytes: the known-size kernel the traffic counters are calibrated on
+        st['copy'] = st['dp'].clone()
+
+    launches = [
+        ('sdd_fwd  q.k^T', k_sdd_fwd, flops_mm, mm_bytes),
+        ('softmax_fwd', k_softmax_fwd, 0.0, 2 * x_bytes + kpm.numel() * es),
+        ('dsd_fwd  p.v', k_dsd_fwd, flops_mm, mm_bytes),
+        ('sdd_bwd  do.v^T', k_sdd_bwd, flops_mm, mm_bytes),
+        ('dsd_bwd  p^T.do', k_dsd_bwd_t, flops_mm, mm_bytes),
+        ('softmax_bwd', k_softmax_bwd, 0.0, 3 * x_bytes),
+        ('dsd_bwd  ds.k', k_dsd_bwd, flops_mm, mm_bytes),
+        ('dds_bwd  (q^T.ds)^T', k_dds_bwd, flops_mm, mm_bytes),
+        ('calibration_copy', k_copy, 0.0, 2 * x_bytes),
+    ]
+    reps = max(args.steps, 10)
+    events = {name: [] for name, _, _, _ in launches}
     with torch.no_grad():
-        for name, (f, flops, nbytes) in launches.items():
-            for _ in range(3):
+        for it in range(3 + reps):
+            for name, f, _, _ in launches:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
                 f()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            reps = max(args.steps, 10)
-            e0.record()
-            for _ in range(reps):
-                f()
-            e1.record()
-            e1.synchronize()
-            ms = e0.elapsed_time(e1) / reps
-            ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
-                   'bytes': nbytes}
-            if flops:
-                ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
-                ent['mfma_frac'] = round(flops / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)
-            kernels[name] = ent
+                e1.record()
+                if it >= 3:
+                    events[name].append((e0, e1))
+    torch.cuda.synchronize()
+    kernels = {}
+    for name, _, flops, nbytes in launches:
+        ms = sum(a.elapsed_time(b) for a, b in events[name]) / len(events[name])
+        ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
+               'bytes': nbytes, 'traffic': TRAFFIC_BYTES.get(name) if B == 8 else None}
+        if flops:
+            ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
+            ent['mfma_frac'] = round(flops / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)
+        kernels[name] = ent
+    calib = kernels.pop('calibration_copy')
     dom = max(kernels, key=lambda n: kernels[n]['ms'])
     roofline = {'kernel': dom, 'bound': 'hbm', 'achieved': kernels[dom]['GB/s'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': kernels[dom]['hbm_frac'], 'traffic': None}
+                'frac': kernels[dom]['hbm_frac'], 'traffic': kernels[dom]['traffic']}
 
     out = {
         'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk64',
@@ -139,8 +176,9 @@ def main():
         'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block 64, fixed '
                                'layout (local 4 blocks + 1 global per 16, causal), scale 1/8, additive key-padding mask' % B,
                    'nnz_blocks': nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
+        'matmul_TFLOP/s_kernel_time_only': round(6 * flops_mm / sum(e['ms'] for n, e in kernels.items() if 'softmax' not in n) * 1e-9, 2),
         'softmax_GB/s': {'fwd': kernels['softmax_fwd']['GB/s'], 'bwd': kernels['softmax_bwd']['GB/s']},
-        'roofline': roofline, 'kernels': kernels,
+        'roofline': roofline, 'kernels': kernels, 'calibration_copy': calib,
     }
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, L)
@@ -157,22 +195,25 @@ def _bwd_softmax(tb, y, dy, scale, lut, maxlut, spdims, block):
 
 def cpu_baseline(lay, block, dh, scale, L):
     """The reference's CPU path = its test oracle: dense fp32 matmuls + layout mask + dense softmax, forward and
-    backward (oracle/dense_oracle.py).  Timed on a slice of the workload (1 sequence, all 16 heads)."""
+    backward (oracle/dense_oracle.py).  Timed on the same workload, one sequence at a time (the dense score tensors
+    of one sequence are ~1 GB each), repeating the sequence-sized pass for about 12 s."""
     import torch
     from oracle import dense_oracle as D
     torch.manual_seed(0)
-    Bs, H = 1, lay.shape[0]
-    q, k, v, do = [torch.randn(Bs, H, L, dh) for _ in range(4)]
-    kpm = torch.zeros(Bs, L)
+    H = lay.shape[0]
+    kpm = torch.zeros(1, L)
     kpm[0, L - L // 8:] = float('-inf')
+    q, k, v, do = [torch.randn(1, H, L, dh) for _ in range(4)]
     D.attention(q[:, :1], k[:, :1], v[:, :1], lay[:1], block, scale, key_padding_mask=kpm, do=do[:, :1])   # warm-up
-    t0 = time.perf_counter()
-    D.attention(q, k, v, lay, block, scale, key_padding_mask=kpm, do=do)
+    done, t0 = 0, time.perf_counter()
+    while done < 24 and time.perf_counter() - t0 < 12.0:
+        D.attention(q, k, v, lay, block, scale, key_padding_mask=kpm, do=do)
+        done += 1
     dt = time.perf_counter() - t0
-    flops = 6 * 2.0 * Bs * dh * int(lay.sum()) * block * block
+    flops = 6 * 2.0 * done * dh * int(lay.sum()) * block * block
     return {'value': round(flops / dt * 1e-12, 5), 'unit': 'TFLOP/s', 'cores': torch.get_num_threads(), 'kind': 'port',
-            'sample': 'same chain fwd+bwd on 1 of the 8 sequences (16 heads, seq 4096), fp32 dense matmul + mask + softmax, '
-                      '%.1f s; throughput counts only the nonzero-block FLOPs, like the GPU figure' % dt}
+            'sample': 'same chain fwd+bwd, %d sequence-sized passes (1 sequence = 16 heads x seq 4096; the workload has 8), fp32 dense matmul + mask + softmax, '
+                      '%.1f s; throughput counts only the nonzero-block FLOPs, like the GPU figure' % (done, dt)}
 
 
 if __name__ == '__main__':

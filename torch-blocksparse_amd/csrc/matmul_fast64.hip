@@ -29,6 +29,9 @@ template <> struct Mma32<bf16> {
   static __device__ __forceinline__ f32x16 run(frag_t a, frag_t b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
 };
 
+constexpr int kLdsRow = 72;     // elements per LDS tile row: 64 + 8 (144 bytes, keeps 16-byte alignment)
+constexpr int kRing = 4;        // blocks in flight per workgroup
+
 template <typename T> __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   union { T h[2]; uint32_t u; } p;
   p.h[0] = from_float<T>(lo);
@@ -84,8 +87,10 @@ __global__ void __launch_bounds__(256) k_sdd64_nt(SddArgs g) {
   }
   // Result element v = 4*gq + e of tile (tn, tm) is C[m = 32*tm + r][n = 32*tn + 8*gq + 4*(lane/32) + e].
   // Exchanging the upper half-wave's values of group gq = 2a with the lower half-wave's of gq = 2a+1 leaves every
-  // lane with 8 consecutive n: one 16-byte store.
-  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz + bk * 4096 + (lane >> 5) * 8;
+  // lane with 8 consecutive n (16 bytes).  The tile then goes through a wave-private LDS buffer so that each store
+  // instruction writes 8 whole rows of the block: 1 KiB of consecutive addresses instead of 32-byte pieces.
+  __shared__ __attribute__((aligned(16))) T Cs[4][64 * kLdsRow];
+  T *cs = Cs[threadIdx.x >> 6];
 #pragma unroll
   for (int tn = 0; tn < 2; tn++)
 #pragma unroll
@@ -98,16 +103,19 @@ __global__ void __launch_bounds__(256) k_sdd64_nt(SddArgs g) {
         auto x = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
         auto y = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
         u32x4 out = {x[0], y[0], x[1], y[1]};
-        *reinterpret_cast<u32x4 *>(pc + (32 * tm + r) * 64 + 32 * tn + 16 * a) = out;
+        *reinterpret_cast<u32x4 *>(cs + (32 * tm + r) * kLdsRow + 32 * tn + 16 * a + (lane >> 5) * 8) = out;
       }
+  __builtin_amdgcn_wave_barrier();   // LDS operations of one wavefront complete in order; this only pins the code order
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz + bk * 4096 + lane * 8;
+  const T *rs = cs + (lane >> 3) * kLdsRow + (lane & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 8; i++)
+    *reinterpret_cast<u32x4 *>(pc + i * 512) = *reinterpret_cast<const u32x4 *>(rs + i * 8 * kLdsRow);
 }
 
 // ---------------------------------------------------------------------------------------------------------
 // xsd, block 64, dense operand and output with the free dimension contiguous
 // ---------------------------------------------------------------------------------------------------------
-constexpr int kLdsRow = 72;     // elements per LDS tile row: 64 + 8 (144 bytes, keeps 16-byte alignment)
-constexpr int kRing = 4;        // blocks in flight per workgroup
-
 template <typename T> __device__ __forceinline__ typename Mma16<T>::frag_t tr_frag(const T *p_lo, const T *p_hi) {
   // two transposing reads: reduction indices 0..3 and 4..7 of this lane's column
   typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
@@ -209,10 +217,24 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
       }
     }
   }
-  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + ((int64_t)column * 64 + wave * 16 + (lane & 15)) * g.ldo +
-          n0 + 4 * (lane >> 4);
+  // Epilogue through LDS (each wavefront its own 16 rows of the first tile buffer, free after the last barrier
+  // below): lanes then store 16 bytes each, 8 lanes per output row, whole 128-byte lines.
+  __syncthreads();
+  T *cs = &Ys[0][(wave * 16) * kLdsRow];
 #pragma unroll
-  for (int j = 0; j < 4; j++) store4<T>(po + 16 * j, acc[j]);
+  for (int j = 0; j < 4; j++) {
+    union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk.e[e] = from_float<T>(acc[j][e]);
+    *reinterpret_cast<u32x2 *>(cs + (lane & 15) * kLdsRow + 16 * j + 4 * (lane >> 4)) = pk.raw;
+  }
+  __builtin_amdgcn_wave_barrier();
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + ((int64_t)column * 64 + wave * 16 + (lane >> 3)) * g.ldo +
+          n0 + (lane & 7) * 8;
+  const T *rs = cs + (lane >> 3) * kLdsRow + (lane & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    *reinterpret_cast<u32x4 *>(po + (int64_t)i * 8 * g.ldo) = *reinterpret_cast<const u32x4 *>(rs + i * 8 * kLdsRow);
 }
 
 bool fast_ok_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc) {

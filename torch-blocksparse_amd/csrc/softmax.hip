@@ -1,18 +1,18 @@
 // Block-sparse softmax, forward and backward, for gfx950.
 //
 // Replaces the reference's softmax_fwd / softmax_bwd (softmax.py:7-138, 144-194).  The reference runs one
-// program per matrix row; here one 64-lane wavefront owns 16 consecutive rows of one block-row: 4 lanes
-// share a row, every lane keeps BLOCK/4 columns of each of the row's nonzero blocks in registers, and the
-// row maximum / sum are two xor-shuffles.  Each block is read and written exactly once with 16-byte
-// accesses, so the kernel moves the algorithmic 2 (forward) or 3 (backward) passes over x and nothing more.
+// program per matrix row; here a few lanes share a row, each owning one 16-byte chunk of every nonzero block of
+// the row (block 64, fp16: 8 lanes per row, a 64-lane wavefront covers 8 consecutive rows, so every load or
+// store instruction of a wavefront touches 1 KiB of consecutive addresses).  The row's values stay in registers
+// between the passes; the row maximum / sum are a few xor-shuffles.  Each block is read and written exactly once,
+// so the kernel moves the algorithmic 2 (forward) or 3 (backward) passes over x and nothing more.  Many small
+// wavefronts rather than few large ones: that is what keeps enough loads in flight to fill the HBM pipe.
 // Rows with more blocks than fit in registers take a streaming variant that re-reads x.
 #include "bsp_common.h"
 
 namespace bsp {
 namespace {
 
-constexpr int kRowsPerWave = 16;
-constexpr int kLanesPerRow = 4;
 constexpr int kWavesPerGroup = 4;
 
 template <typename T, int EV> struct RawVec;
@@ -29,14 +29,25 @@ template <typename T, int EV> struct Pack {
   __device__ __forceinline__ void store(T *p) const { *reinterpret_cast<raw_t *>(p) = raw; }
 };
 
-__device__ __forceinline__ float row_max(float v) {
-  v = fmaxf(v, __shfl_xor(v, 1));
-  v = fmaxf(v, __shfl_xor(v, 2));
+// Geometry: LPR lanes share a row and each owns one chunk of EV consecutive columns of every block (16 bytes,
+// 8 bytes for block 16 in 16-bit types); a wavefront covers RPW = 64 / LPR consecutive rows of one block-row, so a
+// load instruction of the wavefront reads RPW whole rows of a block: consecutive addresses.
+template <typename T, int BLOCK> struct Geo {
+  static constexpr int LPR_ = BLOCK * (int)sizeof(T) / 16;
+  static constexpr int LPR = LPR_ > 64 / BLOCK ? LPR_ : 64 / BLOCK;
+  static constexpr int EV = BLOCK / LPR;
+  static constexpr int RPW = 64 / LPR;
+  static constexpr int G = BLOCK / RPW;   // wavefronts per block-row
+};
+
+template <int LPR> __device__ __forceinline__ float row_max(float v) {
+#pragma unroll
+  for (int d = 1; d < LPR; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
   return v;
 }
-__device__ __forceinline__ float row_sum(float v) {
-  v += __shfl_xor(v, 1);
-  v += __shfl_xor(v, 2);
+template <int LPR> __device__ __forceinline__ float row_sum(float v) {
+#pragma unroll
+  for (int d = 1; d < LPR; d <<= 1) v += __shfl_xor(v, d);
   return v;
 }
 
@@ -53,97 +64,81 @@ struct FwdArgs {
   int Z, H, R; int64_t x_sz; int64_t n_units;
 };
 
-// where does this wavefront work?  unit = ((z * H*R) + block-row) * (BLOCK/16) + 16-row group
-template <int BLOCK> struct Unit {
-  int z, hr, rxm, q;   // batch, head*R + block-row, row inside the block, lane's position inside the row
+// where does this wavefront work?  unit = ((z * H*R) + block-row) * G + row group
+template <typename T, int BLOCK> struct Unit {
+  int z, hr, rxm, col;   // batch, head*R + block-row, row inside the block, lane's first column inside a block
   bool ok;
   __device__ __forceinline__ Unit(int64_t n_units, int HR) {
-    constexpr int G = BLOCK / kRowsPerWave;
+    typedef Geo<T, BLOCK> GE;
     const int64_t n_wg = (n_units + kWavesPerGroup - 1) / kWavesPerGroup;
     const int64_t wg = xcd_remap(blockIdx.x, n_wg);
     const int64_t u = wg * kWavesPerGroup + (threadIdx.x >> 6);
     ok = u < n_units;
     const int lane = threadIdx.x & 63;
-    const int g = (int)(u % G);
-    const int64_t t = u / G;
+    const int g = (int)(u % GE::G);
+    const int64_t t = u / GE::G;
     hr = (int)(t % HR);
     z = (int)(t / HR);
-    rxm = g * kRowsPerWave + lane / kLanesPerRow;
-    q = lane % kLanesPerRow;
+    rxm = g * GE::RPW + lane / GE::LPR;
+    col = (lane % GE::LPR) * GE::EV;
   }
 };
 
-// The lane's columns inside a block: chunk j (of NJ) starts at (j*4 + q)*EV, so that the four lanes of a row
-// cover 4*EV consecutive elements per load instruction.
-template <typename T, int BLOCK> struct Cols {
-  static constexpr int VEC = BLOCK / kLanesPerRow;
-  static constexpr int EV = VEC < (int)(16 / sizeof(T)) ? VEC : (int)(16 / sizeof(T));
-  static constexpr int NJ = VEC / EV;
-  __device__ static __forceinline__ int col(int j, int q) { return (j * kLanesPerRow + q) * EV; }
-};
-
 template <typename T, int BLOCK>
-__device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
-                                           float (&fx)[Cols<T, BLOCK>::VEC]) {
-  typedef Cols<T, BLOCK> CL;
-  const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK;
-  const int64_t grow = (int64_t)brow * BLOCK + u.rxm;   // row in the dense matrix
-  const int64_t gcol = (int64_t)bcol * BLOCK;           // first column of the block in the dense matrix
+__device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
+                                           float (&fx)[Geo<T, BLOCK>::EV]) {
+  constexpr int EV = Geo<T, BLOCK>::EV;
+  const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
+  const int64_t grow = (int64_t)brow * BLOCK + u.rxm;    // row in the dense matrix
+  const int64_t gcol = (int64_t)bcol * BLOCK + u.col;    // lane's first column in the dense matrix
+  Pack<T, EV> px;
+  px.load(x);
 #pragma unroll
-  for (int j = 0; j < CL::NJ; j++) {
-    const int c = CL::col(j, u.q);
-    Pack<T, CL::EV> px;
-    px.load(x + c);
+  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * a.scale;                          // softmax.py:112-116
+  if (a.rpe) {                                                                               // :118-120, address :50-55
+    Pack<T, EV> p;
+    p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
 #pragma unroll
-    for (int e = 0; e < CL::EV; e++) fx[j * CL::EV + e] = to_float(px.e[e]) * a.scale;          // softmax.py:112-116
-    if (a.rpe) {                                                                                // :118-120, address :50-55
-      Pack<T, CL::EV> p;
-      p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol + c);
+    for (int e = 0; e < EV; e++) fx[e] += to_float(p.e[e]);
+  }
+  if (a.kpm) {                                                                               // :122-124, address :60-62
+    Pack<T, EV> p;
+    p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol);
 #pragma unroll
-      for (int e = 0; e < CL::EV; e++) fx[j * CL::EV + e] += to_float(p.e[e]);
+    for (int e = 0; e < EV; e++) {
+      float m = to_float(p.e[e]);
+      if (a.kpm_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                       // :104-106
+      fx[e] += m;
     }
-    if (a.kpm) {                                                                                // :122-124, address :60-62
-      Pack<T, CL::EV> p;
-      p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol + c);
+  }
+  if (a.attn) {                                                                              // :126-128, address :67-70
+    Pack<T, EV> p;
+    p.load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);
 #pragma unroll
-      for (int e = 0; e < CL::EV; e++) {
-        float m = to_float(p.e[e]);
-        if (a.kpm_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                        // :104-106
-        fx[j * CL::EV + e] += m;
-      }
-    }
-    if (a.attn) {                                                                               // :126-128, address :67-70
-      Pack<T, CL::EV> p;
-      p.load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol + c);
-#pragma unroll
-      for (int e = 0; e < CL::EV; e++) {
-        float m = to_float(p.e[e]);
-        if (a.attn_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                       // :108-110
-        fx[j * CL::EV + e] += m;
-      }
+    for (int e = 0; e < EV; e++) {
+      float m = to_float(p.e[e]);
+      if (a.attn_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                      // :108-110
+      fx[e] += m;
     }
   }
 }
 
 template <typename T, int BLOCK>
-__device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<BLOCK> &u, int64_t blockid, const float (&y)[Cols<T, BLOCK>::VEC]) {
-  typedef Cols<T, BLOCK> CL;
-  T *x = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK;
+__device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<T, BLOCK> &u, int64_t blockid, const float (&y)[Geo<T, BLOCK>::EV]) {
+  constexpr int EV = Geo<T, BLOCK>::EV;
+  T *x = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
+  Pack<T, EV> p;
 #pragma unroll
-  for (int j = 0; j < CL::NJ; j++) {
-    Pack<T, CL::EV> p;
-#pragma unroll
-    for (int e = 0; e < CL::EV; e++) p.e[e] = from_float<T>(y[j * CL::EV + e]);
-    p.store(x + CL::col(j, u.q));
-  }
+  for (int e = 0; e < EV; e++) p.e[e] = from_float<T>(y[e]);
+  p.store(x);
 }
 
 // NB = number of blocks of a row kept in registers; NB == 0 selects the streaming variant.
 template <typename T, int BLOCK, int NB>
 __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
-  typedef Cols<T, BLOCK> CL;
+  typedef Geo<T, BLOCK> GE;
   const int HR = a.H * a.R;
-  Unit<BLOCK> u(a.n_units, HR);
+  Unit<T, BLOCK> u(a.n_units, HR);
   if (!u.ok) return;
   const int size = a.lut[2 * u.hr + 0];                 // header (size, offset), softmax.py:30-32
   const int offset = a.lut[2 * u.hr + 1];
@@ -151,7 +146,7 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   if (size <= 0) return;
   const int32_t *core = a.lut + offset;
   if constexpr (NB > 0) {
-    float fx[NB][CL::VEC];
+    float fx[NB][GE::EV];
     int32_t bid[NB];
     float mx = -INFINITY;
 #pragma unroll
@@ -159,47 +154,51 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       if (b < size) {
         bid[b] = core[4 * b + 0];
         fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], bid[b], fx[b]);
-#pragma unroll
-        for (int e = 0; e < CL::VEC; e++) mx = fmaxf(mx, fx[b][e]);
       }
-    mx = row_max(mx);                                   // :130
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[b][e]);
+      }
+    mx = row_max<GE::LPR>(mx);                          // :130
     float sum = 0.f;
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
 #pragma unroll
-        for (int e = 0; e < CL::VEC; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
+        for (int e = 0; e < GE::EV; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
       }
-    sum = row_sum(sum);
+    sum = row_sum<GE::LPR>(sum);
     const float inv = 1.f / sum;
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
 #pragma unroll
-        for (int e = 0; e < CL::VEC; e++) fx[b][e] *= inv;                                            // :137
+        for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
         fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
       }
   } else {
-    float fx[CL::VEC];
+    float fx[GE::EV];
     float mx = -INFINITY;
     for (int b = 0; b < size; b++) {
       fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
 #pragma unroll
-      for (int e = 0; e < CL::VEC; e++) mx = fmaxf(mx, fx[e]);
+      for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[e]);
     }
-    mx = row_max(mx);
+    mx = row_max<GE::LPR>(mx);
     float sum = 0.f;
     for (int b = 0; b < size; b++) {
       fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
 #pragma unroll
-      for (int e = 0; e < CL::VEC; e++) sum += exp_sub<T>(fx[e], mx);
+      for (int e = 0; e < GE::EV; e++) sum += exp_sub<T>(fx[e], mx);
     }
-    sum = row_sum(sum);
+    sum = row_sum<GE::LPR>(sum);
     const float inv = 1.f / sum;
     for (int b = 0; b < size; b++) {
       fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
 #pragma unroll
-      for (int e = 0; e < CL::VEC; e++) fx[e] = exp_sub<T>(fx[e], mx) * inv;
+      for (int e = 0; e < GE::EV; e++) fx[e] = exp_sub<T>(fx[e], mx) * inv;
       fwd_store<T, BLOCK>(a, u, core[4 * b + 0], fx);
     }
   }
@@ -212,19 +211,19 @@ struct BwdArgs {
 
 template <typename T, int BLOCK, int NB>
 __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
-  typedef Cols<T, BLOCK> CL;
-  typedef Pack<T, CL::EV> P;
+  typedef Geo<T, BLOCK> GE;
+  typedef Pack<T, GE::EV> P;
   const int HR = a.H * a.R;
-  Unit<BLOCK> u(a.n_units, HR);
+  Unit<T, BLOCK> u(a.n_units, HR);
   if (!u.ok) return;
   const int size = a.lut[2 * u.hr + 0];
   const int offset = a.lut[2 * u.hr + 1];
   if (size <= 0) return;
   const int32_t *core = a.lut + offset;
-  const T *yb = reinterpret_cast<const T *>(a.y) + (int64_t)u.z * a.y_sz + u.rxm * BLOCK;
-  T *db = reinterpret_cast<T *>(a.dy) + (int64_t)u.z * a.dy_sz + u.rxm * BLOCK;
+  const T *yb = reinterpret_cast<const T *>(a.y) + (int64_t)u.z * a.y_sz + u.rxm * BLOCK + u.col;
+  T *db = reinterpret_cast<T *>(a.dy) + (int64_t)u.z * a.dy_sz + u.rxm * BLOCK + u.col;
   if constexpr (NB > 0) {
-    P py[NB][CL::NJ], pd[NB][CL::NJ];
+    P py[NB], pd[NB];
     int32_t bid[NB];
     float dot = 0.f;
 #pragma unroll
@@ -232,66 +231,51 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
       if (b < size) {
         bid[b] = core[4 * b];
         const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
-#pragma unroll
-        for (int j = 0; j < CL::NJ; j++) {
-          py[b][j].load(yb + o + CL::col(j, u.q));
-          pd[b][j].load(db + o + CL::col(j, u.q));
-        }
+        py[b].load(yb + o);
+        pd[b].load(db + o);
       }
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
 #pragma unroll
-        for (int j = 0; j < CL::NJ; j++)
-#pragma unroll
-          for (int e = 0; e < CL::EV; e++) dot += to_float(py[b][j].e[e]) * to_float(pd[b][j].e[e]);   // softmax.py:187-188
+        for (int e = 0; e < GE::EV; e++) dot += to_float(py[b].e[e]) * to_float(pd[b].e[e]);   // softmax.py:187-188
       }
-    dot = row_sum(dot);
+    dot = row_sum<GE::LPR>(dot);
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
-        const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
+        P out;
 #pragma unroll
-        for (int j = 0; j < CL::NJ; j++) {
-          P out;
-#pragma unroll
-          for (int e = 0; e < CL::EV; e++)
-            out.e[e] = from_float<T>(to_float(py[b][j].e[e]) * (to_float(pd[b][j].e[e]) - dot) * a.scale);   // :189
-          out.store(db + o + CL::col(j, u.q));
-        }
+        for (int e = 0; e < GE::EV; e++)
+          out.e[e] = from_float<T>(to_float(py[b].e[e]) * (to_float(pd[b].e[e]) - dot) * a.scale);   // :189
+        out.store(db + (int64_t)bid[b] * (BLOCK * BLOCK));
       }
   } else {
     float dot = 0.f;
     for (int b = 0; b < size; b++) {
       const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
+      P py, pd;
+      py.load(yb + o);
+      pd.load(db + o);
 #pragma unroll
-      for (int j = 0; j < CL::NJ; j++) {
-        P py, pd;
-        py.load(yb + o + CL::col(j, u.q));
-        pd.load(db + o + CL::col(j, u.q));
-#pragma unroll
-        for (int e = 0; e < CL::EV; e++) dot += to_float(py.e[e]) * to_float(pd.e[e]);
-      }
+      for (int e = 0; e < GE::EV; e++) dot += to_float(py.e[e]) * to_float(pd.e[e]);
     }
-    dot = row_sum(dot);
+    dot = row_sum<GE::LPR>(dot);
     for (int b = 0; b < size; b++) {
       const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
+      P py, pd, out;
+      py.load(yb + o);
+      pd.load(db + o);
 #pragma unroll
-      for (int j = 0; j < CL::NJ; j++) {
-        P py, pd, out;
-        py.load(yb + o + CL::col(j, u.q));
-        pd.load(db + o + CL::col(j, u.q));
-#pragma unroll
-        for (int e = 0; e < CL::EV; e++) out.e[e] = from_float<T>(to_float(py.e[e]) * (to_float(pd.e[e]) - dot) * a.scale);
-        out.store(db + o + CL::col(j, u.q));
-      }
+      for (int e = 0; e < GE::EV; e++) out.e[e] = from_float<T>(to_float(py.e[e]) * (to_float(pd.e[e]) - dot) * a.scale);
+      out.store(db + o);
     }
   }
 }
 
-// Register budget: a lane keeps NB * BLOCK/4 values (forward, fp32) or twice that many raw elements (backward).
-template <typename T, int BLOCK> constexpr int max_nb_fwd() { return 128 / (BLOCK / 4); }
-template <typename T, int BLOCK> constexpr int max_nb_bwd() { return (int)(128 * 4 / (2 * (BLOCK / 4) * sizeof(T))) > 32 ? 32 : (int)(128 * 4 / (2 * (BLOCK / 4) * sizeof(T))); }
+// Register budget: a lane keeps NB * EV fp32 values (forward) or 2 * NB raw chunks (backward).
+template <typename T, int BLOCK> constexpr int max_nb_fwd() { return 128 / Geo<T, BLOCK>::EV > 32 ? 32 : 128 / Geo<T, BLOCK>::EV; }
+template <typename T, int BLOCK> constexpr int max_nb_bwd() { return 16; }
 
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
   const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
@@ -304,22 +288,20 @@ template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hi
 
 template <typename T, int BLOCK> void launch_fwd(const FwdArgs &a, int maxlut, hipStream_t st) {
   constexpr int MX = max_nb_fwd<T, BLOCK>();
-  if (maxlut <= 1 && 1 <= MX) launch_fwd_nb<T, BLOCK, 1>(a, st);
-  else if (maxlut <= 2 && 2 <= MX) launch_fwd_nb<T, BLOCK, 2>(a, st);
-  else if (maxlut <= 4 && 4 <= MX) launch_fwd_nb<T, BLOCK, 4>(a, st);
-  else if (maxlut <= 8 && 8 <= MX) launch_fwd_nb<T, BLOCK, (8 <= MX ? 8 : 0)>(a, st);
+  if (maxlut <= 1) launch_fwd_nb<T, BLOCK, 1>(a, st);
+  else if (maxlut <= 2) launch_fwd_nb<T, BLOCK, 2>(a, st);
+  else if (maxlut <= 4) launch_fwd_nb<T, BLOCK, 4>(a, st);
+  else if (maxlut <= 8) launch_fwd_nb<T, BLOCK, 8>(a, st);
   else if (maxlut <= 16 && 16 <= MX) launch_fwd_nb<T, BLOCK, (16 <= MX ? 16 : 0)>(a, st);
   else if (maxlut <= 32 && 32 <= MX) launch_fwd_nb<T, BLOCK, (32 <= MX ? 32 : 0)>(a, st);
   else launch_fwd_nb<T, BLOCK, 0>(a, st);
 }
 template <typename T, int BLOCK> void launch_bwd(const BwdArgs &a, int maxlut, hipStream_t st) {
-  constexpr int MX = max_nb_bwd<T, BLOCK>();
-  if (maxlut <= 1 && 1 <= MX) launch_bwd_nb<T, BLOCK, 1>(a, st);
-  else if (maxlut <= 2 && 2 <= MX) launch_bwd_nb<T, BLOCK, (2 <= MX ? 2 : 0)>(a, st);
-  else if (maxlut <= 4 && 4 <= MX) launch_bwd_nb<T, BLOCK, (4 <= MX ? 4 : 0)>(a, st);
-  else if (maxlut <= 8 && 8 <= MX) launch_bwd_nb<T, BLOCK, (8 <= MX ? 8 : 0)>(a, st);
-  else if (maxlut <= 16 && 16 <= MX) launch_bwd_nb<T, BLOCK, (16 <= MX ? 16 : 0)>(a, st);
-  else if (maxlut <= 32 && 32 <= MX) launch_bwd_nb<T, BLOCK, (32 <= MX ? 32 : 0)>(a, st);
+  if (maxlut <= 1) launch_bwd_nb<T, BLOCK, 1>(a, st);
+  else if (maxlut <= 2) launch_bwd_nb<T, BLOCK, 2>(a, st);
+  else if (maxlut <= 4) launch_bwd_nb<T, BLOCK, 4>(a, st);
+  else if (maxlut <= 8) launch_bwd_nb<T, BLOCK, 8>(a, st);
+  else if (maxlut <= 16) launch_bwd_nb<T, BLOCK, 16>(a, st);
   else launch_bwd_nb<T, BLOCK, 0>(a, st);
 }
 
@@ -342,6 +324,19 @@ template <typename T> int dispatch_bwd(const BwdArgs &a, int block, int maxlut, 
     default: return BSP_ERR_UNSUPPORTED;
   }
   return BSP_OK;
+}
+
+template <typename T> int64_t units_for(int block, int64_t rows_of_blocks) {
+  switch (block) {
+    case 16: return rows_of_blocks * Geo<T, 16>::G;
+    case 32: return rows_of_blocks * Geo<T, 32>::G;
+    case 64: return rows_of_blocks * Geo<T, 64>::G;
+    case 128: return rows_of_blocks * Geo<T, 128>::G;
+    default: return 0;
+  }
+}
+int64_t n_units(int dtype, int block, int64_t rows_of_blocks) {
+  return dtype == BSP_F32 ? units_for<float>(block, rows_of_blocks) : units_for<f16>(block, rows_of_blocks);
 }
 
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
@@ -370,8 +365,8 @@ extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d
   a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
   a.Z = Z; a.H = H; a.R = R; a.x_sz = x_stride_z;
-  a.n_units = (int64_t)Z * H * R * (block / 16);
-  if (a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
+  if (a.n_units <= 0 || a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_fwd<f16>(a, block, maxlut, as_stream(stream)); break;
@@ -393,8 +388,8 @@ extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, 
   BwdArgs a;
   a.y = y; a.dy = dy; a.scale = scale; a.lut = d_lut;
   a.Z = Z; a.H = H; a.R = R; a.y_sz = y_stride_z; a.dy_sz = dy_stride_z;
-  a.n_units = (int64_t)Z * H * R * (block / 16);
-  if (a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
+  if (a.n_units <= 0 || a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_bwd<f16>(a, block, maxlut, as_stream(stream)); break;
