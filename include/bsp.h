@@ -74,6 +74,16 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
                       uint8_t *d_valid, int64_t cap_rows, void *d_ws, int64_t ws_bytes, int *n_levels,
                       int *packs, int64_t *rows, int64_t *total_rows, int *all_valid, void *stream);
 
+/* Group plan (no counterpart in the reference; an optional accelerator for the launchers below).
+ * BSP_GROUP consecutive block-rows (by_rows != 0) or block-columns of one head form a group that one workgroup
+ * processes together, sharing the dense tiles its members have in common.  d_plan receives 4 ints per group
+ * (first entry, entries, head, group index; sorted by decreasing entries) followed by BSP_GROUP+1 ints per entry
+ * (position along the other dimension, block id of each member or -1).  plan_cap >= bsp_group_plan_cap(...). */
+#define BSP_GROUP 4
+int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);
+int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int32_t *d_plan, int64_t plan_cap,
+                         void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream);
+
 /* ---------------------------------------------------------------------------------------------------
  * Matmul launchers.  Strides are in elements; the innermost stride of every operand is 1 and rows start on
  * 16-byte boundaries.  trans_x means the stored matrix is read transposed, as in the reference.
@@ -82,28 +92,31 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
 /* sparse = dense x dense: replaces _sparse_matmul._sdd_matmul + the SDD branch of the kernel
  * (matmul.py:299-364, 30-54).  One call per pack level of the sdd table.  For every valid table row
  * (h, i, j, p):  C[z, p] = op(A)[z, h, i*block:(i+1)*block, 0:K] . op(B)[z, h, 0:K, j*block:(j+1)*block].
- * lda / ldb: row stride of the stored 2-D matrices.  n_groups = rows / (pack*pack). */
+ * lda / ldb: row stride of the stored 2-D matrices.  n_groups = rows / (pack*pack).
+ * d_gplan / n_plan_groups / plan_lines: optional group plan of the layout built with by_rows = 1, its number of
+ * groups and the number of block-rows per head (NULL / 0 / 0 if none); when given, a kernel that shares operand
+ * tiles inside each group may take the launch. */
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
                    int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                    int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
-                   const uint8_t *d_valid, int64_t n_groups, void *stream);
+                   const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
 
 /* dense = sparse x dense: replaces _sparse_matmul._dsd_matmul + the DSD branch (matmul.py:507-552, 56-82).
  * C[z, h] = op(A_sparse)[h] . op(B)[z, h], written transposed when trans_c.  N = free dimension of op(B).
  * a_stride_z = 0 shares one sparse operand over the batch.  d_lut / d_plan / width from bsp_dxx_lut_build
- * with trans = !trans_a. */
+ * with trans = !trans_a; d_gplan (optional) from bsp_group_plan_build with by_rows = !trans_a. */
 int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                    int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                   const int32_t *d_plan, int width, void *stream);
+                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
 
 /* dense = dense x sparse: replaces _sparse_matmul._dds_matmul + the DDS branch (matmul.py:460-505, 83-99).
  * C[z, h] = op(A)[z, h] . op(B_sparse)[h], written transposed when trans_c.  M = free dimension of op(A).
- * Tables from bsp_dxx_lut_build with trans = trans_b. */
+ * Tables from bsp_dxx_lut_build with trans = trans_b; d_gplan (optional) with by_rows = trans_b. */
 int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                    int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                   const int32_t *d_plan, int width, void *stream);
+                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Softmax launchers: replace softmax_fwd / softmax_bwd and their dispatch (softmax.py:7-138, 144-194,

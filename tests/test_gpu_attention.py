@@ -94,11 +94,14 @@ def test_specialised_and_general_kernels_agree(monkeypatch):
         o = dsd(sm(sdd(qg, kg), scale=0.125), vg)
         o.backward(do)
         return o, qg.grad, kg.grad, vg.grad
-    fast = run()
+    grouped = run()                                   # row-group kernels (default for block 64)
+    monkeypatch.setenv('BSP_NO_GROUPS', '1')
+    fast = run()                                      # per-block / per-segment specialised kernels
     monkeypatch.setenv('BSP_GENERIC_ONLY', '1')
-    general = run()
-    for a, b, name in zip(fast, general, ('out', 'dq', 'dk', 'dv')):
-        assert_close(a, b.float(), torch.float16, name)
+    general = run()                                   # general LDS-tiled kernels
+    for a, b, c, name in zip(grouped, fast, general, ('out', 'dq', 'dk', 'dv')):
+        assert_close(a, c.float(), torch.float16, name + ' grouped vs general')
+        assert_close(b, c.float(), torch.float16, name + ' specialised vs general')
 
 
 def test_full_size_properties():

@@ -66,3 +66,40 @@ def test_empty_head_raises():
     lay[0, 1, 2] = 1
     with pytest.raises(RuntimeError):
         _sparse_matmul.make_dxx_lut(lay, 16, 16, True, DEV)
+
+
+@pytest.mark.parametrize('by_rows', [True, False])
+def test_group_plan(by_rows):
+    # our own work list for the row-group kernels: 4 consecutive lines per group, one entry per position where any
+    # member has a block, header sorted by decreasing number of entries
+    from torch_blocksparse.matmul import GroupPlan
+    for lay in (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64)):
+        plan = GroupPlan.build(lay, by_rows, DEV)
+        t = plan.table.cpu().tolist()
+        H, R, C = lay.shape
+        L, B = (R, C) if by_rows else (C, R)
+        ng = H * ((L + 3) // 4)
+        assert plan.n_groups == ng and plan.lines == L
+        rank = (torch.cumsum(lay.reshape(-1), 0) - 1).reshape(lay.shape)
+        header = [t[4 * i:4 * i + 4] for i in range(ng)]
+        counts = [h[1] for h in header]
+        assert counts == sorted(counts, reverse=True)
+        assert sorted((h[2], h[3]) for h in header) == [(h, g) for h in range(H) for g in range((L + 3) // 4)]
+        total = 0
+        for start, count, h, lg in header:
+            exp = []
+            for b in range(B):
+                bids = []
+                for m in range(4):
+                    line = lg * 4 + m
+                    if line < L:
+                        r, c = (line, b) if by_rows else (b, line)
+                        bids.append(int(rank[h, r, c]) if lay[h, r, c] else -1)
+                    else:
+                        bids.append(-1)
+                if any(x >= 0 for x in bids):
+                    exp.append([b] + bids)
+            got = [t[4 * ng + 5 * (start + k):4 * ng + 5 * (start + k + 1)] for k in range(count)]
+            assert got == exp
+            total += count
+        assert len(t) == 4 * ng + 5 * total

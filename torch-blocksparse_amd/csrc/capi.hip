@@ -7,6 +7,11 @@ using namespace bsp;
 
 namespace {
 // BSP_GENERIC_ONLY=1 in the environment routes every launch to the general kernels (used to test both paths).
+// BSP_NO_GROUPS=1 ignores group plans (the per-block / per-segment specialised kernels run instead).
+bool no_groups() {
+  const char *e = std::getenv("BSP_NO_GROUPS");
+  return e && e[0] == '1';
+}
 bool generic_only() {
   const char *e = std::getenv("BSP_GENERIC_ONLY");
   return e && e[0] == '1';
@@ -35,7 +40,8 @@ extern "C" const char *bsp_strerror(int status) {
 extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
                               int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                               int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
-                              const uint8_t *d_valid, int64_t n_groups, void *stream) {
+                              const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups,
+                              int plan_lines, void *stream) {
   if (!a || !b || !c || !d_lut || Z <= 0 || K <= 0 || n_groups < 0) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   if (K % 16) return BSP_ERR_K_MULTIPLE;   // reference matmul.py:318-319
@@ -47,6 +53,8 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.a_sz = a_stride_z; g.a_sh = a_stride_h; g.lda = lda;
   g.b_sz = b_stride_z; g.b_sh = b_stride_h; g.ldb = ldb; g.c_sz = c_stride_z;
   g.lut = d_lut; g.valid = d_valid; g.n_groups = n_groups;
+  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  if (g.gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
   // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);
@@ -83,8 +91,10 @@ static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, b
 extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                               int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
                               int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                              const int32_t *d_plan, int width, void *stream) {
+                              const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
+                              void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || N <= 0 || width < 0) return BSP_ERR_ARG;
+  if (d_gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   const int u = elems16(dtype);
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
@@ -96,6 +106,7 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.lut = d_lut; g.plan = d_plan; g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));   // step of the table: 8 for fp32, 16 otherwise (matmul.py:617)
   g.n_tiles = (N + 63) / 64;
+  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
   // rows of the kernel = rows of op(A); op(A)(m,k) is stored [k][m] when trans_a.  Dense (n,k) = op(B)[k][n]:
   // reduction contiguous when B is read transposed.  C[m][n] has n contiguous unless written transposed.
   return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, stream);
@@ -104,8 +115,10 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
 extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                               int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
                               int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                              const int32_t *d_plan, int width, void *stream) {
+                              const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
+                              void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || M <= 0 || width < 0) return BSP_ERR_ARG;
+  if (d_gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   const int u = elems16(dtype);
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
@@ -117,6 +130,7 @@ extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, 
   g.lut = d_lut; g.plan = d_plan; g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));
   g.n_tiles = (M + 63) / 64;
+  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
   // dds is dsd on the transposed problem: kernel rows = columns of op(B) (stored [k][col] unless trans_b), dense
   // rows = rows of op(A) (reduction contiguous unless trans_a), and C[row][col] has the kernel's m index contiguous
   // unless written transposed.

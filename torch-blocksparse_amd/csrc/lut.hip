@@ -334,6 +334,65 @@ __global__ void k_sdd_offsets(const int64_t *counts, int64_t *offsets, int nlev,
   (void)scal;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Group plan: the work list of the row-group matmul kernels (no counterpart in the reference).  BSP_GROUP
+// consecutive block-rows (by_rows) or block-columns of one head form a group; an entry of a group is one
+// position b along the other dimension where at least one member has a block: (b, blockid of member 0..3, -1
+// where absent).  Header rows (first entry, number of entries, head, group index) are sorted by decreasing number
+// of entries so that the longest groups are dispatched first.
+// ---------------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int64_t cell(int R, int C, int h, int line, int b, int by_rows) {
+  return by_rows ? ((int64_t)h * R + line) * C + b : ((int64_t)h * R + b) * C + line;
+}
+__global__ void k_gplan_count(const int32_t *lay, int H, int R, int C, int by_rows, int32_t *cnt) {
+  const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= (int64_t)H * NG) return;
+  const int h = (int)(i / NG), lg = (int)(i % NG);
+  int n = 0;
+  for (int b = 0; b < B; b++) {
+    bool any = false;
+    for (int g = 0; g < BSP_GROUP; g++) {
+      const int line = lg * BSP_GROUP + g;
+      if (line < L && lay[cell(R, C, h, line, b, by_rows)] != 0) any = true;
+    }
+    n += any;
+  }
+  cnt[i] = n;
+}
+__global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *cnt, const int32_t *start, int H, int R,
+                             int C, int by_rows, int32_t *plan) {
+  const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
+  const int64_t n_groups = (int64_t)H * NG;
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= n_groups) return;
+  const int h = (int)(i / NG), lg = (int)(i % NG);
+  // position in the sorted header: groups with more entries first, ties in natural order
+  const int mine = cnt[i];
+  int64_t pos = 0;
+  for (int64_t j = 0; j < n_groups; j++) pos += (cnt[j] > mine) || (cnt[j] == mine && j < i);
+  int32_t *hd = plan + 4 * pos;
+  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = lg;
+  int32_t *e = plan + 4 * n_groups + (int64_t)(BSP_GROUP + 1) * start[i];
+  for (int b = 0; b < B; b++) {
+    int32_t bid[BSP_GROUP];
+    bool any = false;
+    for (int g = 0; g < BSP_GROUP; g++) {
+      const int line = lg * BSP_GROUP + g;
+      bid[g] = -1;
+      if (line < L) {
+        const int64_t p = cell(R, C, h, line, b, by_rows);
+        if (lay[p] != 0) { bid[g] = rank[p]; any = true; }
+      }
+    }
+    if (any) {
+      e[0] = b;
+      for (int g = 0; g < BSP_GROUP; g++) e[1 + g] = bid[g];
+      e += BSP_GROUP + 1;
+    }
+  }
+}
+
 int prepare_counts(const int32_t *d_layout, int H, int R, int C, int32_t *ws, const Ws &o, hipStream_t st) {
   const int T = 256;
   hipLaunchKernelGGL(k_fill, dim3(1), dim3(64), 0, st, ws + o.scal, (int64_t)16, 0);
@@ -503,5 +562,41 @@ extern "C" int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, i
   BSP_HIP_CHECK(hipMemcpyAsync(&inval, ws + o.scal + S_INVALID, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   *all_valid = inval ? 0 : 1;
+  return BSP_OK;
+}
+
+extern "C" int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows) {
+  const int64_t L = by_rows ? R : C;
+  return 4 * (int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (BSP_GROUP + 1) * nnz;
+}
+
+extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int32_t *d_plan, int64_t plan_cap,
+                                    void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream) {
+  int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
+  if (rc != BSP_OK) return rc;
+  if (!d_plan || !n_groups || !plan_len) return BSP_ERR_ARG;
+  hipStream_t st = as_stream(stream);
+  Ws o(H, R, C);
+  int32_t *ws = (int32_t *)d_ws;
+  const int T = 256;
+  const int L = by_rows ? R : C;
+  const int64_t ng = (int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP);
+  rc = prepare_counts(d_layout, H, R, C, ws, o, st);
+  if (rc != BSP_OK) return rc;
+  hipLaunchKernelGGL(k_rank, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowstart, ws + o.rank);
+  // linepacks / segstart are free here: group entry counts and their prefix sums
+  hipLaunchKernelGGL(k_gplan_count, dim3(cdiv(ng, T)), dim3(T), 0, st, d_layout, H, R, C, by_rows, ws + o.linepacks);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.linepacks, ws + o.segstart, ng, (int32_t *)nullptr);
+  BSP_LAUNCH_CHECK();
+  int32_t total = 0;
+  BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.segstart + ng, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
+  *n_groups = (int)ng;
+  *plan_len = 4 * ng + (int64_t)(BSP_GROUP + 1) * total;
+  if (*plan_len > plan_cap) return BSP_ERR_CAPACITY;
+  hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(ng, T)), dim3(T), 0, st, d_layout, ws + o.rank, ws + o.linepacks, ws + o.segstart, H, R, C,
+                     by_rows, d_plan);
+  BSP_LAUNCH_CHECK();
+  BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;
 }

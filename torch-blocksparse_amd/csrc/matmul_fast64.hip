@@ -237,6 +237,220 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
     *reinterpret_cast<u32x4 *>(po + (int64_t)i * 8 * g.ldo) = *reinterpret_cast<const u32x4 *>(rs + i * 8 * kLdsRow);
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Row-group kernels.  A workgroup owns BSP_GROUP consecutive block-rows (or block-columns) of one head and walks
+// the entries of its group plan: every entry is one dense tile that at least one member needs.  The tile is
+// fetched once, with whole-line loads, into LDS and serves all members, so the L2-level reads of the shared
+// operand drop by the average number of members per entry (3.4x on the fixed attention layout) and each LDS
+// operand read feeds up to four MFMAs.  Each wavefront computes 16 rows of every member.
+// Workgroup w: batch z = w % Z (one batch per XCD when Z = 8), plan group w / Z in the plan's
+// longest-first order.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int G = BSP_GROUP;
+
+template <typename T> __device__ __forceinline__ void store_slice(T *cs, T *dst, int64_t ld, const f32x4 (&acc)[4], int lane) {
+  // acc[j][e] = out[row lane%16][col 16*j + 4*(lane/16) + e] of a 16 x 64 slice -> LDS -> two stores of 8 whole rows
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk.e[e] = from_float<T>(acc[j][e]);
+    *reinterpret_cast<u32x2 *>(cs + (lane & 15) * kLdsRow + 16 * j + 4 * (lane >> 4)) = pk.raw;
+  }
+  __builtin_amdgcn_wave_barrier();
+  const T *rs = cs + (lane >> 3) * kLdsRow + (lane & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 2; i++)
+    *reinterpret_cast<u32x4 *>(dst + ((lane >> 3) + 8 * i) * ld + (lane & 7) * 8) = *reinterpret_cast<const u32x4 *>(rs + i * 8 * kLdsRow);
+  __builtin_amdgcn_wave_barrier();
+}
+
+// sdd, K = 64: members = block-rows of A (their 16-row slices stay in registers), entries = block-columns (B tiles)
+template <typename T>
+__global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int TILE = 64 * kLdsRow;
+  __shared__ __attribute__((aligned(16))) T Ks[2][TILE];
+  __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int z = blockIdx.x % g.Z;
+  const int32_t *hd = g.gplan + 4 * (int64_t)(blockIdx.x / g.Z);
+  const int e0 = hd[0], ne = hd[1], h = hd[2], lg = hd[3];
+  const int32_t *ent = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const int r = lane & 15, kq = (lane >> 4) * 8;
+  const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
+  const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
+  frag_t xq[G][2];
+#pragma unroll
+  for (int m = 0; m < G; m++) {
+    const int row = lg * G + m;
+    if (row < g.lines) {
+      const T *p = pa + ((int64_t)row * 64 + wave * 16 + r) * g.lda + kq;
+      xq[m][0] = *reinterpret_cast<const frag_t *>(p);
+      xq[m][1] = *reinterpret_cast<const frag_t *>(p + 32);
+    }
+  }
+  const int ck = tid >> 3, cc = (tid & 7) * 8;
+  struct Stage { u32x4 y[2]; };
+  Stage ring[kRing];
+  auto issue = [&](Stage &st, int e) {
+    const T *py = pb + ((int64_t)ent[(G + 1) * e] * 64 + ck) * g.ldb + cc;
+    st.y[0] = *reinterpret_cast<const u32x4 *>(py);
+    st.y[1] = *reinterpret_cast<const u32x4 *>(py + 32 * g.ldb);
+  };
+#pragma unroll
+  for (int u = 0; u < kRing; u++)
+    if (u < ne) issue(ring[u], u);
+  for (int e0i = 0; e0i < ne; e0i += kRing) {
+#pragma unroll
+    for (int u = 0; u < kRing; u++) {
+      const int e = e0i + u;
+      if (e < ne) {
+        const int buf = e & 1;
+        *reinterpret_cast<u32x4 *>(&Ks[buf][ck * kLdsRow + cc]) = ring[u].y[0];
+        *reinterpret_cast<u32x4 *>(&Ks[buf][(ck + 32) * kLdsRow + cc]) = ring[u].y[1];
+        if (e + kRing < ne) issue(ring[u], e + kRing);
+        __syncthreads();
+        frag_t yf[4][2];
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+          for (int s2 = 0; s2 < 2; s2++) yf[j][s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + r) * kLdsRow + 32 * s2 + kq]);
+#pragma unroll
+        for (int m = 0; m < G; m++) {
+          const int bid = ent[(G + 1) * e + 1 + m];
+          if (bid >= 0) {
+            f32x4 acc[4];
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+              acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+              for (int s2 = 0; s2 < 2; s2++) acc[j] = M::run(yf[j][s2], xq[m][s2], acc[j]);   // rows n = 16j + 4*(lane/16) + e, column m-row = lane%16
+            }
+            store_slice<T>(Cs[wave], pc + (int64_t)bid * 4096 + wave * 1024, 64, acc, lane);
+          }
+        }
+      }
+    }
+  }
+}
+
+// dsd / dds: members = output lines (block-rows of the result), entries = positions of the reduction
+template <typename T, bool SP_TRANS>
+__global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int TILE = 64 * kLdsRow;
+  constexpr int RING = 2;
+  __shared__ __attribute__((aligned(16))) T Ys[2][TILE];
+  __shared__ __attribute__((aligned(16))) T Xs[SP_TRANS ? 2 : 1][SP_TRANS ? TILE : 8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int z = blockIdx.x % g.Z;
+  const int64_t rest = blockIdx.x / g.Z;
+  const int n0 = (int)(rest % g.n_tiles) * 64;
+  const int32_t *hd = g.gplan + 4 * (rest / g.n_tiles);
+  const int e0 = hd[0], ne = hd[1], depth = hd[2], lg = hd[3];
+  const int32_t *ent = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
+  const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
+  const int64_t ldd = g.ldd;
+  const int ck = tid >> 3, cc = (tid & 7) * 8;
+  const int xr = wave * 16 + (lane & 15), xq = (lane >> 4) * 8;
+  struct Stage { u32x4 y[2]; u32x4 x[G][2]; };
+  Stage ring[RING];
+  auto issue = [&](Stage &st, int e) {
+    const int32_t *en = ent + (G + 1) * e;
+    const T *py = dn + ((int64_t)en[0] * 64 + ck) * ldd + cc;
+    st.y[0] = *reinterpret_cast<const u32x4 *>(py);
+    st.y[1] = *reinterpret_cast<const u32x4 *>(py + 32 * ldd);
+#pragma unroll
+    for (int m = 0; m < G; m++) {
+      const int bid = en[1 + m];
+      if (bid >= 0) {
+        const T *blk = sp + (int64_t)bid * 4096;
+        if constexpr (SP_TRANS) {
+          st.x[m][0] = *reinterpret_cast<const u32x4 *>(blk + ck * 64 + cc);
+          st.x[m][1] = *reinterpret_cast<const u32x4 *>(blk + (ck + 32) * 64 + cc);
+        } else {
+          st.x[m][0] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + xq);
+          st.x[m][1] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + 32 + xq);
+        }
+      }
+    }
+  };
+  f32x4 acc[G][4];
+#pragma unroll
+  for (int m = 0; m < G; m++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[m][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int u = 0; u < RING; u++)
+    if (u < ne) issue(ring[u], u);
+  const int tr_row = (lane >> 4) * 8 + ((lane & 15) >> 2), tr_col = (lane & 3) * 4;
+  int xb = 0;
+  for (int e0i = 0; e0i < ne; e0i += RING) {
+#pragma unroll
+    for (int u = 0; u < RING; u++) {
+      const int e = e0i + u;
+      if (e < ne) {
+        const int buf = e & 1;
+        Stage &st = ring[u];
+        const int32_t *en = ent + (G + 1) * e;
+        int bid[G];
+#pragma unroll
+        for (int m = 0; m < G; m++) bid[m] = en[1 + m];
+        *reinterpret_cast<u32x4 *>(&Ys[buf][ck * kLdsRow + cc]) = st.y[0];
+        *reinterpret_cast<u32x4 *>(&Ys[buf][(ck + 32) * kLdsRow + cc]) = st.y[1];
+        frag_t xf[G][2];
+        if constexpr (SP_TRANS) {
+#pragma unroll
+          for (int m = 0; m < G; m++)
+            if (bid[m] >= 0) {
+              *reinterpret_cast<u32x4 *>(&Xs[xb][ck * kLdsRow + cc]) = st.x[m][0];
+              *reinterpret_cast<u32x4 *>(&Xs[xb][(ck + 32) * kLdsRow + cc]) = st.x[m][1];
+              __syncthreads();
+#pragma unroll
+              for (int s2 = 0; s2 < 2; s2++) {
+                const T *xrow = &Xs[xb][(32 * s2 + tr_row) * kLdsRow + 16 * wave + tr_col];
+                xf[m][s2] = tr_frag<T>(xrow, xrow + 4 * kLdsRow);
+              }
+              xb ^= 1;
+            }
+        } else {
+#pragma unroll
+          for (int m = 0; m < G; m++) {
+            xf[m][0] = __builtin_bit_cast(frag_t, st.x[m][0]);
+            xf[m][1] = __builtin_bit_cast(frag_t, st.x[m][1]);
+          }
+          __syncthreads();
+        }
+        if (e + RING < ne) issue(st, e + RING);
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) {
+          const T *yrow = &Ys[buf][(32 * s2 + tr_row) * kLdsRow + tr_col];
+#pragma unroll
+          for (int j = 0; j < 4; j++) {
+            frag_t yf = tr_frag<T>(yrow + 16 * j, yrow + 16 * j + 4 * kLdsRow);
+#pragma unroll
+            for (int m = 0; m < G; m++)
+              if (bid[m] >= 0) acc[m][j] = M::run(yf, xf[m][s2], acc[m][j]);
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+  T *cs = &Ys[0][(wave * 16) * kLdsRow];
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
+#pragma unroll
+  for (int m = 0; m < G; m++) {
+    const int line = lg * G + m;
+    if (line < g.lines) store_slice<T>(cs, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, acc[m], lane);
+  }
+}
+
 bool fast_ok_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc) {
   return block == 64 && pack == 1 && a_kc && b_kc && g.K % 64 == 0;
 }
@@ -245,6 +459,12 @@ bool fast_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
 }
 
 template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
+  if (g.gplan && g.n_pgroups > 0 && g.K == 64 && !g.valid) {
+    const int64_t n = (int64_t)g.n_pgroups * g.Z;
+    if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+    hipLaunchKernelGGL(k_sdd64_rg<T>, dim3((unsigned)n), dim3(256), 0, st, g);
+    return BSP_OK;
+  }
   const int64_t n_wg = (g.n_groups * g.Z + 3) / 4;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
@@ -252,6 +472,13 @@ template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
   return BSP_OK;
 }
 template <typename T> int xsd_fast_t(const XsdArgs &g, bool sp_trans, hipStream_t st) {
+  if (g.gplan && g.n_pgroups > 0) {
+    const int64_t n = (int64_t)g.n_pgroups * g.n_tiles * g.Z;
+    if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+    if (sp_trans) hipLaunchKernelGGL((k_xsd64_rg<T, true>), dim3((unsigned)n), dim3(256), 0, st, g);
+    else hipLaunchKernelGGL((k_xsd64_rg<T, false>), dim3((unsigned)n), dim3(256), 0, st, g);
+    return BSP_OK;
+  }
   const int64_t n_wg = (int64_t)g.width * g.n_tiles * g.Z;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;

@@ -183,6 +183,7 @@ struct SddArgs {
   int64_t a_sz, a_sh, lda, b_sz, b_sh, ldb, c_sz;
   const int32_t *lut; const uint8_t *valid;
   int64_t n_groups;
+  const int32_t *gplan; int n_pgroups; int lines;   // optional group plan (by rows), its groups, block-rows per head
 };
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
@@ -242,6 +243,7 @@ struct XsdArgs {
   int64_t sp_sz, dn_sz, dn_sh, ldd, out_sz, out_sh, ldo;
   const int32_t *lut; const int32_t *plan; int width; int div2;   // div2 = 2 * block / step of the table
   int n_tiles;
+  const int32_t *gplan; int n_pgroups; int lines;   // optional group plan, its groups, lines (block-rows or -columns) per head
 };
 
 template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m, k) of the segment's blocks

@@ -43,9 +43,40 @@ class _Timer:
         return self.start.elapsed_time(self.stop)
 
 
+class GroupPlan:
+    """Work list of the row-group kernels (see bsp_group_plan_build): device table, number of groups, lines per head."""
+
+    def __init__(self, table, n_groups, lines):
+        self.table, self.n_groups, self.lines = table, n_groups, lines
+
+    @staticmethod
+    def build(layout, by_rows, device):
+        lib = _lib.load()
+        dev = torch.device(device)
+        lay = _lib.layout_to_device(layout, dev)
+        H, R, C = lay.shape
+        ws, ws_bytes = _lib.workspace(lay, dev)
+        nnz = int((layout != 0).sum())
+        cap = lib.bsp_group_plan_cap(H, R, C, nnz, int(bool(by_rows)))
+        table = torch.empty((cap,), dtype=torch.int32, device=dev)
+        n_groups, n = ctypes.c_int(0), ctypes.c_int64(0)
+        rc = lib.bsp_group_plan_build(_lib.ptr(lay), H, R, C, int(bool(by_rows)), _lib.ptr(table), cap, _lib.ptr(ws), ws_bytes,
+                                      ctypes.byref(n_groups), ctypes.byref(n), _lib.stream_ptr(dev))
+        _lib.check(rc, 'bsp_group_plan_build')
+        return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C)
+
+    @staticmethod
+    def args(plan):
+        if plan is None:
+            return ctypes.c_void_p(0), 0, 0
+        return _lib.ptr(plan.table), plan.n_groups, plan.lines
+
+
 class SddTables(list):
-    """The per-pack sdd tables, in the reference's order; `nnz` is the number of blocks of the output."""
+    """The per-pack sdd tables, in the reference's order; `nnz` is the number of blocks of the output, `gplan` the
+    optional row-group plan of the layout."""
     nnz = 0
+    gplan = None
 
 
 class _sparse_matmul(torch.autograd.Function):
@@ -87,6 +118,8 @@ class _sparse_matmul(torch.autograd.Function):
             break
         luts, widths, out_packs = SddTables(), [], []
         luts.nnz = nnz
+        if block == 64:
+            luts.gplan = GroupPlan.build(layout, True, dev)
         done = 0
         for k in range(n_levels.value):
             p, r = int(packs[k]), int(rows[k])
@@ -114,11 +147,12 @@ class _sparse_matmul(torch.autograd.Function):
         total_width = luts.nnz if isinstance(luts, SddTables) else sum(w * p * p for w, p in zip(widths, packs))
         c = torch.empty((AS0, total_width, block, block), dtype=a.dtype, device=a.device)
         timer = _Timer(bench, a.device)
+        gplan = GroupPlan.args(getattr(luts, 'gplan', None) if len(luts) == 1 else None)
         for lut, width, pack in zip(luts, widths, packs):
             rc = lib.bsp_sdd_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                     AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
                                     c.stride(0), block, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
-                                    _lib.stream_ptr(a.device))
+                                    gplan[0], gplan[1], gplan[2], _lib.stream_ptr(a.device))
             _lib.check(rc, 'bsp_sdd_matmul')
         time[0] = timer.done()
         return c
@@ -153,6 +187,7 @@ class _sparse_matmul(torch.autograd.Function):
         _lib.check(rc, 'bsp_dxx_lut_build')
         lut = lut[:n.value]
         lut.plan = plan
+        lut.gplan = GroupPlan.build(layout, trans, dev) if block == 64 else None
         return lut, num_locks.value, width.value, None
 
     @staticmethod
@@ -179,7 +214,7 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dds_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), a.size(0), M, a.stride(0), a.stride(1), a.stride(2), b_sz, c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
-                                        _lib.stream_ptr(a.device))
+                                        *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(a.device))
         _lib.check(rc, 'bsp_dds_matmul')
         time[0] = timer.done()
         if M != AS2:
@@ -201,7 +236,7 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dsd_matmul(_lib.DTYPES[b.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), b.size(0), N, a_sz, b.stride(0), b.stride(1), b.stride(2), c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
-                                        _lib.stream_ptr(b.device))
+                                        *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(b.device))
         _lib.check(rc, 'bsp_dsd_matmul')
         time[0] = timer.done()
         if N != BS3:
