@@ -43,6 +43,12 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t wg, int64_t n_wg) {
   return (wg & 7) * per + (wg >> 3);
 }
 
+// Look-up tables are read-only for every kernel that consumes them.  Reading them through the constant address
+// space lets the compiler use scalar loads for wave-uniform entries even after a barrier (a plain global pointer
+// falls back to vector loads there, and waiting for such a load means waiting for every prefetch issued before it).
+typedef const int32_t __attribute__((address_space(4))) *table_ptr;
+__device__ __forceinline__ table_ptr as_table(const int32_t *p) { return (table_ptr)p; }
+
 template <typename T> struct TypeInfo;
 template <> struct TypeInfo<f16> { static constexpr int kVec = 8; static constexpr bool k16 = true; };
 template <> struct TypeInfo<bf16> { static constexpr int kVec = 8; static constexpr bool k16 = true; };

@@ -139,11 +139,11 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
   const int z = (int)(w / per_z);
   const int seg = (int)((w % per_z) / g.n_tiles);
   const int n0 = (int)(w % g.n_tiles) * 64;
-  const int32_t *hd = g.lut + 6 * (int64_t)seg;
+  const table_ptr hd = as_table(g.lut) + 6 * (int64_t)seg;
   const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];
   const int nblk = seglen >> 6;
   if (nblk == 0 && seg > 0 && hd[-4] == column && hd[-3] == depth) return;   // see k_xsd: empty twin of a real segment
-  const int32_t *plan = g.plan + 2 * (int64_t)((offset - 6 * g.width) / g.div2);
+  const table_ptr plan = as_table(g.plan) + 2 * (int64_t)((offset - 6 * g.width) / g.div2);
   const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;
@@ -247,6 +247,9 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
 // longest-first order.
 // ---------------------------------------------------------------------------------------------------------
 constexpr int G = BSP_GROUP;
+#ifndef XSD_RING
+#define XSD_RING 2
+#endif
 
 template <typename T> __device__ __forceinline__ void store_slice(T *cs, T *dst, int64_t ld, const f32x4 (&acc)[4], int lane) {
   // acc[j][e] = out[row lane%16][col 16*j + 4*(lane/16) + e] of a 16 x 64 slice -> LDS -> two stores of 8 whole rows
@@ -275,9 +278,9 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int z = blockIdx.x % g.Z;
-  const int32_t *hd = g.gplan + 4 * (int64_t)(blockIdx.x / g.Z);
+  const table_ptr hd = as_table(g.gplan) + 4 * (int64_t)(blockIdx.x / g.Z);
   const int e0 = hd[0], ne = hd[1], h = hd[2], lg = hd[3];
-  const int32_t *ent = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
   const int r = lane & 15, kq = (lane >> 4) * 8;
   const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
   const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
@@ -343,16 +346,16 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
-  constexpr int RING = 2;
+  constexpr int RING = XSD_RING;
   __shared__ __attribute__((aligned(16))) T Ys[2][TILE];
   __shared__ __attribute__((aligned(16))) T Xs[SP_TRANS ? 2 : 1][SP_TRANS ? TILE : 8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int z = blockIdx.x % g.Z;
   const int64_t rest = blockIdx.x / g.Z;
   const int n0 = (int)(rest % g.n_tiles) * 64;
-  const int32_t *hd = g.gplan + 4 * (rest / g.n_tiles);
+  const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
   const int e0 = hd[0], ne = hd[1], depth = hd[2], lg = hd[3];
-  const int32_t *ent = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
   const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;
@@ -361,23 +364,23 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   struct Stage { u32x4 y[2]; u32x4 x[G][2]; };
   Stage ring[RING];
   auto issue = [&](Stage &st, int e) {
-    const int32_t *en = ent + (G + 1) * e;
+    const table_ptr en = ent + (G + 1) * e;
     const T *py = dn + ((int64_t)en[0] * 64 + ck) * ldd + cc;
     st.y[0] = *reinterpret_cast<const u32x4 *>(py);
     st.y[1] = *reinterpret_cast<const u32x4 *>(py + 32 * ldd);
+    // A fixed number of loads per stage whatever the entry holds, so that the wait before a stage is consumed can
+    // count exactly the loads issued after it (a data-dependent count would force a wait for everything in flight).
+    // Absent members read one cache line at the start of the sparse tensor instead.
 #pragma unroll
     for (int m = 0; m < G; m++) {
       const int bid = en[1 + m];
-      if (bid >= 0) {
-        const T *blk = sp + (int64_t)bid * 4096;
-        if constexpr (SP_TRANS) {
-          st.x[m][0] = *reinterpret_cast<const u32x4 *>(blk + ck * 64 + cc);
-          st.x[m][1] = *reinterpret_cast<const u32x4 *>(blk + (ck + 32) * 64 + cc);
-        } else {
-          st.x[m][0] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + xq);
-          st.x[m][1] = *reinterpret_cast<const u32x4 *>(blk + xr * 64 + 32 + xq);
-        }
-      }
+      const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * 4096;
+      const T *p0, *p1;
+      if constexpr (SP_TRANS) { p0 = blk + ck * 64 + cc; p1 = p0 + 32 * 64; }
+      else { p0 = blk + xr * 64 + xq; p1 = p0 + 32; }
+      if (bid < 0) { p0 = sp; p1 = sp; }
+      st.x[m][0] = *reinterpret_cast<const u32x4 *>(p0);
+      st.x[m][1] = *reinterpret_cast<const u32x4 *>(p1);
     }
   };
   f32x4 acc[G][4];
@@ -385,31 +388,36 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   for (int m = 0; m < G; m++)
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[m][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-  for (int u = 0; u < RING; u++)
-    if (u < ne) issue(ring[u], u);
   const int tr_row = (lane >> 4) * 8 + ((lane & 15) >> 2), tr_col = (lane & 3) * 4;
-  int xb = 0;
-  for (int e0i = 0; e0i < ne; e0i += RING) {
+  if (ne > 0) {
+    // Every vector-memory operation below is unconditional: the loop runs a whole number of ring rounds, prefetches
+    // past the end re-read the last entry, and the padding steps mark all members absent.
+    const int last = ne - 1;
 #pragma unroll
-    for (int u = 0; u < RING; u++) {
-      const int e = e0i + u;
-      if (e < ne) {
+    for (int u = 0; u < RING; u++) issue(ring[u], u < last ? u : last);
+    int xb = 0;
+    const int steps = (ne + RING - 1) / RING * RING;
+    for (int e0i = 0; e0i < steps; e0i += RING) {
+#pragma unroll
+      for (int u = 0; u < RING; u++) {
+        const int e = e0i + u;
+        const bool live = e < ne;
         const int buf = e & 1;
         Stage &st = ring[u];
-        const int32_t *en = ent + (G + 1) * e;
+        const table_ptr en = ent + (G + 1) * (live ? e : last);
         int bid[G];
 #pragma unroll
-        for (int m = 0; m < G; m++) bid[m] = en[1 + m];
+        for (int m = 0; m < G; m++) bid[m] = live ? en[1 + m] : -1;
         *reinterpret_cast<u32x4 *>(&Ys[buf][ck * kLdsRow + cc]) = st.y[0];
         *reinterpret_cast<u32x4 *>(&Ys[buf][(ck + 32) * kLdsRow + cc]) = st.y[1];
         frag_t xf[G][2];
         if constexpr (SP_TRANS) {
 #pragma unroll
-          for (int m = 0; m < G; m++)
+          for (int m = 0; m < G; m++) {
+            const u32x4 x0 = st.x[m][0], x1 = st.x[m][1];
             if (bid[m] >= 0) {
-              *reinterpret_cast<u32x4 *>(&Xs[xb][ck * kLdsRow + cc]) = st.x[m][0];
-              *reinterpret_cast<u32x4 *>(&Xs[xb][(ck + 32) * kLdsRow + cc]) = st.x[m][1];
+              *reinterpret_cast<u32x4 *>(&Xs[xb][ck * kLdsRow + cc]) = x0;
+              *reinterpret_cast<u32x4 *>(&Xs[xb][(ck + 32) * kLdsRow + cc]) = x1;
               __syncthreads();
 #pragma unroll
               for (int s2 = 0; s2 < 2; s2++) {
@@ -418,6 +426,8 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
               }
               xb ^= 1;
             }
+          }
+          if (!live) __syncthreads();   // a padding step still has to order its tile store against the next step
         } else {
 #pragma unroll
           for (int m = 0; m < G; m++) {
@@ -426,18 +436,24 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
           }
           __syncthreads();
         }
-        if (e + RING < ne) issue(st, e + RING);
+        frag_t yf[2][4];
 #pragma unroll
         for (int s2 = 0; s2 < 2; s2++) {
           const T *yrow = &Ys[buf][(32 * s2 + tr_row) * kLdsRow + tr_col];
 #pragma unroll
-          for (int j = 0; j < 4; j++) {
-            frag_t yf = tr_frag<T>(yrow + 16 * j, yrow + 16 * j + 4 * kLdsRow);
-#pragma unroll
-            for (int m = 0; m < G; m++)
-              if (bid[m] >= 0) acc[m][j] = M::run(yf, xf[m][s2], acc[m][j]);
-          }
+          for (int j = 0; j < 4; j++) yf[s2][j] = tr_frag<T>(yrow + 16 * j, yrow + 16 * j + 4 * kLdsRow);
         }
+#pragma unroll
+        for (int m = 0; m < G; m++)
+          if (bid[m] >= 0) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+              for (int j = 0; j < 4; j++) acc[m][j] = M::run(yf[s2][j], xf[m][s2], acc[m][j]);
+          }
+        // refill this ring slot only now: its old contents are dead, so the loads can land in the same registers
+        // (issued earlier, the compiler would rotate registers at the loop edge and wait for every load to do so)
+        issue(st, e + RING < last ? e + RING : last);
       }
     }
   }
