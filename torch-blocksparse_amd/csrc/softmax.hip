@@ -51,9 +51,13 @@ template <int LPR> __device__ __forceinline__ float row_sum(float v) {
   return v;
 }
 
+// 16-bit types work in the log2 domain: the logits are built as x * (scale * log2 e) + mask * log2 e, so that the
+// exponential is a bare v_exp_f32 of a difference.  fp32 keeps the natural domain and the accurate expf.
+constexpr float kLog2e = 1.44269504088896340736f;
+template <typename T> __device__ __forceinline__ float logit_unit() { return sizeof(T) == 4 ? 1.f : kLog2e; }
 template <typename T> __device__ __forceinline__ float exp_sub(float x, float mx) {
   if constexpr (sizeof(T) == 4) return expf(x - mx);
-  else return __builtin_amdgcn_exp2f((x - mx) * 1.44269504088896340736f);
+  else return __builtin_amdgcn_exp2f(x - mx);
 }
 
 struct FwdArgs {
@@ -72,7 +76,8 @@ template <typename T, int BLOCK> struct Unit {
     typedef Geo<T, BLOCK> GE;
     const int64_t n_wg = (n_units + kWavesPerGroup - 1) / kWavesPerGroup;
     const int64_t wg = xcd_remap(blockIdx.x, n_wg);
-    const int64_t u = wg * kWavesPerGroup + (threadIdx.x >> 6);
+    // the wavefront index is uniform: as a scalar it keeps row sizes, block ids and base addresses out of the VALU
+    const int64_t u = wg * kWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     ok = u < n_units;
     const int lane = threadIdx.x & 63;
     const int g = (int)(u % GE::G);
@@ -91,34 +96,39 @@ __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK
   const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
   const int64_t grow = (int64_t)brow * BLOCK + u.rxm;    // row in the dense matrix
   const int64_t gcol = (int64_t)bcol * BLOCK + u.col;    // lane's first column in the dense matrix
+  const float unit = logit_unit<T>();
+  const float sc = a.scale * unit;
   Pack<T, EV> px;
   px.load(x);
 #pragma unroll
-  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * a.scale;                          // softmax.py:112-116
+  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;                               // softmax.py:112-116
   if (a.rpe) {                                                                               // :118-120, address :50-55
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
 #pragma unroll
-    for (int e = 0; e < EV; e++) fx[e] += to_float(p.e[e]);
+    for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
   }
+  // the mask modes are uniform: branch once per block, not once per element
   if (a.kpm) {                                                                               // :122-124, address :60-62
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol);
+    if (a.kpm_mul) {                                                                         // :104-106
 #pragma unroll
-    for (int e = 0; e < EV; e++) {
-      float m = to_float(p.e[e]);
-      if (a.kpm_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                       // :104-106
-      fx[e] += m;
+      for (int e = 0; e < EV; e++) fx[e] += (to_float(p.e[e]) == 0.f) ? -INFINITY : 0.f;
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
     }
   }
   if (a.attn) {                                                                              // :126-128, address :67-70
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);
+    if (a.attn_mul) {                                                                        // :108-110
 #pragma unroll
-    for (int e = 0; e < EV; e++) {
-      float m = to_float(p.e[e]);
-      if (a.attn_mul) m = (m == 0.f) ? -INFINITY : 0.f;                                      // :108-110
-      fx[e] += m;
+      for (int e = 0; e < EV; e++) fx[e] += (to_float(p.e[e]) == 0.f) ? -INFINITY : 0.f;
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
     }
   }
 }
@@ -140,11 +150,12 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   const int HR = a.H * a.R;
   Unit<T, BLOCK> u(a.n_units, HR);
   if (!u.ok) return;
-  const int size = a.lut[2 * u.hr + 0];                 // header (size, offset), softmax.py:30-32
-  const int offset = a.lut[2 * u.hr + 1];
+  const table_ptr lut = as_table(a.lut);
+  const int size = lut[2 * u.hr + 0];                   // header (size, offset), softmax.py:30-32
+  const int offset = lut[2 * u.hr + 1];
   const int head = u.hr / a.R, brow = u.hr % a.R;       // = the table's (row, head) fields of every block of this row
   if (size <= 0) return;
-  const int32_t *core = a.lut + offset;
+  const table_ptr core = lut + offset;
   if constexpr (NB > 0) {
     float fx[NB][GE::EV];
     int32_t bid[NB];
@@ -216,10 +227,11 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
   const int HR = a.H * a.R;
   Unit<T, BLOCK> u(a.n_units, HR);
   if (!u.ok) return;
-  const int size = a.lut[2 * u.hr + 0];
-  const int offset = a.lut[2 * u.hr + 1];
+  const table_ptr lut = as_table(a.lut);
+  const int size = lut[2 * u.hr + 0];
+  const int offset = lut[2 * u.hr + 1];
   if (size <= 0) return;
-  const int32_t *core = a.lut + offset;
+  const table_ptr core = lut + offset;
   const T *yb = reinterpret_cast<const T *>(a.y) + (int64_t)u.z * a.y_sz + u.rxm * BLOCK + u.col;
   T *db = reinterpret_cast<T *>(a.dy) + (int64_t)u.z * a.dy_sz + u.rxm * BLOCK + u.col;
   if constexpr (NB > 0) {
