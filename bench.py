@@ -30,10 +30,10 @@ MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 # the same counter reads for the calibration copy of known size (profiles/traffic_attention_seq4096.txt).  None = not
 # measured for this build of the kernel.
 TRAFFIC_BYTES = {
-    'sdd_fwd  q.k^T': 134815882 + 268435456, 'sdd_bwd  do.v^T': 134815882 + 268435456,
-    'dsd_fwd  p.v': 336633312 + 67108864, 'dsd_bwd  ds.k': 336633312 + 67108864,
-    'dsd_bwd  p^T.do': 402584314 + 67108864, 'dds_bwd  (q^T.ds)^T': 402584314 + 67108864,
-    'softmax_fwd': 269257126 + 268435456, 'softmax_bwd': 537486370 + 268435456,
+    'sdd_fwd  q.k^T': 140210325 + 268435464, 'sdd_bwd  do.v^T': 140210325 + 268435464,
+    'dsd_fwd  p.v': 342657616 + 67108864, 'dsd_bwd  ds.k': 342657616 + 67108864,
+    'dsd_bwd  p^T.do': 428109030 + 67108864, 'dds_bwd  (q^T.ds)^T': 428109030 + 67108864,
+    'softmax_fwd': 269876117 + 268435456, 'softmax_bwd': 538087015 + 268435456,
 }
 
 
