@@ -79,6 +79,74 @@ def test_benchmark_chain_block64_seq4096_small_batch():
     assert_close(vg.grad, rv, torch.float16, 'dv')
 
 
+def test_long_context_bigbird_chain_reduced():
+    # config 4 at reduced size: BigBird-style layout (window 3 + 2 global + 3 random blocks, causal), block 64, fp16,
+    # additive relative-position embedding given per block pair and expanded to [B, H, L, L] with stride-0 views,
+    # causal attention mask in 'mul' mode; forward + backward against the dense oracle
+    torch.manual_seed(12)
+    B, H, L, dh, block = 2, 3, 1024, 64, 64
+    nb = L // block
+    lay = tb.bigbird_layout(H, nb, 3, 2, 3, seed=3, causal=True)
+    q, k, v, do = [torch.randn(B, H, L, dh).half() for _ in range(4)]
+    rpe_blocks = (0.1 * torch.randn(nb)).half()                     # one value per block distance
+    dist = (torch.arange(nb)[:, None] - torch.arange(nb)[None, :]).abs()
+    rpe_bb = rpe_blocks[dist]                                       # [nb, nb]
+    rpe = rpe_bb.repeat_interleave(block, 0).repeat_interleave(block, 1)[None, None].expand(B, H, L, L)   # strides 0, 0
+    causal = torch.tril(torch.ones(L, L)).half()
+    ro, rq, rk, rv = D.attention(q, k, v, lay, block, 0.125, rpe=rpe, attn_mask=causal, attn_mask_mode='mul', do=do)
+    sdd = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=True)
+    dsd = tb.MatMul(lay, block, 'dsd')
+    sm = tb.Softmax(lay, block)
+    qg, kg, vg = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+    rpe_dev = rpe_bb.to(DEV).repeat_interleave(block, 0).repeat_interleave(block, 1)[None, None].expand(B, H, L, L)
+    assert rpe_dev.stride(0) == 0 and rpe_dev.stride(1) == 0
+    p = sm(sdd(qg, kg), scale=0.125, rpe=rpe_dev, attn_mask=causal.to(DEV), attn_mask_mode='mul')
+    o = dsd(p, vg)
+    o.backward(do.to(DEV))
+    assert_close(o, ro, torch.float16, 'out')
+    assert_close(qg.grad, rq, torch.float16, 'dq')
+    assert_close(kg.grad, rk, torch.float16, 'dk')
+    assert_close(vg.grad, rv, torch.float16, 'dv')
+
+
+def test_head_dim_128_and_non_contiguous_inputs():
+    # head_dim 128 (two 64-wide tiles, sdd reduction of 128) and q/k/v given as strided views of a packed projection
+    torch.manual_seed(13)
+    B, H, L, dh, block = 2, 2, 512, 128, 64
+    lay = tb.sparse_transformer_layout(H, L // block, 2, 4, True)
+    qkv = torch.randn(B, L, 3, H, dh).half()
+    q, k, v = [qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3)]          # [B, H, L, dh], not contiguous
+    do = torch.randn(B, H, L, dh).half()
+    ro, rq, rk, rv = D.attention(q, k, v, lay, block, dh ** -0.5, do=do)
+    mod = tb.SparseSelfAttention(tb.SparsityConfig(mode='fixed', block=64, stride=128, attention='unidirectional'))
+    lay2 = tb.fixed_layout(H, L // block, 'fixed', 2, 'unidirectional', 1, 1)
+    ro2, rq2, rk2, rv2 = D.attention(q, k, v, lay2, block, dh ** -0.5, do=do)
+    qkv_dev = qkv.to(DEV).requires_grad_(True)
+    qd, kd, vd = [qkv_dev[:, :, i].permute(0, 2, 1, 3) for i in range(3)]
+    o = mod(qd, kd, vd)
+    o.backward(do.to(DEV))
+    assert_close(o, ro2, torch.float16, 'out')
+    g = qkv_dev.grad
+    assert_close(g[:, :, 0].permute(0, 2, 1, 3), rq2, torch.float16, 'dq')
+    assert_close(g[:, :, 1].permute(0, 2, 1, 3), rk2, torch.float16, 'dk')
+    assert_close(g[:, :, 2].permute(0, 2, 1, 3), rv2, torch.float16, 'dv')
+
+
+def test_bench_flag_and_second_stream():
+    torch.manual_seed(14)
+    lay = tb.sparse_transformer_layout(2, 8, 2, 4, True)
+    op = tb.MatMul(lay, 64, 'sdd', trans_b=True, bench=True)
+    a, b = [torch.randn(1, 2, 512, 64, device=DEV, dtype=torch.float16) for _ in range(2)]
+    c = op(a, b)
+    assert op.time_c is not None and op.time_c > 0
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        c2 = tb.MatMul(lay, 64, 'sdd', trans_b=True)(a, b)
+    s.synchronize()
+    assert torch.equal(c, c2)
+
+
 def test_specialised_and_general_kernels_agree(monkeypatch):
     # block 64 / fp16 / head_dim 64 takes specialised kernels; the general ones must give the same numbers
     torch.manual_seed(9)
