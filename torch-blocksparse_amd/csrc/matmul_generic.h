@@ -3,9 +3,10 @@
 //
 // Replaces the reference's single Triton-C kernel with its SDD / DSD / DDS branches (matmul.py:6-205).
 // Structure: a workgroup of four wavefronts owns one output tile; both operand tiles are staged through LDS
-// in a reduction-contiguous layout (rows of TK elements plus padding) so that every MFMA operand is one
-// 16-byte LDS read whatever the operand's orientation in memory; an operand stored with the reduction
-// dimension strided is transposed while it is written to LDS.  Global loads for step s+1 are issued before
+// An operand whose reduction dimension is contiguous in memory sits in LDS as rows of TK elements plus padding
+// and every MFMA operand is one 16-byte LDS read; an operand stored with the reduction dimension strided sits in
+// LDS as it lies in memory and is read with the transposing LDS load (16-bit types; 32-bit ones are transposed
+// while they are written).  Global loads for step s+1 are issued before
 // the MFMAs of step s (two LDS buffers, one barrier per step).  fp32 accumulation in 16x16 MFMA tiles.
 //
 // "xsd" is the kernel behind both dsd and dds: dds is dsd with the roles of rows and columns exchanged
@@ -16,8 +17,9 @@
 namespace bsp {
 
 // ---------------------------------------------------------------------------------------------------------
-// 16x16 MFMA per element type.  Lane l supplies row (l % 16) of its operand, reduction indices
-// (l / 16) * KV .. + KV - 1; the result tile has row 4 * (l / 16) + e, column l % 16 in element e.
+// MFMA per element type and tile size MS (16 or 32).  Lane l supplies row (l % MS) of its operand, reduction
+// indices (l / MS) * KV .. + KV - 1.  Result: MS = 16 -> element e is (row 4*(l/16) + e, column l % 16);
+// MS = 32 -> element 4*g + e is (row 8*g + 4*(l/32) + e, column l % 32).
 // ---------------------------------------------------------------------------------------------------------
 template <typename T> struct Mma16;
 template <> struct Mma16<f16> {
@@ -36,12 +38,37 @@ template <> struct Mma16<float> {
   static __device__ __forceinline__ f32x4 run(frag_t a, frag_t b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
 };
 
+template <typename T, int MS> struct Mma;
+template <typename T> struct Mma<T, 16> : Mma16<T> {
+  static constexpr int NACC = 4;
+  typedef f32x4 acc_t;
+};
+template <> struct Mma<f16, 32> {
+  static constexpr int KSTEP = 16, KV = 8, NACC = 16;
+  typedef f16x8 frag_t;
+  typedef f32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(frag_t a, frag_t b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mma<bf16, 32> {
+  static constexpr int KSTEP = 16, KV = 8, NACC = 16;
+  typedef bf16x8 frag_t;
+  typedef f32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(frag_t a, frag_t b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+template <> struct Mma<float, 32> {
+  static constexpr int KSTEP = 2, KV = 1, NACC = 16;
+  typedef float frag_t;
+  typedef f32x16 acc_t;
+  static __device__ __forceinline__ acc_t run(frag_t a, frag_t b, acc_t c) { return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0); }
+};
+
 template <typename T> struct TileK { static constexpr int TK = 64 / sizeof(T), PAD = 16 / sizeof(T); };  // 64-byte rows + 16 bytes
 
 // ---------------------------------------------------------------------------------------------------------
 // One operand tile: ROWS x TK, fetched by NT threads in 16-byte chunks, kept in registers until the LDS
-// buffer is free.  View::ptr_k(row, k) -> address of elements (row, k..k+VE-1) or nullptr (zero fill);
-// View::ptr_r(row, k) -> address of elements (row..row+VE-1, k) or nullptr.
+// buffer is free.  View::step(k0) -> the part of the addressing that is uniform for the reduction step starting at
+// k0; View::ptr_k(step, row, k) -> address of elements (row, k0+k .. k0+k+VE-1) or nullptr (zero fill);
+// View::ptr_r(step, row, k) -> address of elements (row..row+VE-1, k0+k) or nullptr.
 // ---------------------------------------------------------------------------------------------------------
 template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   static constexpr int TK = TileK<T>::TK, LDK = TK + TileK<T>::PAD;
@@ -50,19 +77,27 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   static constexpr int ITER = (NCH + NT - 1) / NT;
   static constexpr int CPR = TK / VE;    // chunks per row when the reduction is contiguous
   static constexpr int RCH = ROWS / VE;  // chunks per reduction index otherwise
+  // A 16-bit operand stored with the reduction dimension strided is kept in LDS as it lies in memory, [TK][ROWS + 8],
+  // and handed to the MFMA through the transposing LDS read; a 32-bit one is transposed while it is written.
+  static constexpr bool TR = !KCONTIG && sizeof(T) == 2;
+  static constexpr int LDR = ROWS + 8;
+  static constexpr int ELEMS = TR ? TK * LDR : ROWS * LDK;
   u32x4 reg[ITER];
+  bool ok[ITER];
 
+  // Every thread issues exactly ITER loads whatever the tile holds (chunks outside the operand read a dummy line
+  // and are zeroed afterwards): with a fixed count the wait before a stage is consumed is exact.
   template <class View> __device__ __forceinline__ void load(const View &v, int k0, int tid) {
+    const auto st = v.step(k0);   // what is uniform for the whole reduction step (table look-ups), kept scalar
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
-      const int c = tid + it * NT;
-      const T *p = nullptr;
-      if (NCH % NT == 0 || c < NCH) {
-        if constexpr (KCONTIG) p = v.ptr_k(c / CPR, k0 + (c % CPR) * VE);
-        else p = v.ptr_r((c % RCH) * VE, k0 + c / RCH);
-      }
-      u32x4 z = {0u, 0u, 0u, 0u};
-      reg[it] = p ? *reinterpret_cast<const u32x4 *>(p) : z;
+      int c = tid + it * NT;
+      if (NCH % NT != 0 && c >= NCH) c = NCH - 1;
+      const T *p;
+      if constexpr (KCONTIG) p = v.ptr_k(st, c / CPR, (c % CPR) * VE);
+      else p = v.ptr_r(st, (c % RCH) * VE, c / RCH);
+      ok[it] = p != nullptr;            // zero-filling happens when the stage is consumed, not here: a use of the loaded
+      reg[it] = *reinterpret_cast<const u32x4 *>(p ? p : v.base);   // value right away would make the wait for it immediate
     }
   }
   __device__ __forceinline__ void store(T *S, int tid) const {
@@ -70,16 +105,37 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
     for (int it = 0; it < ITER; it++) {
       const int c = tid + it * NT;
       if (NCH % NT == 0 || c < NCH) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        const u32x4 val = ok[it] ? reg[it] : z;
         if constexpr (KCONTIG) {
-          *reinterpret_cast<u32x4 *>(S + (c / CPR) * LDK + (c % CPR) * VE) = reg[it];
+          *reinterpret_cast<u32x4 *>(S + (c / CPR) * LDK + (c % CPR) * VE) = val;
+        } else if constexpr (TR) {
+          *reinterpret_cast<u32x4 *>(S + (c / RCH) * LDR + (c % RCH) * VE) = val;
         } else {
           union { u32x4 raw; T e[VE]; } u;
-          u.raw = reg[it];
+          u.raw = val;
           const int row0 = (c % RCH) * VE, k = c / RCH;
 #pragma unroll
           for (int e = 0; e < VE; e++) S[(row0 + e) * LDK + k] = u.e[e];
         }
       }
+    }
+  }
+  // operand fragment of an MS-row MFMA tile starting at tile row `row0`, reduction step kk (KSTEP wide)
+  template <int MS, class M> __device__ __forceinline__ static typename M::frag_t frag(const T *S, int row0, int kk, int lane) {
+    if constexpr (TR) {
+      typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+      const int t = lane & 15, gi = lane >> 4;
+      // MS 16: the four 16-lane groups are the four reduction groups; MS 32: two row halves x two reduction groups
+      const int kq = (MS == 16) ? gi : (gi >> 1), rh = (MS == 16) ? 0 : 16 * (gi & 1);
+      const T *p = S + (kk * M::KSTEP + 8 * kq + (t >> 2)) * LDR + row0 + rh + 4 * (t & 3);
+      s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p);
+      s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 4 * LDR));
+      typedef short s16x8 __attribute__((ext_vector_type(8)));
+      s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(typename M::frag_t, v);
+    } else {
+      return *reinterpret_cast<const typename M::frag_t *>(S + (row0 + lane % MS) * LDK + (lane / MS) * M::KV + kk * M::KSTEP);
     }
   }
 };
@@ -92,12 +148,14 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
 template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_KCONTIG, bool OUT_NCONTIG> struct TileGemm {
   static constexpr int NT = 64 * WGM * WGN;
   static constexpr int TK = TileK<T>::TK, LDK = TK + TileK<T>::PAD;
-  static constexpr int RM = TM / (16 * WGM), RN = TN / (16 * WGN);
-  static constexpr int X_ELEMS = TM * LDK, Y_ELEMS = TN * LDK;
-  static constexpr int SMEM_BYTES = 2 * (X_ELEMS + Y_ELEMS) * (int)sizeof(T);
-  typedef Mma16<T> M;
+  // 32x32 MFMA tiles when a wavefront's region allows it (half the LDS operand traffic per flop), 16x16 otherwise
+  static constexpr int MS = (TM / WGM >= 32 && TN / WGN >= 32) ? 32 : 16;
+  static constexpr int RM = TM / (MS * WGM), RN = TN / (MS * WGN);
+  typedef Mma<T, MS> M;
   typedef TileLoader<T, TM, NT, X_KCONTIG> XL;
   typedef TileLoader<T, TN, NT, Y_KCONTIG> YL;
+  static constexpr int X_ELEMS = (XL::ELEMS + 7) & ~7, Y_ELEMS = (YL::ELEMS + 7) & ~7;
+  static constexpr int SMEM_BYTES = 2 * (X_ELEMS + Y_ELEMS) * (int)sizeof(T);
 
   // ksteps = number of TK-wide reduction steps.  Store(m, n, vals): vals[4] run along n (OUT_NCONTIG) or m.
   template <class XView, class YView, class Store>
@@ -106,57 +164,66 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
     const int wm = wave / WGN, wn = wave % WGN;
     T *Xs[2] = {smem, smem + X_ELEMS + Y_ELEMS};
     T *Ys[2] = {smem + X_ELEMS, smem + 2 * X_ELEMS + Y_ELEMS};
-    f32x4 acc[RM][RN];
+    typename M::acc_t acc[RM][RN];
 #pragma unroll
     for (int i = 0; i < RM; i++)
 #pragma unroll
-      for (int j = 0; j < RN; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    XL xl;
-    YL yl;
-    if (ksteps > 0) {
-      xl.load(xv, 0, tid);
-      yl.load(yv, 0, tid);
-      xl.store(Xs[0], tid);
-      yl.store(Ys[0], tid);
+      for (int j = 0; j < RN; j++)
+#pragma unroll
+        for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
+    // Register ring of NS stages: global loads run NS - 1 reduction steps ahead of the MFMAs; two LDS buffers, one
+    // barrier per step.  The loop runs whole rounds of NS steps; steps past the end load zeros and skip the MFMAs.
+    constexpr int NS = 4;
+    XL xl[NS];
+    YL yl[NS];
+#pragma unroll
+    for (int u = 0; u < NS; u++) {
+      xl[u].load(xv, u * TK, tid);
+      yl[u].load(yv, u * TK, tid);
     }
-    __syncthreads();
-    for (int s = 0; s < ksteps; s++) {
-      const int cur = s & 1;
-      if (s + 1 < ksteps) {
-        xl.load(xv, (s + 1) * TK, tid);
-        yl.load(yv, (s + 1) * TK, tid);
-      }
-      const T *xs = Xs[cur] + (wm * RM * 16 + (lane & 15)) * LDK + (lane >> 4) * M::KV;
-      const T *ys = Ys[cur] + (wn * RN * 16 + (lane & 15)) * LDK + (lane >> 4) * M::KV;
+    for (int s0 = 0; s0 < ksteps; s0 += NS) {
 #pragma unroll
-      for (int kk = 0; kk < TK / M::KSTEP; kk++) {
-        typename M::frag_t xf[RM], yf[RN];
+      for (int u = 0; u < NS; u++) {
+        const int s = s0 + u;
+        const int cur = u & 1;
+        xl[u].store(Xs[cur], tid);   // this buffer was last read two steps ago, before the previous barrier
+        yl[u].store(Ys[cur], tid);
+        __syncthreads();
+        if (s < ksteps) {
 #pragma unroll
-        for (int i = 0; i < RM; i++) xf[i] = *reinterpret_cast<const typename M::frag_t *>(xs + i * 16 * LDK + kk * M::KSTEP);
+          for (int kk = 0; kk < TK / M::KSTEP; kk++) {
+            typename M::frag_t xf[RM], yf[RN];
 #pragma unroll
-        for (int j = 0; j < RN; j++) yf[j] = *reinterpret_cast<const typename M::frag_t *>(ys + j * 16 * LDK + kk * M::KSTEP);
+            for (int i = 0; i < RM; i++) xf[i] = XL::template frag<MS, M>(Xs[cur], (wm * RM + i) * MS, kk, lane);
 #pragma unroll
-        for (int i = 0; i < RM; i++)
+            for (int j = 0; j < RN; j++) yf[j] = YL::template frag<MS, M>(Ys[cur], (wn * RN + j) * MS, kk, lane);
 #pragma unroll
-          for (int j = 0; j < RN; j++) {
-            if constexpr (OUT_NCONTIG) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // result rows = n, column = m
-            else acc[i][j] = M::run(xf[i], yf[j], acc[i][j]);                          // result rows = m, column = n
+            for (int i = 0; i < RM; i++)
+#pragma unroll
+              for (int j = 0; j < RN; j++) {
+                if constexpr (OUT_NCONTIG) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // result rows = n, column = m
+                else acc[i][j] = M::run(xf[i], yf[j], acc[i][j]);                          // result rows = m, column = n
+              }
           }
+        }
+        xl[u].load(xv, (s + NS) * TK, tid);   // refill the slot only after its contents are dead
+        yl[u].load(yv, (s + NS) * TK, tid);
       }
-      if (s + 1 < ksteps) {
-        xl.store(Xs[cur ^ 1], tid);   // the other buffer was last read before the previous barrier
-        yl.store(Ys[cur ^ 1], tid);
-      }
-      __syncthreads();
     }
+    // a lane's values come in groups of 4 consecutive result rows: row 4*(lane/16) (MS 16) or 8*g + 4*(lane/32) (MS 32)
 #pragma unroll
     for (int i = 0; i < RM; i++)
 #pragma unroll
-      for (int j = 0; j < RN; j++) {
-        const int m0 = (wm * RM + i) * 16, n0 = (wn * RN + j) * 16;
-        if constexpr (OUT_NCONTIG) store(m0 + (lane & 15), n0 + 4 * (lane >> 4), acc[i][j]);
-        else store(m0 + 4 * (lane >> 4), n0 + (lane & 15), acc[i][j]);
-      }
+      for (int j = 0; j < RN; j++)
+#pragma unroll
+        for (int g4 = 0; g4 < M::NACC / 4; g4++) {
+          const f32x4 v = {acc[i][j][4 * g4 + 0], acc[i][j][4 * g4 + 1], acc[i][j][4 * g4 + 2], acc[i][j][4 * g4 + 3]};
+          const int rr = (MS == 16) ? 4 * (lane >> 4) : 8 * g4 + 4 * (lane >> 5);
+          const int cc = lane % MS;
+          const int m0 = (wm * RM + i) * MS, n0 = (wn * RN + j) * MS;
+          if constexpr (OUT_NCONTIG) store(m0 + cc, n0 + rr, v);
+          else store(m0 + rr, n0 + cc, v);
+        }
   }
 };
 
@@ -187,15 +254,21 @@ struct SddArgs {
 };
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
-  const T *base; int64_t ld; int K; int idx[PACK];
+  const T *base; int64_t ld; int K; int idx[PACK];   // base doubles as the dummy address of out-of-range chunks
+  struct Step { int k0; };
+  __device__ __forceinline__ Step step(int k0) const { return Step{k0}; }
   __device__ __forceinline__ int blk(int row) const {
     int r = idx[0];
 #pragma unroll
     for (int p = 1; p < PACK; p++) r = (row / BLOCK == p) ? idx[p] : r;
     return r * BLOCK + row % BLOCK;
   }
-  __device__ __forceinline__ const T *ptr_k(int row, int k) const { return k < K ? base + (int64_t)blk(row) * ld + k : nullptr; }
-  __device__ __forceinline__ const T *ptr_r(int row, int k) const { return k < K ? base + (int64_t)k * ld + blk(row) : nullptr; }
+  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {
+    return st.k0 + k < K ? base + (int64_t)blk(row) * ld + st.k0 + k : nullptr;
+  }
+  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {
+    return st.k0 + k < K ? base + (int64_t)(st.k0 + k) * ld + blk(row) : nullptr;
+  }
 };
 
 template <int T_> struct SddShape { static constexpr int WG = T_ >= 32 ? 2 : 1; };
@@ -209,7 +282,7 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
   const int64_t w = xcd_remap(blockIdx.x, n_wg);
   const int z = (int)(w / g.n_groups);
   const int64_t grp = w % g.n_groups;
-  const int32_t *e = g.lut + grp * (PACK * PACK * 4);
+  const table_ptr e = as_table(g.lut) + grp * (PACK * PACK * 4);
   const int h = e[0];
   SddView<T, BLOCK, PACK, A_KCONTIG> av;
   SddView<T, BLOCK, PACK, B_KCONTIG> bv;
@@ -234,7 +307,7 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
 // ---------------------------------------------------------------------------------------------------------
 // xsd: out[col*BLOCK + m, n] = sum over the blocks t of one table segment  S_t(m, :) . D(n, pos_t + :)
 // (dsd: S = op(A) blocks, D = op(B)^T rows; dds: S = op(B)^T blocks, D = op(A) rows).
-// One workgroup per (segment, 64-wide tile of the dense free dimension, batch).  Reads the segment header
+// One workgroup per (segment, tile of the dense free dimension, batch).  Reads the segment header
 // of the reference table (offset, length, column, depth; matmul.py:57-63) and the per-block positions.
 // ---------------------------------------------------------------------------------------------------------
 struct XsdArgs {
@@ -242,40 +315,75 @@ struct XsdArgs {
   int Z, NF;                            // batch, size of the dense free dimension
   int64_t sp_sz, dn_sz, dn_sh, ldd, out_sz, out_sh, ldo;
   const int32_t *lut; const int32_t *plan; int width; int div2;   // div2 = 2 * block / step of the table
-  int n_tiles;
+  int n_tiles;                          // 64-wide tiles of the free dimension (specialised kernels)
   const int32_t *gplan; int n_pgroups; int lines;   // optional group plan, its groups, lines (block-rows or -columns) per head
 };
 
+// A reduction step of TK elements lies inside one block (BLOCK >= TK) or covers TK / BLOCK whole blocks.
+template <typename T, int BLOCK> struct StepBlocks { static constexpr int TK = TileK<T>::TK, NB = TK > BLOCK ? TK / BLOCK : 1; };
+
 template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m, k) of the segment's blocks
-  const T *base; const int32_t *plan; int nblk;
-  __device__ __forceinline__ const T *blk(int k) const {
-    const int ord = k / BLOCK;
-    return ord < nblk ? base + (int64_t)plan[2 * ord + 1] * (BLOCK * BLOCK) : nullptr;
+  const T *base; table_ptr plan; int nblk;
+  static constexpr int NB = StepBlocks<T, BLOCK>::NB;
+  struct Step { const T *blk[NB]; int kin; };                      // block base pointers (nullptr past the end), offset inside
+  __device__ __forceinline__ Step step(int k0) const {
+    Step st;
+    st.kin = k0 % BLOCK;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+      const int ord = k0 / BLOCK + i;
+      st.blk[i] = ord < nblk ? base + (int64_t)plan[2 * ord + 1] * (BLOCK * BLOCK) : nullptr;
+    }
+    return st;
   }
-  __device__ __forceinline__ const T *ptr_k(int row, int k) const {   // stored [m][k]
-    const T *b = blk(k);
-    return b ? b + row * BLOCK + k % BLOCK : nullptr;
+  __device__ __forceinline__ const T *pick(const Step &st, int k) const {
+    const T *b = st.blk[0];
+#pragma unroll
+    for (int i = 1; i < NB; i++) b = (k / BLOCK == i) ? st.blk[i] : b;
+    return b;
   }
-  __device__ __forceinline__ const T *ptr_r(int row, int k) const {   // stored [k][m]
-    const T *b = blk(k);
-    return b ? b + (k % BLOCK) * BLOCK + row : nullptr;
+  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [m][k]
+    const T *b = pick(st, k);
+    return b ? b + row * BLOCK + (st.kin + k) % BLOCK : nullptr;
+  }
+  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {   // stored [k][m]
+    const T *b = pick(st, k);
+    return b ? b + ((st.kin + k) % BLOCK) * BLOCK + row : nullptr;
   }
 };
 
 template <typename T, int BLOCK> struct DenseView {                   // element (n, k): dense row/col n, reduction position k
-  const T *base; const int32_t *plan; int nblk; int64_t ld; int n0, NF;
-  __device__ __forceinline__ int64_t pos(int k) const { return (int64_t)plan[2 * (k / BLOCK)] + k % BLOCK; }
-  __device__ __forceinline__ const T *ptr_k(int row, int k) const {   // stored [n][k]
-    return (n0 + row < NF && k / BLOCK < nblk) ? base + (int64_t)(n0 + row) * ld + pos(k) : nullptr;
+  const T *base; table_ptr plan; int nblk; int64_t ld; int n0, NF;
+  static constexpr int NB = StepBlocks<T, BLOCK>::NB;
+  struct Step { int64_t pos[NB]; };                                   // position of each block in the dense operand, -1 past the end
+  __device__ __forceinline__ Step step(int k0) const {
+    Step st;
+#pragma unroll
+    for (int i = 0; i < NB; i++) {
+      const int ord = k0 / BLOCK + i;
+      st.pos[i] = ord < nblk ? (int64_t)plan[2 * ord] + k0 % BLOCK : -1;
+    }
+    return st;
   }
-  __device__ __forceinline__ const T *ptr_r(int row, int k) const {   // stored [k][n]
-    return (n0 + row < NF && k / BLOCK < nblk) ? base + pos(k) * ld + n0 + row : nullptr;
+  __device__ __forceinline__ int64_t pick(const Step &st, int k) const {
+    int64_t p = st.pos[0];
+#pragma unroll
+    for (int i = 1; i < NB; i++) p = (k / BLOCK == i) ? st.pos[i] : p;
+    return p;
+  }
+  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [n][k]
+    const int64_t p = pick(st, k);
+    return (n0 + row < NF && p >= 0) ? base + (int64_t)(n0 + row) * ld + p + k % BLOCK : nullptr;
+  }
+  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {   // stored [k][n]
+    const int64_t p = pick(st, k);
+    return (n0 + row < NF && p >= 0) ? base + (p + k % BLOCK) * ld + n0 + row : nullptr;
   }
 };
 
 template <int BLOCK> struct XsdShape {
-  static constexpr int TN = 64;
-  static constexpr int WGM = BLOCK >= 32 ? 2 : 1;
+  static constexpr int TN = BLOCK >= 32 ? 128 : 64;      // tile of the dense free dimension
+  static constexpr int WGM = BLOCK >= 64 ? 2 : 1;        // 32 -> 1x4 wavefronts of 32x32; 64 -> 2x2 of 32x64; 128 -> 2x2 of 64x64
   static constexpr int WGN = 4 / WGM;
 };
 
@@ -284,12 +392,15 @@ __global__ void __launch_bounds__(256) k_xsd(XsdArgs g) {
   typedef XsdShape<BLOCK> S;
   typedef TileGemm<T, BLOCK, S::TN, S::WGM, S::WGN, !SP_TRANS, DN_KCONTIG, OUT_NCONTIG> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  const int64_t per_z = (int64_t)g.width * g.n_tiles;
+  const int n_tiles = (g.NF + S::TN - 1) / S::TN;
+  const int64_t per_z = (int64_t)g.width * n_tiles;
   const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
   const int z = (int)(w / per_z);
-  const int seg = (int)((w % per_z) / g.n_tiles);
-  const int nt = (int)(w % g.n_tiles);
-  const int32_t *hd = g.lut + 6 * (int64_t)seg;
+  // segment index fastest: consecutive workgroups (same XCD after the re-numbering) walk the segments of a head
+  // against one slab of TN columns of the dense operand, which then stays in L2 between its uses
+  const int nt = (int)((w % per_z) / g.width);
+  const int seg = (int)((w % per_z) % g.width);
+  const table_ptr hd = as_table(g.lut) + 6 * (int64_t)seg;
   const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];
   const int nblk = seglen / BLOCK;
   if (nblk == 0) {
@@ -299,7 +410,7 @@ __global__ void __launch_bounds__(256) k_xsd(XsdArgs g) {
   }
   const int t0 = (offset - 6 * g.width) / g.div2;   // first block of the segment in table order
   SparseView<T, BLOCK, SP_TRANS> sv;
-  sv.base = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz; sv.plan = g.plan + 2 * (int64_t)t0; sv.nblk = nblk;
+  sv.base = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz; sv.plan = as_table(g.plan) + 2 * (int64_t)t0; sv.nblk = nblk;
   DenseView<T, BLOCK> dv;
   dv.base = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh; dv.plan = sv.plan; dv.nblk = nblk; dv.ld = g.ldd;
   dv.n0 = nt * S::TN; dv.NF = g.NF;
@@ -347,7 +458,7 @@ template <typename T> int launch_sdd(const SddArgs &g, int block, int pack, bool
 
 template <typename T, int BLOCK> int launch_xsd_b(const XsdArgs &g, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
   typedef XsdShape<BLOCK> S;
-  const int64_t n_wg = (int64_t)g.width * g.n_tiles * g.Z;
+  const int64_t n_wg = (int64_t)g.width * ((g.NF + S::TN - 1) / S::TN) * g.Z;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   dim3 grid((unsigned)n_wg), blockdim(256);
