@@ -135,11 +135,11 @@ def main():
         ('sdd_fwd  q.k^T', k_sdd_fwd, flops_mm, mm_bytes),
         ('softmax_fwd', k_softmax_fwd, 0.0, 2 * x_bytes + kpm.numel() * es),
         ('dsd_fwd  p.v', k_dsd_fwd, flops_mm, mm_bytes),
-        ('sdd_bwd  do.v^T', k_sdd_bwd, flops_mm, mm_bytes),
         ('dsd_bwd  p^T.do', k_dsd_bwd_t, flops_mm, mm_bytes),
+        ('sdd_bwd  do.v^T', k_sdd_bwd, flops_mm, mm_bytes),
         ('softmax_bwd', k_softmax_bwd, 0.0, 3 * x_bytes),
-        ('dsd_bwd  ds.k', k_dsd_bwd, flops_mm, mm_bytes),
         ('dds_bwd  (q^T.ds)^T', k_dds_bwd, flops_mm, mm_bytes),
+        ('dsd_bwd  ds.k', k_dsd_bwd, flops_mm, mm_bytes),
         ('calibration_copy', k_copy, 0.0, 2 * x_bytes),
     ]
     reps = max(args.steps, 10)

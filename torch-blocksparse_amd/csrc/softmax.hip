@@ -82,7 +82,10 @@ template <typename T, int BLOCK> struct Unit {
     const int lane = threadIdx.x & 63;
     const int g = (int)(u % GE::G);
     const int64_t t = u / GE::G;
-    hr = (int)(t % HR);
+    // Block-rows are taken from the last one down.  The matmul kernels on either side of this one walk a causal
+    // layout from its longest rows (the last ones) to its shortest, so this order reads first what the producer wrote
+    // last; measured in the attention chain it makes this kernel and its consumer 3-5 % faster than the ascending order.
+    hr = HR - 1 - (int)(t % HR);
     z = (int)(t / HR);
     rxm = g * GE::RPW + lane / GE::LPR;
     col = (lane % GE::LPR) * GE::EV;
