@@ -92,9 +92,11 @@ template <typename T, int BLOCK> struct Unit {
   }
 };
 
-template <typename T, int BLOCK>
+// KPM_LDS: the caller staged the key-padding term of this block in LDS, already as what has to be added to the
+// logits (`kpm_s` points at the block's BLOCK floats); otherwise the mask is read from global memory.
+template <typename T, int BLOCK, bool KPM_LDS = false>
 __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
-                                           float (&fx)[Geo<T, BLOCK>::EV]) {
+                                           float (&fx)[Geo<T, BLOCK>::EV], const float *kpm_s = nullptr) {
   constexpr int EV = Geo<T, BLOCK>::EV;
   const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
   const int64_t grow = (int64_t)brow * BLOCK + u.rxm;    // row in the dense matrix
@@ -103,8 +105,13 @@ __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK
   const float sc = a.scale * unit;
   Pack<T, EV> px;
   px.load(x);
+  if (KPM_LDS && a.kpm) {                                                                    // softmax.py:112-116, 122-124
 #pragma unroll
-  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;                               // softmax.py:112-116
+    for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(px.e[e]), sc, kpm_s[u.col + e]);
+  } else {
+#pragma unroll
+    for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;
+  }
   if (a.rpe) {                                                                               // :118-120, address :50-55
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
@@ -112,7 +119,7 @@ __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK
     for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
   }
   // the mask modes are uniform: branch once per block, not once per element
-  if (a.kpm) {                                                                               // :122-124, address :60-62
+  if (!KPM_LDS && a.kpm) {                                                                   // :122-124, address :60-62
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol);
     if (a.kpm_mul) {                                                                         // :104-106
@@ -161,14 +168,46 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   const table_ptr core = lut + offset;
   if constexpr (NB > 0) {
     float fx[NB][GE::EV];
-    int32_t bid[NB];
+    int32_t bid[NB], bcol[NB];
     float mx = -INFINITY;
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
-        bid[b] = core[4 * b + 0];
-        fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], bid[b], fx[b]);
+    for (int b = 0; b < NB; b++) {
+      const int bb = b < size ? b : 0;                  // blocks past the end repeat the first one (never used, valid to read)
+      bid[b] = core[4 * bb + 0];
+      bcol[b] = core[4 * bb + 1];
+    }
+    // All rows of a wavefront need the same BLOCK key-padding values per block.  The wavefront fetches them once
+    // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
+    // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
+    // the CU, and of the conversions, compared with every row reading the mask itself.
+    __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
+    float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
+    if (a.kpm) {
+      const int lane = threadIdx.x & 63;
+      const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz;
+      constexpr int CH = NB * GE::LPR;                  // chunks of EV values
+#pragma unroll
+      for (int c0 = 0; c0 < CH; c0 += 64) {
+        const int c = c0 + lane, b = c / GE::LPR;
+        int col = bcol[0];
+#pragma unroll
+        for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
+        if (CH % 64 == 0 || c < CH) {
+          Pack<T, GE::EV> p;
+          p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
+          const float unit = logit_unit<T>();
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) {
+            const float m = to_float(p.e[e]);
+            kpm_s[c * GE::EV + e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+          }
+        }
       }
+      __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
+    }
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) fwd_logits<T, BLOCK, true>(a, u, head, brow, bcol[b], bid[b], fx[b], kpm_s + b * BLOCK);
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
