@@ -76,6 +76,22 @@ def test_long_rows_streaming_variant(block, cols):
     run_case(1, 1, 2, cols, block, torch.float32, 0.95, cols + 1, scale=0.5)
 
 
+@pytest.mark.parametrize('longest', [1, 2, 3, 4, 5, 6, 7, 8, 9, 16, 17, 32, 33])
+def test_every_row_length_bucket(longest):
+    # one kernel instantiation per bucket of "blocks kept in registers": the longest row decides which one runs, the
+    # other rows (1 block, longest - 1 blocks, none) exercise its partially filled and empty paths
+    C = longest + 1
+    lay = torch.zeros(2, 4, C, dtype=torch.int64)
+    lay[0, 0, :longest] = 1
+    lay[0, 1, C - 1] = 1
+    lay[0, 3, 1:longest] = 1
+    lay[1, 2, 1:1 + longest] = 1
+    lay[1, 0, 0] = 1
+    run_case(2, 2, 4, C, 64, torch.float16, 0, 100 + longest, scale=0.3, kpm='add', layout=lay)
+    run_case(1, 2, 4, C, 16, torch.bfloat16, 0, 200 + longest, scale=0.3, kpm='mul', attn='add', layout=lay)
+    run_case(1, 2, 4, C, 32, torch.float32, 0, 300 + longest, scale=0.3, rpe=True, kpm='add', layout=lay)
+
+
 def test_rows_without_blocks_and_single_block():
     lay = torch.zeros(2, 4, 4, dtype=torch.int64)
     lay[0, 0, 1] = 1

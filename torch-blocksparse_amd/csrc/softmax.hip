@@ -345,6 +345,8 @@ template <typename T, int BLOCK> void launch_fwd(const FwdArgs &a, int maxlut, h
   if (maxlut <= 1) launch_fwd_nb<T, BLOCK, 1>(a, st);
   else if (maxlut <= 2) launch_fwd_nb<T, BLOCK, 2>(a, st);
   else if (maxlut <= 4) launch_fwd_nb<T, BLOCK, 4>(a, st);
+  else if (maxlut <= 6) launch_fwd_nb<T, BLOCK, 6>(a, st);
+  else if (maxlut <= 7) launch_fwd_nb<T, BLOCK, 7>(a, st);
   else if (maxlut <= 8) launch_fwd_nb<T, BLOCK, 8>(a, st);
   else if (maxlut <= 16 && 16 <= MX) launch_fwd_nb<T, BLOCK, (16 <= MX ? 16 : 0)>(a, st);
   else if (maxlut <= 32 && 32 <= MX) launch_fwd_nb<T, BLOCK, (32 <= MX ? 32 : 0)>(a, st);
@@ -354,6 +356,8 @@ template <typename T, int BLOCK> void launch_bwd(const BwdArgs &a, int maxlut, h
   if (maxlut <= 1) launch_bwd_nb<T, BLOCK, 1>(a, st);
   else if (maxlut <= 2) launch_bwd_nb<T, BLOCK, 2>(a, st);
   else if (maxlut <= 4) launch_bwd_nb<T, BLOCK, 4>(a, st);
+  else if (maxlut <= 6) launch_bwd_nb<T, BLOCK, 6>(a, st);
+  else if (maxlut <= 7) launch_bwd_nb<T, BLOCK, 7>(a, st);
   else if (maxlut <= 8) launch_bwd_nb<T, BLOCK, 8>(a, st);
   else if (maxlut <= 16) launch_bwd_nb<T, BLOCK, 16>(a, st);
   else launch_bwd_nb<T, BLOCK, 0>(a, st);
