@@ -92,11 +92,10 @@ template <typename T, int BLOCK> struct Unit {
   }
 };
 
-// KPM_LDS: the caller staged the key-padding term of this block in LDS, already as what has to be added to the
-// logits (`kpm_s` points at the block's BLOCK floats); otherwise the mask is read from global memory.
-template <typename T, int BLOCK, bool KPM_LDS = false>
+// logits of one block, everything read from global memory (streaming variant)
+template <typename T, int BLOCK>
 __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
-                                           float (&fx)[Geo<T, BLOCK>::EV], const float *kpm_s = nullptr) {
+                                           float (&fx)[Geo<T, BLOCK>::EV]) {
   constexpr int EV = Geo<T, BLOCK>::EV;
   const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
   const int64_t grow = (int64_t)brow * BLOCK + u.rxm;    // row in the dense matrix
@@ -105,13 +104,8 @@ __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK
   const float sc = a.scale * unit;
   Pack<T, EV> px;
   px.load(x);
-  if (KPM_LDS && a.kpm) {                                                                    // softmax.py:112-116, 122-124
 #pragma unroll
-    for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(px.e[e]), sc, kpm_s[u.col + e]);
-  } else {
-#pragma unroll
-    for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;
-  }
+  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;                               // softmax.py:112-116
   if (a.rpe) {                                                                               // :118-120, address :50-55
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
@@ -119,7 +113,7 @@ __device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK
     for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
   }
   // the mask modes are uniform: branch once per block, not once per element
-  if (!KPM_LDS && a.kpm) {                                                                   // :122-124, address :60-62
+  if (a.kpm) {                                                                               // :122-124, address :60-62
     Pack<T, EV> p;
     p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol);
     if (a.kpm_mul) {                                                                         // :104-106
@@ -153,8 +147,10 @@ __device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<T, BLOCK>
   p.store(x);
 }
 
-// NB = number of blocks of a row kept in registers; NB == 0 selects the streaming variant.
-template <typename T, int BLOCK, int NB>
+// NB = number of blocks of a row kept in registers; NB == 0 selects the streaming variant.  EXTRA = a relative
+// position embedding or an attention mask is present (their values are kept beside x until the logits are built; the
+// plain variant does not pay registers for them).
+template <typename T, int BLOCK, int NB, bool EXTRA>
 __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   typedef Geo<T, BLOCK> GE;
   const int HR = a.H * a.R;
@@ -167,7 +163,10 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   if (size <= 0) return;
   const table_ptr core = lut + offset;
   if constexpr (NB > 0) {
+    typedef Pack<T, GE::EV> P;
+    constexpr int NX = EXTRA ? NB : 1;
     float fx[NB][GE::EV];
+    P px[NB], pr[NX], pa[NX];
     int32_t bid[NB], bcol[NB];
     float mx = -INFINITY;
 #pragma unroll
@@ -176,12 +175,28 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       bid[b] = core[4 * bb + 0];
       bcol[b] = core[4 * bb + 1];
     }
+    // Every load of the row is issued before anything waits for one: the wavefront pays the memory latency once,
+    // not once per block.  (Loads and the arithmetic on them in one per-block branch end up serialised.)
+    const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
+    const int64_t grow = (int64_t)brow * BLOCK + u.rxm;  // row in the dense matrix
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+        px[b].load(xb + (int64_t)bid[b] * (BLOCK * BLOCK));
+        if constexpr (EXTRA) {
+          const int64_t gcol = (int64_t)bcol[b] * BLOCK + u.col;   // lane's first column in the dense matrix
+          if (a.rpe)                                               // address: softmax.py:50-55
+            pr[b].load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
+          if (a.attn) pa[b].load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);   // :67-70
+        }
+      }
     // All rows of a wavefront need the same BLOCK key-padding values per block.  The wavefront fetches them once
     // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
     // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
     // the CU, and of the conversions, compared with every row reading the mask itself.
     __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
     float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
+    const float unit = logit_unit<T>();
     if (a.kpm) {
       const int lane = threadIdx.x & 63;
       const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz;
@@ -193,9 +208,8 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
 #pragma unroll
         for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
         if (CH % 64 == 0 || c < CH) {
-          Pack<T, GE::EV> p;
+          P p;
           p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
-          const float unit = logit_unit<T>();
 #pragma unroll
           for (int e = 0; e < GE::EV; e++) {
             const float m = to_float(p.e[e]);
@@ -205,9 +219,43 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       }
       __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
     }
+    const float sc = a.scale * unit;
+    if (a.kpm) {                                        // softmax.py:112-116, 122-124
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) fwd_logits<T, BLOCK, true>(a, u, head, brow, bcol[b], bid[b], fx[b], kpm_s + b * BLOCK);
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(px[b].e[e]), sc, kpm_s[b * BLOCK + u.col + e]);
+        }
+    } else {
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) fx[b][e] = to_float(px[b].e[e]) * sc;
+        }
+    }
+    if constexpr (EXTRA) {
+      if (a.rpe) {                                      // :118-120
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+          if (b < size) {
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(pr[b].e[e]), unit, fx[b][e]);
+          }
+      }
+      if (a.attn) {                                     // :126-128, 'mul' mode :108-110
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+          if (b < size) {
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) {
+              const float m = to_float(pa[b].e[e]);
+              fx[b][e] += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+            }
+          }
+      }
+    }
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
@@ -333,7 +381,8 @@ template <typename T, int BLOCK> constexpr int max_nb_bwd() { return 16; }
 
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
   const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
-  hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+  if (NB > 0 && (a.rpe || a.attn)) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, NB != 0>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+  else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
 }
 template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hipStream_t st) {
   const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
