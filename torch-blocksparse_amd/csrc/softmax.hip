@@ -14,6 +14,7 @@ namespace bsp {
 namespace {
 
 constexpr int kWavesPerGroup = 4;
+constexpr int kChunk = 8;           // blocks per step of the streaming variants
 
 template <typename T, int EV> struct RawVec;
 template <> struct RawVec<f16, 8> { typedef u32x4 type; };
@@ -91,51 +92,6 @@ template <typename T, int BLOCK> struct Unit {
     col = (lane % GE::LPR) * GE::EV;
   }
 };
-
-// logits of one block, everything read from global memory (streaming variant)
-template <typename T, int BLOCK>
-__device__ __forceinline__ void fwd_logits(const FwdArgs &a, const Unit<T, BLOCK> &u, int head, int brow, int bcol, int64_t blockid,
-                                           float (&fx)[Geo<T, BLOCK>::EV]) {
-  constexpr int EV = Geo<T, BLOCK>::EV;
-  const T *x = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
-  const int64_t grow = (int64_t)brow * BLOCK + u.rxm;    // row in the dense matrix
-  const int64_t gcol = (int64_t)bcol * BLOCK + u.col;    // lane's first column in the dense matrix
-  const float unit = logit_unit<T>();
-  const float sc = a.scale * unit;
-  Pack<T, EV> px;
-  px.load(x);
-#pragma unroll
-  for (int e = 0; e < EV; e++) fx[e] = to_float(px.e[e]) * sc;                               // softmax.py:112-116
-  if (a.rpe) {                                                                               // :118-120, address :50-55
-    Pack<T, EV> p;
-    p.load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
-#pragma unroll
-    for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
-  }
-  // the mask modes are uniform: branch once per block, not once per element
-  if (a.kpm) {                                                                               // :122-124, address :60-62
-    Pack<T, EV> p;
-    p.load(reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + gcol);
-    if (a.kpm_mul) {                                                                         // :104-106
-#pragma unroll
-      for (int e = 0; e < EV; e++) fx[e] += (to_float(p.e[e]) == 0.f) ? -INFINITY : 0.f;
-    } else {
-#pragma unroll
-      for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
-    }
-  }
-  if (a.attn) {                                                                              // :126-128, address :67-70
-    Pack<T, EV> p;
-    p.load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);
-    if (a.attn_mul) {                                                                        // :108-110
-#pragma unroll
-      for (int e = 0; e < EV; e++) fx[e] += (to_float(p.e[e]) == 0.f) ? -INFINITY : 0.f;
-    } else {
-#pragma unroll
-      for (int e = 0; e < EV; e++) fx[e] = fmaf(to_float(p.e[e]), unit, fx[e]);
-    }
-  }
-}
 
 template <typename T, int BLOCK>
 __device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<T, BLOCK> &u, int64_t blockid, const float (&y)[Geo<T, BLOCK>::EV]) {
@@ -280,27 +236,94 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
         fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
       }
   } else {
-    float fx[GE::EV];
-    float mx = -INFINITY;
-    for (int b = 0; b < size; b++) {
-      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+    // Rows with more blocks than the register variant holds: two passes over x, kChunk blocks at a time with all loads
+    // of a chunk in flight together.  Pass 1 keeps a running maximum and a running sum per lane (the sum is rescaled
+    // when the maximum grows), pass 2 reads x again and writes the result: 2 reads + 1 write of x.
+    typedef Pack<T, GE::EV> P;
+    constexpr int CH = kChunk, NX = EXTRA ? CH : 1;
+    const float unit = logit_unit<T>();
+    const float sc = a.scale * unit;
+    const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
+    T *yb = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
+    const int64_t grow = (int64_t)brow * BLOCK + u.rxm;
+    const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + u.col;
+    const T *rz = reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + u.col;
+    const T *az = reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + u.col;
+    P px[CH], pk[CH], pr[NX], pa[NX];
+    int32_t bid[CH];
+    auto load_chunk = [&](int b0) {
 #pragma unroll
-      for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[e]);
-    }
-    mx = row_max<GE::LPR>(mx);
-    float sum = 0.f;
-    for (int b = 0; b < size; b++) {
-      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+          bid[j] = core[4 * (b0 + j) + 0];
+          const int64_t c0 = (int64_t)core[4 * (b0 + j) + 1] * BLOCK;   // first column of the block in the dense matrix
+          px[j].load(xb + (int64_t)bid[j] * (BLOCK * BLOCK));
+          if (a.kpm) pk[j].load(kz + c0);
+          if constexpr (EXTRA) {
+            if (a.rpe) pr[j].load(rz + c0);
+            if (a.attn) pa[j].load(az + c0);
+          }
+        }
+    };
+    auto logits = [&](int j, float (&l)[GE::EV]) {      // softmax.py:104-128
 #pragma unroll
-      for (int e = 0; e < GE::EV; e++) sum += exp_sub<T>(fx[e], mx);
+      for (int e = 0; e < GE::EV; e++) l[e] = to_float(px[j].e[e]) * sc;
+      if (a.kpm) {
+#pragma unroll
+        for (int e = 0; e < GE::EV; e++) {
+          const float m = to_float(pk[j].e[e]);
+          l[e] += a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+        }
+      }
+      if constexpr (EXTRA) {
+        if (a.rpe) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) l[e] = fmaf(to_float(pr[j].e[e]), unit, l[e]);
+        }
+        if (a.attn) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) {
+            const float m = to_float(pa[j].e[e]);
+            l[e] += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+          }
+        }
+      }
+    };
+    float mx = -INFINITY, sum = 0.f;
+    for (int b0 = 0; b0 < size; b0 += CH) {
+      load_chunk(b0);
+#pragma unroll
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+          float l[GE::EV];
+          logits(j, l);
+          float m = mx;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) m = fmaxf(m, l[e]);
+          const float ms = m == -INFINITY ? 0.f : m;    // everything masked so far: any finite shift does
+          float part = 0.f;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) part += exp_sub<T>(l[e], ms);
+          sum = sum * exp_sub<T>(mx, ms) + part;
+          mx = m;
+        }
     }
-    sum = row_sum<GE::LPR>(sum);
+    const float rmx = row_max<GE::LPR>(mx);             // :130
+    const float shift = rmx == -INFINITY ? 0.f : rmx;   // a fully masked row ends as 0 * inf = NaN, like the register variant
+    sum = row_sum<GE::LPR>(sum * exp_sub<T>(mx, shift));
     const float inv = 1.f / sum;
-    for (int b = 0; b < size; b++) {
-      fwd_logits<T, BLOCK>(a, u, head, brow, core[4 * b + 1], core[4 * b + 0], fx);
+    for (int b0 = 0; b0 < size; b0 += CH) {
+      load_chunk(b0);
 #pragma unroll
-      for (int e = 0; e < GE::EV; e++) fx[e] = exp_sub<T>(fx[e], mx) * inv;
-      fwd_store<T, BLOCK>(a, u, core[4 * b + 0], fx);
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+          float l[GE::EV];
+          logits(j, l);
+          P out;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) out.e[e] = from_float<T>(exp_sub<T>(l[e], shift) * inv);   // :131-137
+          out.store(yb + (int64_t)bid[j] * (BLOCK * BLOCK));
+        }
     }
   }
 }
@@ -353,24 +376,41 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
         out.store(db + (int64_t)bid[b] * (BLOCK * BLOCK));
       }
   } else {
-    float dot = 0.f;
-    for (int b = 0; b < size; b++) {
-      const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
-      P py, pd;
-      py.load(yb + o);
-      pd.load(db + o);
+    // longer rows: two passes, kChunk blocks at a time with all loads of a chunk in flight together
+    constexpr int CH = kChunk;
+    P py[CH], pd[CH];
+    int64_t off[CH];
+    auto load_chunk = [&](int b0) {
 #pragma unroll
-      for (int e = 0; e < GE::EV; e++) dot += to_float(py.e[e]) * to_float(pd.e[e]);
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+          off[j] = (int64_t)core[4 * (b0 + j)] * (BLOCK * BLOCK);
+          py[j].load(yb + off[j]);
+          pd[j].load(db + off[j]);
+        }
+    };
+    float dot = 0.f;
+    for (int b0 = 0; b0 < size; b0 += CH) {
+      load_chunk(b0);
+#pragma unroll
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) dot += to_float(py[j].e[e]) * to_float(pd[j].e[e]);
+        }
     }
     dot = row_sum<GE::LPR>(dot);
-    for (int b = 0; b < size; b++) {
-      const int64_t o = (int64_t)core[4 * b] * (BLOCK * BLOCK);
-      P py, pd, out;
-      py.load(yb + o);
-      pd.load(db + o);
+    for (int b0 = 0; b0 < size; b0 += CH) {
+      load_chunk(b0);
 #pragma unroll
-      for (int e = 0; e < GE::EV; e++) out.e[e] = from_float<T>(to_float(py.e[e]) * (to_float(pd.e[e]) - dot) * a.scale);
-      out.store(db + o);
+      for (int j = 0; j < CH; j++)
+        if (b0 + j < size) {
+          P out;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++)
+            out.e[e] = from_float<T>(to_float(py[j].e[e]) * (to_float(pd[j].e[e]) - dot) * a.scale);
+          out.store(db + off[j]);
+        }
     }
   }
 }
@@ -381,7 +421,7 @@ template <typename T, int BLOCK> constexpr int max_nb_bwd() { return 16; }
 
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
   const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
-  if (NB > 0 && (a.rpe || a.attn)) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, NB != 0>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+  if (a.rpe || a.attn) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
   else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
 }
 template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hipStream_t st) {
