@@ -30,10 +30,10 @@ MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 # the same counter reads for the calibration copy of known size (profiles/traffic_attention_seq4096.txt).  None = not
 # measured for this build of the kernel.
 TRAFFIC_BYTES = {
-    'sdd_fwd  q.k^T': 140210325 + 268435464, 'sdd_bwd  do.v^T': 140210325 + 268435464,
-    'dsd_fwd  p.v': 342657616 + 67108864, 'dsd_bwd  ds.k': 342657616 + 67108864,
-    'dsd_bwd  p^T.do': 428109030 + 67108864, 'dds_bwd  (q^T.ds)^T': 428109030 + 67108864,
-    'softmax_fwd': 269876117 + 268435456, 'softmax_bwd': 538087015 + 268435456,
+    'sdd_fwd  q.k^T': 140072457 + 268435460, 'sdd_bwd  do.v^T': 140072457 + 268435460,
+    'dsd_fwd  p.v': 342691472 + 67108864, 'dsd_bwd  ds.k': 342691472 + 67108864,
+    'dsd_bwd  p^T.do': 428215956 + 67108864, 'dds_bwd  (q^T.ds)^T': 428215956 + 67108864,
+    'softmax_fwd': 269785972 + 268435456, 'softmax_bwd': 538129920 + 268435456,
 }
 
 
