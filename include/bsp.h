@@ -78,7 +78,8 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * BSP_GROUP consecutive block-rows (by_rows != 0) or block-columns of one head form a group that one workgroup
  * processes together, sharing the dense tiles its members have in common.  d_plan receives 4 ints per group
  * (first entry, entries, head, group index; sorted by decreasing entries) followed by BSP_GROUP+1 ints per entry
- * (position along the other dimension, block id of each member or -1).  plan_cap >= bsp_group_plan_cap(...). */
+ * (position along the other dimension, block id of each member or -1), positions ascending for row groups and
+ * descending for column groups.  plan_cap >= bsp_group_plan_cap(...). */
 #define BSP_GROUP 4
 int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);
 int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int32_t *d_plan, int64_t plan_cap,

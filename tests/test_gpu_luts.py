@@ -71,7 +71,8 @@ def test_empty_head_raises():
 @pytest.mark.parametrize('by_rows', [True, False])
 def test_group_plan(by_rows):
     # our own work list for the row-group kernels: 4 consecutive lines per group, one entry per position where any
-    # member has a block, header sorted by decreasing number of entries
+    # member has a block (positions ascending for row groups, descending for column groups), header sorted by
+    # decreasing number of entries
     from torch_blocksparse.matmul import GroupPlan
     for lay in (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64)):
         plan = GroupPlan.build(lay, by_rows, DEV)
@@ -88,7 +89,7 @@ def test_group_plan(by_rows):
         total = 0
         for start, count, h, lg in header:
             exp = []
-            for b in range(B):
+            for b in (range(B) if by_rows else range(B - 1, -1, -1)):
                 bids = []
                 for m in range(4):
                     line = lg * 4 + m
