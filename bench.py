@@ -27,7 +27,7 @@ HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 
 # HBM bytes per launch at batch 8, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what
-# the same counter reads for the calibration copy of known size (profiles/traffic_attention_seq4096.txt).  None = not
+# the same counter reads for the calibration copy of known size (profiles/attention_seq4096_fp16_blk64.txt).  None = not
 # measured for this build of the kernel.
 TRAFFIC_BYTES = {
     'sdd_fwd  q.k^T': 140072457 + 268435460, 'sdd_bwd  do.v^T': 140072457 + 268435460,
@@ -44,10 +44,14 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--batch', type=int, default=8)
+    ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
+                    help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: the path shards over batch and heads without communication, '
                  'and no multi-GPU run is part of this build (got --gpus %d)' % args.gpus)
+    if args.config != 3:
+        return other_config(args)
 
     import torch
     import torch_blocksparse as tb
@@ -183,6 +187,108 @@ def main():
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, L)
     print(json.dumps(out))
+
+
+def other_config(args):
+    """The configurations the headline metric is not quoted on: every launch timed on its own (HIP events, mean of
+    `--steps` back-to-back launches), effective throughput over the nonzero blocks.  One JSON line, not the headline."""
+    import torch
+    import torch_blocksparse as tb
+    dev = torch.device('cuda:0')
+    out = []
+
+    def timeit(f):
+        for _ in range(max(args.warmup, 1)):
+            f()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            f()
+        e1.record()
+        e1.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    def bernoulli(shape, density, seed, one_per_row=False):
+        g = torch.Generator().manual_seed(seed)
+        lay = (torch.rand(shape, generator=g) < density).long()
+        if one_per_row:
+            for h in range(shape[0]):
+                for r in range(shape[1]):
+                    if lay[h, r].sum() == 0:
+                        lay[h, r, int(torch.randint(0, shape[2], (1,), generator=g))] = 1
+        return lay
+
+    def mm(name, mode, ta, tb_, block, dtype, Z, H, M, N, K, lay, scale=1.0):
+        nnz = int(lay.sum())
+        a = torch.randn((Z, H) + ((K, M) if ta else (M, K)), device=dev, dtype=dtype) * scale
+        b = torch.randn((Z, H) + ((N, K) if tb_ else (K, N)), device=dev, dtype=dtype) * scale
+        if mode == 'dsd':
+            a = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype)
+        if mode == 'dds':
+            b = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype)
+        op = tb.MatMul(lay, block, mode, trans_a=ta, trans_b=tb_)
+        with torch.no_grad():
+            ms = timeit(lambda: op(a, b))
+        D = {'sdd': K, 'dsd': N, 'dds': M}[mode]
+        fl = 2.0 * Z * D * nnz * block * block
+        peak = 157.3 if dtype == torch.float32 else MFMA_PEAK_TFLOPS
+        out.append({'launch': name, 'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'mfma_frac': round(fl / ms * 1e-9 / peak, 4)})
+
+    if args.config == 1:
+        torch.manual_seed(0)
+        lay = torch.randint(0, 2, (2, 16, 32))
+        mm('sdd trans_a fp32 blk16 Z4 H2 256x512x384', 'sdd', True, False, 16, torch.float32, 4, 2, 256, 512, 384, lay)
+        x = torch.rand(4, int(lay.sum()), 16, 16, device=dev)
+        sm = tb.Softmax(lay, 16)
+        with torch.no_grad():
+            ms = timeit(lambda: sm(x))
+        out.append({'launch': 'softmax fwd fp32 blk16', 'ms': round(ms, 4), 'GB/s': round(2 * x.numel() * 4 / ms * 1e-6, 1)})
+        workload = 'README shape: sdd trans_a fp32 block 16 + softmax'
+    elif args.config == 2:
+        lay = bernoulli((16, 64, 64), 0.25, 2, one_per_row=True)
+        for ta in (False, True):
+            for tb_ in (False, True):
+                mm('dsd trans_a=%d trans_b=%d' % (ta, tb_), 'dsd', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
+                mm('dds trans_a=%d trans_b=%d' % (ta, tb_), 'dds', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
+        mm('sdd (gradient of the sparse operand)', 'sdd', False, True, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay)
+        workload = 'fp16 block 32, Z 8, H 16, M=N=K=2048, Bernoulli(0.25) layout'
+    elif args.config == 5:
+        lay = bernoulli((1, 32, 32), 0.1, 5)
+        mm('dds trans_b (y = x.W^T)', 'dds', False, True, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
+        mm('dds (dx = dy.W)', 'dds', False, False, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
+        mm('sdd trans_a (dW = dy^T.x on the layout)', 'sdd', True, False, 128, torch.float16, 1, 1, 4096, 4096, 8192, lay, 0.1)
+        workload = 'block-sparse linear layer: 8192 tokens, 4096x4096 weight, block 128, 10 % density, fp16'
+    else:
+        lay = tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True)
+        B, H, L, dh, block = 2, 12, 16384, 64, 64
+        nnz = int(lay.sum())
+        q, k, v = [torch.randn(B, H, L, dh, device=dev, dtype=torch.float16) for _ in range(3)]
+        sdd = tb.MatMul(lay, block, 'sdd', trans_b=True)
+        dsd = tb.MatMul(lay, block, 'dsd')
+        sm = tb.Softmax(lay, block)
+        nb = L // block
+        idx = torch.arange(nb)
+        rpe_bb = (0.1 * torch.randn(nb)).half()[(idx[:, None] - idx[None, :]).abs()].to(dev)
+        rpe = rpe_bb.repeat_interleave(block, 0).repeat_interleave(block, 1)[None, None].expand(B, H, L, L)
+        causal = torch.tril(torch.ones(L, L, dtype=torch.float16, device=dev))
+        fl = 2.0 * B * dh * nnz * block * block
+        xb = B * nnz * block * block * 2
+        with torch.no_grad():
+            w = sdd(q, k)
+            for name, f, flops, nbytes in (
+                    ('sdd q.k^T', lambda: sdd(q, k), fl, xb + 2 * B * H * L * dh * 2),
+                    ('softmax fwd, scale only', lambda: sm(w, scale=0.125), 0, 2 * xb),
+                    ('softmax fwd, rpe + causal mask', lambda: sm(w, scale=0.125, rpe=rpe, attn_mask=causal, attn_mask_mode='mul'), 0, 2 * xb),   # x only: both masks are shared by batch and heads
+                    ('dsd p.v', lambda: dsd(w, v), fl, xb + 2 * B * H * L * dh * 2)):
+                ms = timeit(f)
+                ent = {'launch': name, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)}
+                if flops:
+                    ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
+                out.append(ent)
+        workload = 'BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, forward chain'
+    print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
+                      'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic', 'config': {'workload': workload, 'config': args.config},
+                      'launches': out}))
 
 
 def _bwd_softmax(tb, y, dy, scale, lut, maxlut, spdims, block):
