@@ -79,11 +79,15 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * processes together, sharing the dense tiles its members have in common.  d_plan receives 4 ints per group
  * (first entry, entries, head, group index; sorted by decreasing entries) followed by BSP_GROUP+1 ints per entry
  * (position along the other dimension, block id of each member or -1), positions ascending for row groups and
- * descending for column groups.  plan_cap >= bsp_group_plan_cap(...). */
+ * descending for column groups.  thin_min > 0: a line with at least thin_min blocks leaves its group and becomes a
+ * chain of its own (group index field = -(line + 1), member 0 = the line), whose entries bsp_dsd_matmul /
+ * bsp_dds_matmul spread over the wavefronts of a workgroup; bits 24..27 of a group's index field mark the members
+ * that left it (needs fewer than 2^24 groups per head).  Pass 0 for a plan given to bsp_sdd_matmul.
+ * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */
 #define BSP_GROUP 4
 int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);
-int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int32_t *d_plan, int64_t plan_cap,
-                         void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream);
+int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int32_t *d_plan,
+                         int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Matmul launchers.  Strides are in elements; the innermost stride of every operand is 1 and rows start on

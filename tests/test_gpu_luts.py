@@ -69,37 +69,60 @@ def test_empty_head_raises():
 
 
 @pytest.mark.parametrize('by_rows', [True, False])
-def test_group_plan(by_rows):
+@pytest.mark.parametrize('thin_min', [0, 6])
+def test_group_plan(by_rows, thin_min):
     # our own work list for the row-group kernels: 4 consecutive lines per group, one entry per position where any
-    # member has a block (positions ascending for row groups, descending for column groups), header sorted by
-    # decreasing number of entries
+    # member has a block (positions ascending for row groups, descending for column groups); lines with at least
+    # thin_min blocks leave their group (bit 24 + member of its index field) and become chains (index field
+    # -(line + 1)); header sorted by decreasing number of entries, groups before chains at equal length
     from torch_blocksparse.matmul import GroupPlan
-    for lay in (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64)):
-        plan = GroupPlan.build(lay, by_rows, DEV)
+    for lay in (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64),
+                torch.ones(2, 7, 9, dtype=torch.int64)):
+        plan = GroupPlan.build(lay, by_rows, DEV, thin_min=thin_min)
         t = plan.table.cpu().tolist()
         H, R, C = lay.shape
         L, B = (R, C) if by_rows else (C, R)
-        ng = H * ((L + 3) // 4)
-        assert plan.n_groups == ng and plan.lines == L
+        NG = (L + 3) // 4
+        linecnt = lay.sum(2 if by_rows else 1)                      # [H, L]
+        thin = (linecnt >= thin_min) if thin_min else torch.zeros_like(linecnt, dtype=torch.bool)
         rank = (torch.cumsum(lay.reshape(-1), 0) - 1).reshape(lay.shape)
-        header = [t[4 * i:4 * i + 4] for i in range(ng)]
-        counts = [h[1] for h in header]
-        assert counts == sorted(counts, reverse=True)
-        assert sorted((h[2], h[3]) for h in header) == [(h, g) for h in range(H) for g in range((L + 3) // 4)]
-        total = 0
-        for start, count, h, lg in header:
-            exp = []
-            for b in (range(B) if by_rows else range(B - 1, -1, -1)):
+        order = range(B) if by_rows else range(B - 1, -1, -1)
+
+        def entries(h, lines):                                      # lines: 4 line indices or None
+            out = []
+            for b in order:
                 bids = []
-                for m in range(4):
-                    line = lg * 4 + m
-                    if line < L:
+                for line in lines:
+                    if line is None:
+                        bids.append(-1)
+                    else:
                         r, c = (line, b) if by_rows else (b, line)
                         bids.append(int(rank[h, r, c]) if lay[h, r, c] else -1)
-                    else:
-                        bids.append(-1)
                 if any(x >= 0 for x in bids):
-                    exp.append([b] + bids)
+                    out.append([b] + bids)
+            return out
+
+        slots = []                                                  # (slot order, code, head, expected entries)
+        for h in range(H):
+            for lg in range(NG):
+                lines, skip = [], 0
+                for m in range(4):
+                    line = lg * 4 + m
+                    if line < L and thin[h, line]:
+                        skip |= 1 << m
+                    lines.append(line if line < L and not thin[h, line] else None)
+                slots.append((lg | (skip << 24), h, entries(h, lines)))
+        for h in range(H):
+            for line in range(L):
+                if thin[h, line]:
+                    slots.append((-(line + 1), h, entries(h, [line, None, None, None])))
+        slots.sort(key=lambda s: -len(s[2]))                        # stable: ties stay in slot order
+        ng = len(slots)
+        assert plan.n_groups == ng and plan.lines == L
+        total = 0
+        for i, (code, h, exp) in enumerate(slots):
+            start, count, gh, gcode = t[4 * i:4 * i + 4]
+            assert (count, gh, gcode) == (len(exp), h, code)
             got = [t[4 * ng + 5 * (start + k):4 * ng + 5 * (start + k + 1)] for k in range(count)]
             assert got == exp
             total += count

@@ -82,6 +82,32 @@ def test_normal_inputs_with_cancellation():
     run_case('sdd', False, True, 64, torch.float32, dist='randn', scale=1.0, seed=9)
 
 
+@pytest.mark.parametrize('mode,trans_a,trans_b', [('dsd', False, False), ('dsd', True, False), ('dds', False, False), ('dds', True, True)])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_long_lines_become_chains(mode, trans_a, trans_b, dtype):
+    # block 64: lines far longer than the average leave their group and are reduced by the four wavefronts of a
+    # workgroup in parallel.  A full column, a full row, a 19-block line (19 = 4*4 + 3: wavefronts with unequal shares)
+    # and ordinary lines around them, including a group whose four lines are all chains.
+    R = C = 40
+    lay = torch.zeros(2, R, C, dtype=torch.int64)
+    for i in range(R):
+        lay[:, i, max(0, i - 1):i + 1] = 1           # two-block diagonal band
+    lay[0, :, 5] = 1                                  # global column
+    lay[0, 9, :] = 1                                  # global row
+    lay[1, 12:16, :] = 1                              # a whole group of long rows
+    lay[1, :, 20:24] = 1                              # a whole group of long columns
+    lay[1, 30, :19] = 1
+    lay[1, :19, 33] = 1
+    from torch_blocksparse.matmul import GroupPlan
+    assert GroupPlan.thin_min(lay, True) == 16 and GroupPlan.thin_min(lay, False) == 16
+    Z, H = 2, 2
+    F = 128                                           # dense free dimension: two 64-wide tiles
+    if mode == 'dsd':
+        run_case(mode, trans_a, trans_b, 64, dtype, Z=Z, H=H, M=64 * R, N=F, K=64 * C, layout=lay, seed=5, dist='randn', scale=0.25)
+    else:
+        run_case(mode, trans_a, trans_b, 64, dtype, Z=Z, H=H, M=F, N=64 * C, K=64 * R, layout=lay, seed=5, dist='randn', scale=0.25)
+
+
 def test_degenerate_layouts():
     # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
     lay = torch.zeros(2, 4, 6, dtype=torch.int64)

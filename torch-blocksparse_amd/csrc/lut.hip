@@ -15,7 +15,8 @@ namespace {
 // workspace carving (int32 units)
 // ---------------------------------------------------------------------------------------------------------
 struct Ws {
-  int64_t rowcnt, rowstart, colcnt, colstart, linepacks, segstart, headmax, rank, lay, tmp, top, counts, offsets, scal, end;
+  int64_t rowcnt, rowstart, colcnt, colstart, linepacks, segstart, headmax, rank, lay, tmp, top, counts, offsets, scal;
+  int64_t gcnt, gstart, galive, gapos, end;   // group plan: per slot entries, their prefix sums, alive flag, its prefix sums
   __host__ Ws(int H, int R, int C) {
     int64_t hr = (int64_t)H * R, hc = (int64_t)H * C, cells = (int64_t)H * R * C, hl = hr > hc ? hr : hc;
     int64_t o = 0;
@@ -26,6 +27,8 @@ struct Ws {
     counts = take(2 * 8 * (int64_t)H);   // int64 [8 levels][H]
     offsets = take(2 * 8 * (int64_t)H);  // int64 [8 levels][H]
     scal = take(16);
+    const int64_t slots = 2 * hl + H + 8;   // groups of BSP_GROUP lines + one potential chain per line
+    gcnt = take(slots); gstart = take(slots + 1); galive = take(slots); gapos = take(slots + 1);
     end = o;
   }
 };
@@ -338,55 +341,84 @@ __global__ void k_sdd_offsets(const int64_t *counts, int64_t *offsets, int nlev,
 // Group plan: the work list of the row-group matmul kernels (no counterpart in the reference).  BSP_GROUP
 // consecutive block-rows (by_rows) or block-columns of one head form a group; an entry of a group is one
 // position b along the other dimension where at least one member has a block: (b, blockid of member 0..3, -1
-// where absent).  Header rows (first entry, number of entries, head, group index) are sorted by decreasing number
-// of entries so that the longest groups are dispatched first (measured: dispatching them late costs far more than
-// the L2 locality of a head-by-head order gains).
+// where absent).  A line with at least `thin_min` blocks (thin_min > 0) is taken out of its group and becomes a
+// chain of its own (group index field = -(line + 1), member 0 = the line): the kernels split a chain's entries over
+// their wavefronts instead of walking them one after the other, so that one long line (a global column of an
+// attention layout seen from the transposed product) is not the critical path of the launch.
+// Header rows (first entry, number of entries, head, group index) are sorted by decreasing number of entries so
+// that the longest are dispatched first (measured: dispatching them late costs far more than the L2 locality of a
+// head-by-head order gains).  Slots: [0, H*NG) the groups, then one slot per line for its chain (unused if not thin).
 // ---------------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int64_t cell(int R, int C, int h, int line, int b, int by_rows) {
   return by_rows ? ((int64_t)h * R + line) * C + b : ((int64_t)h * R + b) * C + line;
 }
-__global__ void k_gplan_count(const int32_t *lay, int H, int R, int C, int by_rows, int32_t *cnt) {
+__device__ __forceinline__ bool thin_line(const int32_t *linecnt, int64_t j, int thin_min) {
+  return thin_min > 0 && linecnt[j] >= thin_min;
+}
+__global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H, int R, int C, int by_rows, int thin_min,
+                              int32_t *cnt, int32_t *alive) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
+  const int64_t ng = (int64_t)H * NG;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-  if (i >= (int64_t)H * NG) return;
+  if (i >= ng + (int64_t)H * L) return;
+  if (i >= ng) {
+    const bool thin = thin_line(linecnt, i - ng, thin_min);
+    cnt[i] = thin ? linecnt[i - ng] : 0;
+    alive[i] = thin;
+    return;
+  }
   const int h = (int)(i / NG), lg = (int)(i % NG);
+  bool use[BSP_GROUP];
+  for (int g = 0; g < BSP_GROUP; g++) {
+    const int line = lg * BSP_GROUP + g;
+    use[g] = line < L && !thin_line(linecnt, (int64_t)h * L + line, thin_min);
+  }
   int n = 0;
   for (int b = 0; b < B; b++) {
     bool any = false;
-    for (int g = 0; g < BSP_GROUP; g++) {
-      const int line = lg * BSP_GROUP + g;
-      if (line < L && lay[cell(R, C, h, line, b, by_rows)] != 0) any = true;
-    }
+    for (int g = 0; g < BSP_GROUP; g++)
+      if (use[g] && lay[cell(R, C, h, lg * BSP_GROUP + g, b, by_rows)] != 0) any = true;
     n += any;
   }
   cnt[i] = n;
+  alive[i] = 1;   // a group without entries still zero-fills the output of its (non-thin) lines
 }
-__global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *cnt, const int32_t *start, int H, int R,
-                             int C, int by_rows, int32_t *plan) {
+__global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *linecnt, const int32_t *cnt,
+                             const int32_t *start, const int32_t *alive, int H, int R, int C, int by_rows, int thin_min,
+                             int64_t n_alive, int32_t *plan) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
-  const int64_t n_groups = (int64_t)H * NG;
+  const int64_t ng = (int64_t)H * NG, slots = ng + (int64_t)H * L;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
-  if (i >= n_groups) return;
-  const int h = (int)(i / NG), lg = (int)(i % NG);
-  // position in the sorted header: groups with more entries first, ties in natural order
+  if (i >= slots || !alive[i]) return;
+  // position in the sorted header: more entries first, ties in slot order
   const int mine = cnt[i];
   int64_t pos = 0;
-  for (int64_t j = 0; j < n_groups; j++) pos += (cnt[j] > mine) || (cnt[j] == mine && j < i);
+  for (int64_t j = 0; j < slots; j++) pos += alive[j] && ((cnt[j] > mine) || (cnt[j] == mine && j < i));
   int32_t *hd = plan + 4 * pos;
-  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = lg;
-  int32_t *e = plan + 4 * n_groups + (int64_t)(BSP_GROUP + 1) * start[i];
+  int32_t *e = plan + 4 * n_alive + (int64_t)(BSP_GROUP + 1) * start[i];
+  const bool chain = i >= ng;
+  const int h = chain ? (int)((i - ng) / L) : (int)(i / NG);
+  const int first = chain ? (int)((i - ng) % L) : (int)(i % NG) * BSP_GROUP;   // first (or only) line
+  bool use[BSP_GROUP];
+  int skip = 0;   // members of a group that are chains: bits 24.. of the group index field
+  for (int g = 0; g < BSP_GROUP; g++) {
+    const int line = first + g;
+    const bool thin = !chain && line < L && thin_line(linecnt, (int64_t)h * L + line, thin_min);
+    use[g] = chain ? g == 0 : (line < L && !thin);
+    skip |= thin ? 1 << g : 0;
+  }
+  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = chain ? -(first + 1) : (first / BSP_GROUP) | (skip << 24);
   for (int bb = 0; bb < B; bb++) {
-    // Column groups list their positions from the last one down: the long groups of a causal layout (global
+    // Column groups list their positions from the last one down: the long lines of a causal layout (global
     // columns) then walk the dense operand's rows in step with each other and share them in L2 (measured: 12 % fewer
     // bytes fetched from memory by the transposed products).
     const int b = by_rows ? bb : B - 1 - bb;
     int32_t bid[BSP_GROUP];
     bool any = false;
     for (int g = 0; g < BSP_GROUP; g++) {
-      const int line = lg * BSP_GROUP + g;
       bid[g] = -1;
-      if (line < L) {
-        const int64_t p = cell(R, C, h, line, b, by_rows);
+      if (use[g]) {
+        const int64_t p = cell(R, C, h, first + g, b, by_rows);
         if (lay[p] != 0) { bid[g] = rank[p]; any = true; }
       }
     }
@@ -572,35 +604,40 @@ extern "C" int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, i
 
 extern "C" int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows) {
   const int64_t L = by_rows ? R : C;
-  return 4 * (int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (BSP_GROUP + 1) * nnz;
+  return 4 * ((int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (int64_t)H * L) + (BSP_GROUP + 1) * nnz;
 }
 
-extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int32_t *d_plan, int64_t plan_cap,
-                                    void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream) {
+extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int32_t *d_plan,
+                                    int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len,
+                                    void *stream) {
   int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
   if (rc != BSP_OK) return rc;
-  if (!d_plan || !n_groups || !plan_len) return BSP_ERR_ARG;
+  if (!d_plan || !n_groups || !plan_len || thin_min < 0) return BSP_ERR_ARG;
   hipStream_t st = as_stream(stream);
   Ws o(H, R, C);
   int32_t *ws = (int32_t *)d_ws;
   const int T = 256;
   const int L = by_rows ? R : C;
-  const int64_t ng = (int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP);
+  const int64_t ng = (int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP), slots = ng + (int64_t)H * L;
   rc = prepare_counts(d_layout, H, R, C, ws, o, st);
   if (rc != BSP_OK) return rc;
+  if (!by_rows) hipLaunchKernelGGL(k_col_counts, dim3(cdiv((int64_t)H * C, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.colcnt);
+  const int32_t *linecnt = ws + (by_rows ? o.rowcnt : o.colcnt);
   hipLaunchKernelGGL(k_rank, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowstart, ws + o.rank);
-  // linepacks / segstart are free here: group entry counts and their prefix sums
-  hipLaunchKernelGGL(k_gplan_count, dim3(cdiv(ng, T)), dim3(T), 0, st, d_layout, H, R, C, by_rows, ws + o.linepacks);
-  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.linepacks, ws + o.segstart, ng, (int32_t *)nullptr);
+  hipLaunchKernelGGL(k_gplan_count, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, linecnt, H, R, C, by_rows, thin_min,
+                     ws + o.gcnt, ws + o.galive);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.gcnt, ws + o.gstart, slots, (int32_t *)nullptr);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.galive, ws + o.gapos, slots, (int32_t *)nullptr);
   BSP_LAUNCH_CHECK();
-  int32_t total = 0;
-  BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.segstart + ng, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  int32_t total = 0, n_alive = 0;
+  BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.gstart + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipMemcpyAsync(&n_alive, ws + o.gapos + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipStreamSynchronize(st));
-  *n_groups = (int)ng;
-  *plan_len = 4 * ng + (int64_t)(BSP_GROUP + 1) * total;
+  *n_groups = (int)n_alive;
+  *plan_len = 4 * (int64_t)n_alive + (int64_t)(BSP_GROUP + 1) * total;
   if (*plan_len > plan_cap) return BSP_ERR_CAPACITY;
-  hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(ng, T)), dim3(T), 0, st, d_layout, ws + o.rank, ws + o.linepacks, ws + o.segstart, H, R, C,
-                     by_rows, d_plan);
+  hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, ws + o.rank, linecnt, ws + o.gcnt, ws + o.gstart,
+                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, d_plan);
   BSP_LAUNCH_CHECK();
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;

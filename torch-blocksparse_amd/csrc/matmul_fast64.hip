@@ -340,6 +340,111 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   }
 }
 
+// A chain = one output line with many blocks (the plan builder takes such lines out of their groups).  Walking its
+// entries one after the other would make this workgroup the last to finish by far, so the four wavefronts split
+// the reduction instead: wavefront w takes entries w, w+4, ... and computes all 64 rows of the line for them, in its
+// own piece of LDS and without workgroup barriers; the four partial results are added through LDS at the end.
+template <typename T, bool SP_TRANS>
+__device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int n0, int depth, int line, table_ptr ent, int ne) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int TILE = 64 * kLdsRow;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
+  const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
+  const int64_t ldd = g.ldd;
+  T *Yw = smem + wave * TILE;
+  T *Xw = smem + (4 + wave) * TILE;              // used only when the sparse operand is read transposed
+  const int lr = lane >> 3, lc = (lane & 7) * 8;  // a lane's row (of 8) and 16-byte column chunk in a 64 x 64 tile
+  u32x4 y[8], x[8];
+  auto issue = [&](int e) {
+    const table_ptr en = ent + (G + 1) * e;
+    const T *py = dn + ((int64_t)en[0] * 64 + lr) * ldd + lc;
+#pragma unroll
+    for (int i = 0; i < 8; i++) y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)i * 8 * ldd);
+    const T *blk = sp + (int64_t)en[1] * 4096;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+      if constexpr (SP_TRANS) x[i] = *reinterpret_cast<const u32x4 *>(blk + (i * 8 + lr) * 64 + lc);   // as stored, [k][m]
+      else x[i] = *reinterpret_cast<const u32x4 *>(blk + ((i >> 1) * 16 + (lane & 15)) * 64 + 32 * (i & 1) + (lane >> 4) * 8);   // operand layout
+    }
+  };
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[mt][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int tr_row = (lane >> 4) * 8 + ((lane & 15) >> 2), tr_col = (lane & 3) * 4;
+  const int mine = (ne - wave + 3) / 4;          // entries wave, wave + 4, ...
+  if (mine > 0) issue(wave);
+  for (int k = 0; k < mine; k++) {
+#pragma unroll
+    for (int i = 0; i < 8; i++) *reinterpret_cast<u32x4 *>(&Yw[(i * 8 + lr) * kLdsRow + lc]) = y[i];
+    frag_t xf[4][2];
+    if constexpr (SP_TRANS) {
+#pragma unroll
+      for (int i = 0; i < 8; i++) *reinterpret_cast<u32x4 *>(&Xw[(i * 8 + lr) * kLdsRow + lc]) = x[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; i++) xf[i >> 1][i & 1] = __builtin_bit_cast(frag_t, x[i]);
+    }
+    // the LDS operations of one wavefront complete in order: no barrier between its own stores and loads
+    __builtin_amdgcn_wave_barrier();
+    frag_t yf[2][4];
+#pragma unroll
+    for (int s2 = 0; s2 < 2; s2++) {
+      const T *yrow = &Yw[(32 * s2 + tr_row) * kLdsRow + tr_col];
+#pragma unroll
+      for (int j = 0; j < 4; j++) yf[s2][j] = tr_frag<T>(yrow + 16 * j, yrow + 16 * j + 4 * kLdsRow);
+      if constexpr (SP_TRANS) {
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) {
+          const T *xrow = &Xw[(32 * s2 + tr_row) * kLdsRow + 16 * mt + tr_col];
+          xf[mt][s2] = tr_frag<T>(xrow, xrow + 4 * kLdsRow);
+        }
+      }
+    }
+    if (k + 1 < mine) issue(wave + 4 * (k + 1));   // the stage's registers are free again
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; s2++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[mt][j] = M::run(yf[s2][j], xf[mt][s2], acc[mt][j]);
+    __builtin_amdgcn_wave_barrier();
+  }
+  // add the four partial results: two rounds of 32 floats per lane and wavefront through LDS, after which wavefront w
+  // holds rows 16w.. of the line
+  float *red = reinterpret_cast<float *>(smem);   // [wavefront][32][lane], 32 KiB
+  f32x4 fin[4];
+#pragma unroll
+  for (int half = 0; half < 2; half++) {
+    __syncthreads();
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) red[(wave * 32 + (t * 4 + j) * 4 + c) * 64 + lane] = acc[2 * half + t][j][c];
+    __syncthreads();
+    if ((wave >> 1) == half) {
+      const int t = wave & 1;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < 4; w++) v += red[(w * 32 + (t * 4 + j) * 4 + c) * 64 + lane];
+          fin[j][c] = v;
+        }
+    }
+  }
+  __syncthreads();
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
+  store_slice<T>(smem + (wave * 16) * kLdsRow, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, fin, lane);
+}
+
 // dsd / dds: members = output lines (block-rows of the result), entries = positions of the reduction
 template <typename T, bool SP_TRANS>
 __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
@@ -347,15 +452,22 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
   constexpr int RING = XSD_RING;
-  __shared__ __attribute__((aligned(16))) T Ys[2][TILE];
-  __shared__ __attribute__((aligned(16))) T Xs[SP_TRANS ? 2 : 1][SP_TRANS ? TILE : 8];
+  // groups: two dense tiles (+ two sparse tiles when read transposed); chains: one of each per wavefront
+  __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 4) * TILE];
+  T (*Ys)[TILE] = reinterpret_cast<T (*)[TILE]>(smem);
+  T (*Xs)[TILE] = reinterpret_cast<T (*)[TILE]>(smem + 2 * TILE);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int z = blockIdx.x % g.Z;
   const int64_t rest = blockIdx.x / g.Z;
   const int n0 = (int)(rest % g.n_tiles) * 64;
   const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
-  const int e0 = hd[0], ne = hd[1], depth = hd[2], lg = hd[3];
+  const int e0 = hd[0], ne = hd[1], depth = hd[2], code = hd[3];
   const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  if (code < 0) {   // a chain: the line -(code + 1) on its own
+    xsd_chain<T, SP_TRANS>(g, smem, z, n0, depth, -(code + 1), ent, ne);
+    return;
+  }
+  const int lg = code & 0xffffff, skip = code >> 24;   // members whose line is a chain are left to that chain
   const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;
@@ -463,7 +575,7 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
 #pragma unroll
   for (int m = 0; m < G; m++) {
     const int line = lg * G + m;
-    if (line < g.lines) store_slice<T>(cs, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, acc[m], lane);
+    if (line < g.lines && !((skip >> m) & 1)) store_slice<T>(cs, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, acc[m], lane);
   }
 }
 

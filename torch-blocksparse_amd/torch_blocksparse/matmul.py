@@ -50,7 +50,16 @@ class GroupPlan:
         self.table, self.n_groups, self.lines = table, n_groups, lines
 
     @staticmethod
-    def build(layout, by_rows, device):
+    def thin_min(layout, by_rows):
+        """Lines at least this long become chains: well above the average line, so that dense-ish layouts (whose
+        groups share every dense tile four times) keep their groups and only outliers such as global columns split."""
+        H, R, C = layout.shape
+        mean = float((layout != 0).sum()) / max(1, H * (R if by_rows else C))
+        return max(16, int(2 * mean + 0.5))
+
+    @staticmethod
+    def build(layout, by_rows, device, thin_min=None):
+        """thin_min: lines at least this long become chains; None = GroupPlan.thin_min(...), 0 = no chains."""
         lib = _lib.load()
         dev = torch.device(device)
         lay = _lib.layout_to_device(layout, dev)
@@ -60,7 +69,8 @@ class GroupPlan:
         cap = lib.bsp_group_plan_cap(H, R, C, nnz, int(bool(by_rows)))
         table = torch.empty((cap,), dtype=torch.int32, device=dev)
         n_groups, n = ctypes.c_int(0), ctypes.c_int64(0)
-        rc = lib.bsp_group_plan_build(_lib.ptr(lay), H, R, C, int(bool(by_rows)), _lib.ptr(table), cap, _lib.ptr(ws), ws_bytes,
+        thin = GroupPlan.thin_min(layout, by_rows) if thin_min is None else int(thin_min)
+        rc = lib.bsp_group_plan_build(_lib.ptr(lay), H, R, C, int(bool(by_rows)), thin, _lib.ptr(table), cap, _lib.ptr(ws), ws_bytes,
                                       ctypes.byref(n_groups), ctypes.byref(n), _lib.stream_ptr(dev))
         _lib.check(rc, 'bsp_group_plan_build')
         return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C)
@@ -119,7 +129,7 @@ class _sparse_matmul(torch.autograd.Function):
         luts, widths, out_packs = SddTables(), [], []
         luts.nnz = nnz
         if block == 64:
-            luts.gplan = GroupPlan.build(layout, True, dev)
+            luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0)
         done = 0
         for k in range(n_levels.value):
             p, r = int(packs[k]), int(rows[k])
