@@ -140,6 +140,25 @@ int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int m
 int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
                     int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream);
 
+/* ---------------------------------------------------------------------------------------------------
+ * Dense utility ops of the reference package.
+ * ReLU: replaces the relu_y / relu_dxdsdbdres kernels and their launches (relu.py:8-91).  All tensors hold n
+ * elements in the same memory order; scale and bias are one-element device tensors of the data type (the
+ * reference reads them on the host with .item(); here nothing synchronises).
+ *   forward : y = max(x*scale + bias + res, 0)
+ *   backward: du = (y > 0) ? dy : 0; dx = du*scale; dres = du; *d_dbias = sum(du); *d_dscale = sum(du*x), both in
+ *             fp32, added in a fixed order (the reference uses floating-point atomics); d_ws is scratch of at
+ *             least bsp_relu_workspace_bytes() bytes. */
+int64_t bsp_relu_workspace_bytes(void);
+int bsp_relu_fwd(int dtype, const void *x, const void *res, void *y, const void *d_scale, const void *d_bias, int64_t n,
+                 void *stream);
+int bsp_relu_bwd(int dtype, const void *x, const void *y, const void *dy, void *dx, void *dres, const void *d_scale,
+                 float *d_dscale, float *d_dbias, void *d_ws, int64_t ws_bytes, int64_t n, void *stream);
+
+/* Permutation: replaces the permute kernel of permute.py:5-30, 45-93.  NCHW -> CHWN is the transposition of an
+ * [N, C*H*W] matrix, CHWN -> NCHW that of a [C*H*W, N] matrix: y[c*rows + r] = x[r*cols + c]. */
+int bsp_transpose(int dtype, const void *x, void *y, int64_t rows, int64_t cols, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -13,7 +13,7 @@ CSRC = os.path.join(HERE, 'csrc')
 LIBDIR = os.path.join(HERE, 'lib')
 OBJDIR = os.path.join(HERE, 'build')
 LIBNAME = 'libbsp_hip.so'
-SOURCES = ['lut.hip', 'softmax.hip', 'matmul_f16.hip', 'matmul_bf16.hip', 'matmul_f32.hip', 'matmul_fast64.hip', 'capi.hip']
+SOURCES = ['lut.hip', 'softmax.hip', 'matmul_f16.hip', 'matmul_bf16.hip', 'matmul_f32.hip', 'matmul_fast64.hip', 'elementwise.hip', 'capi.hip']
 FLAGS = ['--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-fno-gpu-rdc', '-Wall', '-Wno-unused-function',
          # packed-fp32 instruction selection is switched off on purpose
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']

@@ -46,6 +46,10 @@ SIGNATURES = {
     'bsp_softmax_fwd': (_i, [_i, _vp, _f, _vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _i, _vp, _i64, _i, _i, _i, _i, _i,
                              _i64, _vp]),
     'bsp_softmax_bwd': (_i, [_i, _vp, _vp, _f, _vp, _i, _i, _i, _i, _i, _i64, _i64, _vp]),
+    'bsp_relu_workspace_bytes': (_i64, []),
+    'bsp_relu_fwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    'bsp_relu_bwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp]),
+    'bsp_transpose': (_i, [_i, _vp, _vp, _i64, _i64, _vp]),
 }
 
 _lib = None
