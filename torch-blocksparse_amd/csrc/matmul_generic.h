@@ -87,8 +87,7 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
 
   // Every thread issues exactly ITER loads whatever the tile holds (chunks outside the operand read a dummy line
   // and are zeroed afterwards): with a fixed count the wait before a stage is consumed is exact.
-  template <class View> __device__ __forceinline__ void load(const View &v, int k0, int tid) {
-    const auto st = v.step(k0);   // what is uniform for the whole reduction step (table look-ups), kept scalar
+  template <class View> __device__ __forceinline__ void load(const View &v, const typename View::Step &st, int tid) {
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
       int c = tid + it * NT;
@@ -178,9 +177,11 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
     YL yl[NS];
 #pragma unroll
     for (int u = 0; u < NS; u++) {
-      xl[u].load(xv, u * TK, tid);
-      yl[u].load(yv, u * TK, tid);
+      xl[u].load(xv, xv.step(u * TK), tid);
+      yl[u].load(yv, yv.step(u * TK), tid);
     }
+    auto xst = xv.step(NS * TK);
+    auto yst = yv.step(NS * TK);
     for (int s0 = 0; s0 < ksteps; s0 += NS) {
 #pragma unroll
       for (int u = 0; u < NS; u++) {
@@ -206,8 +207,14 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
               }
           }
         }
-        xl[u].load(xv, (s + NS) * TK, tid);   // refill the slot only after its contents are dead
-        yl[u].load(yv, (s + NS) * TK, tid);
+        // The table look-ups run one step ahead of the refill that uses them: started here, needed a whole step
+        // later, their (scalar) latency is not in front of the loads.
+        const auto xnext = xv.step((s + NS + 1) * TK);
+        const auto ynext = yv.step((s + NS + 1) * TK);
+        xl[u].load(xv, xst, tid);   // refill the slot only after its contents are dead
+        yl[u].load(yv, yst, tid);
+        xst = xnext;
+        yst = ynext;
       }
     }
     // a lane's values come in groups of 4 consecutive result rows: row 4*(lane/16) (MS 16) or 8*g + 4*(lane/32) (MS 32)
@@ -322,25 +329,33 @@ struct XsdArgs {
 // A reduction step of TK elements lies inside one block (BLOCK >= TK) or covers TK / BLOCK whole blocks.
 template <typename T, int BLOCK> struct StepBlocks { static constexpr int TK = TileK<T>::TK, NB = TK > BLOCK ? TK / BLOCK : 1; };
 
+// The Step of a view holds the raw table values only; all arithmetic on them happens when the addresses are formed,
+// so that a look-up started one step ahead is not waited for before it is needed.
 template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m, k) of the segment's blocks
   const T *base; table_ptr plan; int nblk;
   static constexpr int NB = StepBlocks<T, BLOCK>::NB;
-  struct Step { const T *blk[NB]; int kin; };                      // block base pointers (nullptr past the end), offset inside
+  struct Step { int32_t bid[NB]; bool live[NB]; int kin; };        // storage index of each block, whether it exists, offset inside
   __device__ __forceinline__ Step step(int k0) const {
     Step st;
     st.kin = k0 % BLOCK;
 #pragma unroll
     for (int i = 0; i < NB; i++) {
       const int ord = k0 / BLOCK + i;
-      st.blk[i] = ord < nblk ? base + (int64_t)plan[2 * ord + 1] * (BLOCK * BLOCK) : nullptr;
+      // unconditional read of a clamped index (nblk >= 1): a load under a branch could not be started early
+      st.bid[i] = plan[2 * (ord < nblk ? ord : nblk - 1) + 1];
+      st.live[i] = ord < nblk;
     }
     return st;
   }
   __device__ __forceinline__ const T *pick(const Step &st, int k) const {
-    const T *b = st.blk[0];
+    int32_t b = st.bid[0];
+    bool live = st.live[0];
 #pragma unroll
-    for (int i = 1; i < NB; i++) b = (k / BLOCK == i) ? st.blk[i] : b;
-    return b;
+    for (int i = 1; i < NB; i++) {
+      b = (k / BLOCK == i) ? st.bid[i] : b;
+      live = (k / BLOCK == i) ? st.live[i] : live;
+    }
+    return live ? base + (int64_t)b * (BLOCK * BLOCK) : nullptr;
   }
   __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [m][k]
     const T *b = pick(st, k);
@@ -355,21 +370,27 @@ template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m
 template <typename T, int BLOCK> struct DenseView {                   // element (n, k): dense row/col n, reduction position k
   const T *base; table_ptr plan; int nblk; int64_t ld; int n0, NF;
   static constexpr int NB = StepBlocks<T, BLOCK>::NB;
-  struct Step { int64_t pos[NB]; };                                   // position of each block in the dense operand, -1 past the end
+  struct Step { int32_t pos[NB]; bool live[NB]; int kin; };           // position of each block in the dense operand, whether it exists
   __device__ __forceinline__ Step step(int k0) const {
     Step st;
+    st.kin = k0 % BLOCK;
 #pragma unroll
     for (int i = 0; i < NB; i++) {
       const int ord = k0 / BLOCK + i;
-      st.pos[i] = ord < nblk ? (int64_t)plan[2 * ord] + k0 % BLOCK : -1;
+      st.pos[i] = plan[2 * (ord < nblk ? ord : nblk - 1)];
+      st.live[i] = ord < nblk;
     }
     return st;
   }
   __device__ __forceinline__ int64_t pick(const Step &st, int k) const {
-    int64_t p = st.pos[0];
+    int32_t p = st.pos[0];
+    bool live = st.live[0];
 #pragma unroll
-    for (int i = 1; i < NB; i++) p = (k / BLOCK == i) ? st.pos[i] : p;
-    return p;
+    for (int i = 1; i < NB; i++) {
+      p = (k / BLOCK == i) ? st.pos[i] : p;
+      live = (k / BLOCK == i) ? st.live[i] : live;
+    }
+    return live ? (int64_t)p + st.kin : -1;
   }
   __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [n][k]
     const int64_t p = pick(st, k);
@@ -422,6 +443,14 @@ __global__ void __launch_bounds__(256) k_xsd(XsdArgs g) {
     if constexpr (OUT_NCONTIG) store4<T>(oz + ((int64_t)column * BLOCK + m) * ldo + n0 + n, v);
     else store4<T>(oz + (int64_t)(n0 + n) * ldo + column * BLOCK + m, v);
   };
+  if (nblk == 0) {   // nothing to read (the views below assume at least one block): write the zeros and leave
+    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
+    for (int i = threadIdx.x; i < BLOCK * S::TN / 4; i += 256) {
+      if constexpr (OUT_NCONTIG) store(i / (S::TN / 4), (i % (S::TN / 4)) * 4, zero);
+      else store((i % (BLOCK / 4)) * 4, i / (BLOCK / 4), zero);
+    }
+    return;
+  }
   G::run(sv, dv, (nblk * BLOCK + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
 }
 
