@@ -66,10 +66,16 @@ template <typename T> struct TileK { static constexpr int TK = 64 / sizeof(T), P
 
 // ---------------------------------------------------------------------------------------------------------
 // One operand tile: ROWS x TK, fetched by NT threads in 16-byte chunks, kept in registers until the LDS
-// buffer is free.  View::step(k0) -> the part of the addressing that is uniform for the reduction step starting at
-// k0; View::ptr_k(step, row, k) -> address of elements (row, k0+k .. k0+k+VE-1) or nullptr (zero fill);
-// View::ptr_r(step, row, k) -> address of elements (row..row+VE-1, k0+k) or nullptr.
+// buffer is free.  The address of a chunk is split into the part that never changes for a thread (computed once, before
+// the reduction loop) and the part that is the same for all threads of a step (scalar arithmetic on the step's table
+// values): a load costs one 64-bit add, not the multiplications and selects of a full index computation.
+//   View::part_k(row, k) / part_r(row, k) -> Part{off, ok, sel, k}: element offset of chunk (row, k..k+VE-1) resp.
+//     (row..row+VE-1, k) inside the step, whether the rows exist, which of the step's blocks it belongs to
+//   View::step(k0) -> Step{..., live[NB], klim}: raw table values of the reduction step starting at k0
+//   View::scalar_k(step, i) / scalar_r(step, i) -> element offset of block i of the step
 // ---------------------------------------------------------------------------------------------------------
+struct Part { int64_t off; bool ok; int sel; int k; };
+
 template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   static constexpr int TK = TileK<T>::TK, LDK = TK + TileK<T>::PAD;
   static constexpr int VE = 16 / sizeof(T);
@@ -85,20 +91,6 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   u32x4 reg[ITER];
   bool ok[ITER];
 
-  // Every thread issues exactly ITER loads whatever the tile holds (chunks outside the operand read a dummy line
-  // and are zeroed afterwards): with a fixed count the wait before a stage is consumed is exact.
-  template <class View> __device__ __forceinline__ void load(const View &v, const typename View::Step &st, int tid) {
-#pragma unroll
-    for (int it = 0; it < ITER; it++) {
-      int c = tid + it * NT;
-      if (NCH % NT != 0 && c >= NCH) c = NCH - 1;
-      const T *p;
-      if constexpr (KCONTIG) p = v.ptr_k(st, c / CPR, (c % CPR) * VE);
-      else p = v.ptr_r(st, (c % RCH) * VE, c / RCH);
-      ok[it] = p != nullptr;            // zero-filling happens when the stage is consumed, not here: a use of the loaded
-      reg[it] = *reinterpret_cast<const u32x4 *>(p ? p : v.base);   // value right away would make the wait for it immediate
-    }
-  }
   __device__ __forceinline__ void store(T *S, int tid) const {
 #pragma unroll
     for (int it = 0; it < ITER; it++) {
@@ -139,6 +131,42 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   }
 };
 
+// The thread-invariant half of a loader's addressing (one per operand, shared by all ring stages).
+template <typename T, int ROWS, int NT, bool KCONTIG> struct TileAddr {
+  typedef TileLoader<T, ROWS, NT, KCONTIG> L;
+  Part part[L::ITER];
+  template <class View> __device__ __forceinline__ void init(const View &v, int tid) {
+#pragma unroll
+    for (int it = 0; it < L::ITER; it++) {
+      int c = tid + it * NT;
+      if (L::NCH % NT != 0 && c >= L::NCH) c = L::NCH - 1;
+      if constexpr (KCONTIG) part[it] = v.part_k(c / L::CPR, (c % L::CPR) * L::VE);
+      else part[it] = v.part_r((c % L::RCH) * L::VE, c / L::RCH);
+    }
+  }
+  // Every thread issues exactly ITER loads whatever the tile holds (chunks outside the operand read a dummy line
+  // and are zeroed afterwards): with a fixed count the wait before a stage is consumed is exact.
+  template <class View> __device__ __forceinline__ void load(L &dst, const View &v, const typename View::Step &st) const {
+    constexpr int NB = View::NB;
+    int64_t so[NB];
+#pragma unroll
+    for (int i = 0; i < NB; i++) so[i] = KCONTIG ? v.scalar_k(st, i) : v.scalar_r(st, i);
+#pragma unroll
+    for (int it = 0; it < L::ITER; it++) {
+      int64_t o = so[0];
+      bool live = st.live[0];
+#pragma unroll
+      for (int i = 1; i < NB; i++) {
+        o = part[it].sel == i ? so[i] : o;
+        live = part[it].sel == i ? st.live[i] : live;
+      }
+      const bool good = part[it].ok && live && part[it].k < st.klim;
+      dst.ok[it] = good;                // zero-filling happens when the stage is consumed, not here: a use of the loaded
+      dst.reg[it] = *reinterpret_cast<const u32x4 *>(good ? v.base + part[it].off + o : v.base);   // value right away would make the wait for it immediate
+    }
+  }
+};
+
 // ---------------------------------------------------------------------------------------------------------
 // The tile product.  X supplies TM rows ("m"), Y supplies TN rows ("n"); out(m, n) = sum_k X(m,k) * Y(n,k).
 // WGM x WGN wavefronts, each RM x RN MFMA tiles.  OUT_NCONTIG chooses which index the four values of a lane
@@ -170,51 +198,63 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
       for (int j = 0; j < RN; j++)
 #pragma unroll
         for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
-    // Register ring of NS stages: global loads run NS - 1 reduction steps ahead of the MFMAs; two LDS buffers, one
-    // barrier per step.  The loop runs whole rounds of NS steps; steps past the end load zeros and skip the MFMAs.
+    // Register ring of NS stages: global loads run NS - 1 reduction steps ahead of their use; two LDS buffers, one
+    // barrier per step.  Step s first writes stage s + 1 to the other LDS buffer, then reads stage s and issues its
+    // MFMAs, then refills the ring slot it has just emptied, and only then meets the barrier: the LDS write and the
+    // barrier wait pass while the matrix pipe works instead of in front of it.  The loop runs whole rounds of NS
+    // steps; steps past the end hold zeros.
     constexpr int NS = 4;
+    static_assert(NS % 2 == 0, "the LDS buffer of a step is chosen by the ring slot's parity");
     XL xl[NS];
     YL yl[NS];
+    TileAddr<T, TM, NT, X_KCONTIG> xa;
+    TileAddr<T, TN, NT, Y_KCONTIG> ya;
+    xa.init(xv, tid);
+    ya.init(yv, tid);
 #pragma unroll
     for (int u = 0; u < NS; u++) {
-      xl[u].load(xv, xv.step(u * TK), tid);
-      yl[u].load(yv, yv.step(u * TK), tid);
+      xa.load(xl[u], xv, xv.step(u * TK));
+      ya.load(yl[u], yv, yv.step(u * TK));
     }
-    auto xst = xv.step(NS * TK);
-    auto yst = yv.step(NS * TK);
+    xl[0].store(Xs[0], tid);
+    yl[0].store(Ys[0], tid);
+    xa.load(xl[0], xv, xv.step(NS * TK));
+    ya.load(yl[0], yv, yv.step(NS * TK));
+    // The table look-ups run one step ahead of the refill that uses them: started a whole step before they are needed,
+    // their (scalar) latency is not in front of the loads.
+    auto xst = xv.step((NS + 1) * TK);
+    auto yst = yv.step((NS + 1) * TK);
+    __syncthreads();
     for (int s0 = 0; s0 < ksteps; s0 += NS) {
 #pragma unroll
       for (int u = 0; u < NS; u++) {
         const int s = s0 + u;
-        const int cur = u & 1;
-        xl[u].store(Xs[cur], tid);   // this buffer was last read two steps ago, before the previous barrier
-        yl[u].store(Ys[cur], tid);
-        __syncthreads();
-        if (s < ksteps) {
+        const int cur = u & 1, nxt = cur ^ 1, u1 = (u + 1) % NS;
+        xl[u1].store(Xs[nxt], tid);   // stage s + 1; this buffer was last read in step s - 1, before the previous barrier
+        yl[u1].store(Ys[nxt], tid);
+        // (steps past the end multiply zeros: cheaper than a branch, which would copy the accumulators around)
 #pragma unroll
-          for (int kk = 0; kk < TK / M::KSTEP; kk++) {
-            typename M::frag_t xf[RM], yf[RN];
+        for (int kk = 0; kk < TK / M::KSTEP; kk++) {
+          typename M::frag_t xf[RM], yf[RN];
 #pragma unroll
-            for (int i = 0; i < RM; i++) xf[i] = XL::template frag<MS, M>(Xs[cur], (wm * RM + i) * MS, kk, lane);
+          for (int i = 0; i < RM; i++) xf[i] = XL::template frag<MS, M>(Xs[cur], (wm * RM + i) * MS, kk, lane);
 #pragma unroll
-            for (int j = 0; j < RN; j++) yf[j] = YL::template frag<MS, M>(Ys[cur], (wn * RN + j) * MS, kk, lane);
+          for (int j = 0; j < RN; j++) yf[j] = YL::template frag<MS, M>(Ys[cur], (wn * RN + j) * MS, kk, lane);
 #pragma unroll
-            for (int i = 0; i < RM; i++)
+          for (int i = 0; i < RM; i++)
 #pragma unroll
-              for (int j = 0; j < RN; j++) {
-                if constexpr (OUT_NCONTIG) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // result rows = n, column = m
-                else acc[i][j] = M::run(xf[i], yf[j], acc[i][j]);                          // result rows = m, column = n
-              }
-          }
+            for (int j = 0; j < RN; j++) {
+              if constexpr (OUT_NCONTIG) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // result rows = n, column = m
+              else acc[i][j] = M::run(xf[i], yf[j], acc[i][j]);                          // result rows = m, column = n
+            }
         }
-        // The table look-ups run one step ahead of the refill that uses them: started here, needed a whole step
-        // later, their (scalar) latency is not in front of the loads.
-        const auto xnext = xv.step((s + NS + 1) * TK);
-        const auto ynext = yv.step((s + NS + 1) * TK);
-        xl[u].load(xv, xst, tid);   // refill the slot only after its contents are dead
-        yl[u].load(yv, yst, tid);
+        const auto xnext = xv.step((s + NS + 2) * TK);
+        const auto ynext = yv.step((s + NS + 2) * TK);
+        xa.load(xl[u1], xv, xst);   // stage s + 1 + NS into the slot emptied above
+        ya.load(yl[u1], yv, yst);
         xst = xnext;
         yst = ynext;
+        __syncthreads();
       }
     }
     // a lane's values come in groups of 4 consecutive result rows: row 4*(lane/16) (MS 16) or 8*g + 4*(lane/32) (MS 32)
@@ -262,20 +302,19 @@ struct SddArgs {
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
   const T *base; int64_t ld; int K; int idx[PACK];   // base doubles as the dummy address of out-of-range chunks
-  struct Step { int k0; };
-  __device__ __forceinline__ Step step(int k0) const { return Step{k0}; }
+  static constexpr int NB = 1;
+  struct Step { int k0; bool live[1]; int klim; };
+  __device__ __forceinline__ Step step(int k0) const { return Step{k0, {true}, K - k0}; }
   __device__ __forceinline__ int blk(int row) const {
     int r = idx[0];
 #pragma unroll
     for (int p = 1; p < PACK; p++) r = (row / BLOCK == p) ? idx[p] : r;
     return r * BLOCK + row % BLOCK;
   }
-  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {
-    return st.k0 + k < K ? base + (int64_t)blk(row) * ld + st.k0 + k : nullptr;
-  }
-  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {
-    return st.k0 + k < K ? base + (int64_t)(st.k0 + k) * ld + blk(row) : nullptr;
-  }
+  __device__ __forceinline__ Part part_k(int row, int k) const { return Part{(int64_t)blk(row) * ld + k, true, 0, k}; }
+  __device__ __forceinline__ Part part_r(int row, int k) const { return Part{(int64_t)k * ld + blk(row), true, 0, k}; }
+  __device__ __forceinline__ int64_t scalar_k(const Step &st, int) const { return st.k0; }
+  __device__ __forceinline__ int64_t scalar_r(const Step &st, int) const { return (int64_t)st.k0 * ld; }
 };
 
 template <int T_> struct SddShape { static constexpr int WG = T_ >= 32 ? 2 : 1; };
@@ -334,10 +373,11 @@ template <typename T, int BLOCK> struct StepBlocks { static constexpr int TK = T
 template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m, k) of the segment's blocks
   const T *base; table_ptr plan; int nblk;
   static constexpr int NB = StepBlocks<T, BLOCK>::NB;
-  struct Step { int32_t bid[NB]; bool live[NB]; int kin; };        // storage index of each block, whether it exists, offset inside
+  struct Step { int32_t bid[NB]; bool live[NB]; int kin; int klim; };   // storage index of each block, whether it exists, offset inside
   __device__ __forceinline__ Step step(int k0) const {
     Step st;
     st.kin = k0 % BLOCK;
+    st.klim = 1 << 30;
 #pragma unroll
     for (int i = 0; i < NB; i++) {
       const int ord = k0 / BLOCK + i;
@@ -347,33 +387,21 @@ template <typename T, int BLOCK, bool TRANS> struct SparseView {   // element (m
     }
     return st;
   }
-  __device__ __forceinline__ const T *pick(const Step &st, int k) const {
-    int32_t b = st.bid[0];
-    bool live = st.live[0];
-#pragma unroll
-    for (int i = 1; i < NB; i++) {
-      b = (k / BLOCK == i) ? st.bid[i] : b;
-      live = (k / BLOCK == i) ? st.live[i] : live;
-    }
-    return live ? base + (int64_t)b * (BLOCK * BLOCK) : nullptr;
-  }
-  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [m][k]
-    const T *b = pick(st, k);
-    return b ? b + row * BLOCK + (st.kin + k) % BLOCK : nullptr;
-  }
-  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {   // stored [k][m]
-    const T *b = pick(st, k);
-    return b ? b + ((st.kin + k) % BLOCK) * BLOCK + row : nullptr;
-  }
+  // stored [m][k] (part_k) or [k][m] (part_r); k / BLOCK picks the block when a step spans several
+  __device__ __forceinline__ Part part_k(int row, int k) const { return Part{(int64_t)row * BLOCK + k % BLOCK, true, k / BLOCK, k}; }
+  __device__ __forceinline__ Part part_r(int row, int k) const { return Part{(int64_t)(k % BLOCK) * BLOCK + row, true, k / BLOCK, k}; }
+  __device__ __forceinline__ int64_t scalar_k(const Step &st, int i) const { return (int64_t)st.bid[i] * (BLOCK * BLOCK) + st.kin; }
+  __device__ __forceinline__ int64_t scalar_r(const Step &st, int i) const { return (int64_t)st.bid[i] * (BLOCK * BLOCK) + st.kin * BLOCK; }
 };
 
 template <typename T, int BLOCK> struct DenseView {                   // element (n, k): dense row/col n, reduction position k
   const T *base; table_ptr plan; int nblk; int64_t ld; int n0, NF;
   static constexpr int NB = StepBlocks<T, BLOCK>::NB;
-  struct Step { int32_t pos[NB]; bool live[NB]; int kin; };           // position of each block in the dense operand, whether it exists
+  struct Step { int32_t pos[NB]; bool live[NB]; int kin; int klim; };  // position of each block in the dense operand, whether it exists
   __device__ __forceinline__ Step step(int k0) const {
     Step st;
     st.kin = k0 % BLOCK;
+    st.klim = 1 << 30;
 #pragma unroll
     for (int i = 0; i < NB; i++) {
       const int ord = k0 / BLOCK + i;
@@ -382,24 +410,11 @@ template <typename T, int BLOCK> struct DenseView {                   // element
     }
     return st;
   }
-  __device__ __forceinline__ int64_t pick(const Step &st, int k) const {
-    int32_t p = st.pos[0];
-    bool live = st.live[0];
-#pragma unroll
-    for (int i = 1; i < NB; i++) {
-      p = (k / BLOCK == i) ? st.pos[i] : p;
-      live = (k / BLOCK == i) ? st.live[i] : live;
-    }
-    return live ? (int64_t)p + st.kin : -1;
-  }
-  __device__ __forceinline__ const T *ptr_k(const Step &st, int row, int k) const {   // stored [n][k]
-    const int64_t p = pick(st, k);
-    return (n0 + row < NF && p >= 0) ? base + (int64_t)(n0 + row) * ld + p + k % BLOCK : nullptr;
-  }
-  __device__ __forceinline__ const T *ptr_r(const Step &st, int row, int k) const {   // stored [k][n]
-    const int64_t p = pick(st, k);
-    return (n0 + row < NF && p >= 0) ? base + (p + k % BLOCK) * ld + n0 + row : nullptr;
-  }
+  // stored [n][k] (part_k) or [k][n] (part_r); rows past the free dimension are zero-filled
+  __device__ __forceinline__ Part part_k(int row, int k) const { return Part{(int64_t)(n0 + row) * ld + k % BLOCK, n0 + row < NF, k / BLOCK, k}; }
+  __device__ __forceinline__ Part part_r(int row, int k) const { return Part{(int64_t)(k % BLOCK) * ld + n0 + row, n0 + row < NF, k / BLOCK, k}; }
+  __device__ __forceinline__ int64_t scalar_k(const Step &st, int i) const { return (int64_t)st.pos[i] + st.kin; }
+  __device__ __forceinline__ int64_t scalar_r(const Step &st, int i) const { return ((int64_t)st.pos[i] + st.kin) * ld; }
 };
 
 template <int BLOCK> struct XsdShape {
