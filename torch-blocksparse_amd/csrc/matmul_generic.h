@@ -198,12 +198,13 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
       for (int j = 0; j < RN; j++)
 #pragma unroll
         for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
-    // Register ring of NS stages: global loads run NS - 1 reduction steps ahead of their use; two LDS buffers, one
+    // Register ring of NS stages (two: deeper rings were measured slower or equal, the loop is not waiting for its
+    // loads): global loads run NS - 1 reduction steps ahead of their use; two LDS buffers, one
     // barrier per step.  Step s first writes stage s + 1 to the other LDS buffer, then reads stage s and issues its
     // MFMAs, then refills the ring slot it has just emptied, and only then meets the barrier: the LDS write and the
     // barrier wait pass while the matrix pipe works instead of in front of it.  The loop runs whole rounds of NS
     // steps; steps past the end hold zeros.
-    constexpr int NS = 4;
+    constexpr int NS = 2;
     static_assert(NS % 2 == 0, "the LDS buffer of a step is chosen by the ring slot's parity");
     XL xl[NS];
     YL yl[NS];
@@ -418,13 +419,14 @@ template <typename T, int BLOCK> struct DenseView {                   // element
 };
 
 template <int BLOCK> struct XsdShape {
-  static constexpr int TN = BLOCK >= 32 ? 128 : 64;      // tile of the dense free dimension
-  static constexpr int WGM = BLOCK >= 64 ? 2 : 1;        // 32 -> 1x4 wavefronts of 32x32; 64 -> 2x2 of 32x64; 128 -> 2x2 of 64x64
+  static constexpr int TN = BLOCK >= 128 ? 256 : BLOCK >= 32 ? 128 : 64;      // tile of the dense free dimension
+  static constexpr int WGM = BLOCK >= 64 ? 2 : 1;        // 32 -> 1x4 wavefronts of 32x32; 64 -> 2x2 of 32x64; 128 -> 2x2 of 64x128
   static constexpr int WGN = 4 / WGM;
 };
 
+// (at least two wavefronts per SIMD: the 128 x 256 tile of block 128 would otherwise take 266 registers and run alone)
 template <typename T, int BLOCK, bool SP_TRANS, bool DN_KCONTIG, bool OUT_NCONTIG>
-__global__ void __launch_bounds__(256) k_xsd(XsdArgs g) {
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_xsd(XsdArgs g) {
   typedef XsdShape<BLOCK> S;
   typedef TileGemm<T, BLOCK, S::TN, S::WGM, S::WGN, !SP_TRANS, DN_KCONTIG, OUT_NCONTIG> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
