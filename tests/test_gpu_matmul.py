@@ -108,6 +108,15 @@ def test_long_lines_become_chains(mode, trans_a, trans_b, dtype):
         run_case(mode, trans_a, trans_b, 64, dtype, Z=Z, H=H, M=F, N=64 * C, K=64 * R, layout=lay, seed=5, dist='randn', scale=0.25)
 
 
+@pytest.mark.parametrize('Z', [1, 4])
+def test_block128_sdd_one_or_four_workgroups_per_block(Z):
+    # 128 blocks: with Z = 4 there are 512 block products and each gets one workgroup; with Z = 1 every block is split
+    # into four 64 x 64 workgroups so that the chip is not left half empty
+    lay = torch.ones(2, 8, 8, dtype=torch.int64)
+    run_case('sdd', True, False, 128, torch.float16, Z=Z, H=2, M=1024, N=1024, K=64, layout=lay, seed=9, backward=False)
+    run_case('sdd', False, True, 128, torch.bfloat16, Z=Z, H=2, M=1024, N=1024, K=48, layout=lay, seed=10, backward=False)
+
+
 def test_degenerate_layouts():
     # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
     lay = torch.zeros(2, 4, 6, dtype=torch.int64)

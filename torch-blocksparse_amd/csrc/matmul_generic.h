@@ -303,6 +303,7 @@ struct SddArgs {
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
   const T *base; int64_t ld; int K; int idx[PACK];   // base doubles as the dummy address of out-of-range chunks
+  int off = 0;                                        // first row of the tile inside its block (tiles smaller than a block)
   static constexpr int NB = 1;
   struct Step { int k0; bool live[1]; int klim; };
   __device__ __forceinline__ Step step(int k0) const { return Step{k0, {true}, K - k0}; }
@@ -310,7 +311,7 @@ template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
     int r = idx[0];
 #pragma unroll
     for (int p = 1; p < PACK; p++) r = (row / BLOCK == p) ? idx[p] : r;
-    return r * BLOCK + row % BLOCK;
+    return r * BLOCK + off + row % BLOCK;
   }
   __device__ __forceinline__ Part part_k(int row, int k) const { return Part{(int64_t)blk(row) * ld + k, true, 0, k}; }
   __device__ __forceinline__ Part part_r(int row, int k) const { return Part{(int64_t)k * ld + blk(row), true, 0, k}; }
@@ -348,6 +349,32 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
     const int64_t bk = e[ent * 4 + 3];
     store4<T>(cz + bk * (BLOCK * BLOCK) + (m % BLOCK) * BLOCK + n % BLOCK, v);
   };
+  G::run(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
+}
+
+// sdd with SPLIT x SPLIT workgroups per block (pack 1): for layouts with so few blocks that one workgroup per block
+// would leave most of the chip idle (a 10 % dense 32 x 32 layout of 128-blocks has 100 blocks for 256 CUs).  The
+// sub-tiles of a block are neighbours in the grid, so that they meet their shared operand rows in L2.
+template <typename T, int BLOCK, int SPLIT, bool A_KCONTIG, bool B_KCONTIG>
+__global__ void __launch_bounds__(64 * SddShape<BLOCK / SPLIT>::WG * SddShape<BLOCK / SPLIT>::WG) k_sdd_split(SddArgs g) {
+  constexpr int TT = BLOCK / SPLIT, WG = SddShape<TT>::WG;
+  typedef TileGemm<T, TT, TT, WG, WG, A_KCONTIG, B_KCONTIG, true> G;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  const int64_t n_wg = g.n_groups * g.Z * (SPLIT * SPLIT);
+  const int64_t w = xcd_remap(blockIdx.x, n_wg);
+  const int sub = (int)(w % (SPLIT * SPLIT));
+  const int z = (int)(w / (SPLIT * SPLIT) / g.n_groups);
+  const int64_t grp = w / (SPLIT * SPLIT) % g.n_groups;
+  const table_ptr e = as_table(g.lut) + grp * 4;
+  if (g.valid && !g.valid[grp]) return;
+  SddView<T, BLOCK, 1, A_KCONTIG> av;
+  SddView<T, BLOCK, 1, B_KCONTIG> bv;
+  av.base = reinterpret_cast<const T *>(g.a) + z * g.a_sz + e[0] * g.a_sh; av.ld = g.lda; av.K = g.K;
+  bv.base = reinterpret_cast<const T *>(g.b) + z * g.b_sz + e[0] * g.b_sh; bv.ld = g.ldb; bv.K = g.K;
+  av.idx[0] = e[1]; av.off = (sub / SPLIT) * TT;
+  bv.idx[0] = e[2]; bv.off = (sub % SPLIT) * TT;
+  T *cb = reinterpret_cast<T *>(g.c) + z * g.c_sz + (int64_t)e[3] * (BLOCK * BLOCK) + av.off * BLOCK + bv.off;
+  auto store = [&](int m, int n, f32x4 v) { store4<T>(cb + m * BLOCK + n, v); };
   G::run(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
 }
 
@@ -493,7 +520,25 @@ template <typename T, int BLOCK, int PACK> int launch_sdd_tp(const SddArgs &g, b
   return BSP_OK;
 }
 
+template <typename T, int BLOCK, int SPLIT> int launch_sdd_split(const SddArgs &g, bool a_kc, bool b_kc, hipStream_t st) {
+  constexpr int TT = BLOCK / SPLIT, WG = SddShape<TT>::WG;
+  const int64_t n_wg = g.n_groups * g.Z * (SPLIT * SPLIT);
+  if (n_wg <= 0) return BSP_OK;
+  dim3 grid((unsigned)n_wg), blockdim(64 * WG * WG);
+#define BSP_SDD_LAUNCH(AK, BK)                                                                                   \
+  hipLaunchKernelGGL((k_sdd_split<T, BLOCK, SPLIT, AK, BK>), grid, blockdim,                                    \
+                     (TileGemm<T, TT, TT, WG, WG, AK, BK, true>::SMEM_BYTES), st, g)
+  if (a_kc && b_kc) BSP_SDD_LAUNCH(true, true);
+  else if (a_kc && !b_kc) BSP_SDD_LAUNCH(true, false);
+  else if (!a_kc && b_kc) BSP_SDD_LAUNCH(false, true);
+  else BSP_SDD_LAUNCH(false, false);
+#undef BSP_SDD_LAUNCH
+  return BSP_OK;
+}
+
 template <typename T> int launch_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st) {
+  // fewer than two workgroups per CU: four 64 x 64 workgroups per 128-block instead of one
+  if (block == 128 && pack == 1 && g.n_groups * g.Z < 512) return launch_sdd_split<T, 128, 2>(g, a_kc, b_kc, st);
   if (block == 16 && pack == 4) return launch_sdd_tp<T, 16, 4>(g, a_kc, b_kc, st);
   if (block == 16 && pack == 2) return launch_sdd_tp<T, 16, 2>(g, a_kc, b_kc, st);
   if (block == 16 && pack == 1) return launch_sdd_tp<T, 16, 1>(g, a_kc, b_kc, st);
