@@ -31,8 +31,8 @@ MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 # measured for this build of the kernel.
 TRAFFIC_BYTES = {
     'sdd_fwd  q.k^T': 140072457 + 268435460, 'sdd_bwd  do.v^T': 140072457 + 268435460,
-    'dsd_fwd  p.v': 342691472 + 67108864, 'dsd_bwd  ds.k': 342691472 + 67108864,
-    'dsd_bwd  p^T.do': 378216913 + 67108864, 'dds_bwd  (q^T.ds)^T': 378216913 + 67108864,
+    'dsd_fwd  p.v': 342712366 + 67108864, 'dsd_bwd  ds.k': 342712366 + 67108864,
+    'dsd_bwd  p^T.do': 394366158 + 67108864, 'dds_bwd  (q^T.ds)^T': 394366158 + 67108864,
     'softmax_fwd': 269785972 + 268435456, 'softmax_bwd': 538129920 + 268435456,
 }
 
