@@ -172,6 +172,12 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileAddr {
 // WGM x WGN wavefronts, each RM x RN MFMA tiles.  OUT_NCONTIG chooses which index the four values of a lane
 // run along, so that the epilogue writes 4 consecutive elements whatever the output orientation.
 // ---------------------------------------------------------------------------------------------------------
+constexpr int stage_tiles(int nc, int ms, int ve, int bytes_per_elem_all_waves, int limit) {
+  int cg = nc;
+  while (cg > 1 && ms * (cg * ms + ve) * bytes_per_elem_all_waves > limit) cg /= 2;
+  return cg;
+}
+
 template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_KCONTIG, bool OUT_NCONTIG> struct TileGemm {
   static constexpr int NT = 64 * WGM * WGN;
   static constexpr int TK = TileK<T>::TK, LDK = TK + TileK<T>::PAD;
@@ -258,33 +264,53 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
         __syncthreads();
       }
     }
-    // a lane's values come in groups of 4 consecutive result rows: row 4*(lane/16) (MS 16) or 8*g + 4*(lane/32) (MS 32)
+    // Epilogue.  A lane's values come in groups of 4 consecutive positions along the output's contiguous index
+    // (4*(lane/16) for MS 16, 8*g + 4*(lane/32) for MS 32) at row lane % MS of a tile, so a direct store would write
+    // 8- or 16-byte pieces of 32 different rows per instruction.  Each wavefront instead passes one row of tiles at a
+    // time through its own piece of LDS (free after the last barrier) and writes whole 16-byte chunks, consecutive
+    // lanes along a row.  store(r, c, chunk): r = row (m if OUT_NCONTIG, else n), c = first of VE consecutive columns.
+    constexpr int VE = 16 / (int)sizeof(T);
+    constexpr int NR = OUT_NCONTIG ? RM : RN, NC = OUT_NCONTIG ? RN : RM;   // tiles along the row / contiguous index
+    // tiles staged per pass: all NC of them if that fits the tile buffers, else half, a quarter ...
+    constexpr int CG = stage_tiles(NC, MS, VE, (int)sizeof(T) * WGM * WGN, SMEM_BYTES);
+    constexpr int CW = CG * MS, LDS_ROW = CW + VE;                            // staged row, padded by one chunk
+    static_assert(MS * LDS_ROW * (int)sizeof(T) * WGM * WGN <= SMEM_BYTES, "epilogue staging must fit the tile buffers");
+    T *stage = smem + wave * (MS * LDS_ROW);
+    const int cc = lane % MS;
+    const int r_wave = OUT_NCONTIG ? wm * RM * MS : wn * RN * MS, c_wave = OUT_NCONTIG ? wn * RN * MS : wm * RM * MS;
 #pragma unroll
-    for (int i = 0; i < RM; i++)
+    for (int pass = 0; pass < NR * (NC / CG); pass++) {
+      const int rt = pass / (NC / CG), c0 = (pass % (NC / CG)) * CG;
 #pragma unroll
-      for (int j = 0; j < RN; j++)
+      for (int ct = 0; ct < CG; ct++)
 #pragma unroll
         for (int g4 = 0; g4 < M::NACC / 4; g4++) {
-          const f32x4 v = {acc[i][j][4 * g4 + 0], acc[i][j][4 * g4 + 1], acc[i][j][4 * g4 + 2], acc[i][j][4 * g4 + 3]};
+          const typename M::acc_t &t = OUT_NCONTIG ? acc[rt][c0 + ct] : acc[c0 + ct][rt];
           const int rr = (MS == 16) ? 4 * (lane >> 4) : 8 * g4 + 4 * (lane >> 5);
-          const int cc = lane % MS;
-          const int m0 = (wm * RM + i) * MS, n0 = (wn * RN + j) * MS;
-          if constexpr (OUT_NCONTIG) store(m0 + cc, n0 + rr, v);
-          else store(m0 + rr, n0 + cc, v);
+          T *dst = stage + cc * LDS_ROW + ct * MS + rr;
+          if constexpr (sizeof(T) == 4) {
+            *reinterpret_cast<f32x4 *>(dst) = f32x4{t[4 * g4 + 0], t[4 * g4 + 1], t[4 * g4 + 2], t[4 * g4 + 3]};
+          } else {
+            union { u32x2 raw; T e[4]; } u;
+#pragma unroll
+            for (int e = 0; e < 4; e++) u.e[e] = from_float<T>(t[4 * g4 + e]);
+            *reinterpret_cast<u32x2 *>(dst) = u.raw;
+          }
         }
+      __builtin_amdgcn_wave_barrier();   // the LDS operations of one wavefront complete in order
+      constexpr int CHUNKS = MS * CW / VE;
+#pragma unroll
+      for (int it = 0; it < (CHUNKS + 63) / 64; it++) {
+        const int idx = it * 64 + lane;
+        if (CHUNKS % 64 == 0 || idx < CHUNKS) {
+          const int row = idx / (CW / VE), ch = idx % (CW / VE);
+          store(r_wave + rt * MS + row, c_wave + c0 * MS + ch * VE, *reinterpret_cast<const u32x4 *>(stage + row * LDS_ROW + ch * VE));
+        }
+      }
+      __builtin_amdgcn_wave_barrier();
+    }
   }
 };
-
-template <typename T> __device__ __forceinline__ void store4(T *p, f32x4 v) {
-  if constexpr (sizeof(T) == 4) {
-    *reinterpret_cast<f32x4 *>(p) = v;
-  } else {
-    union { u32x2 raw; T e[4]; } u;
-#pragma unroll
-    for (int e = 0; e < 4; e++) u.e[e] = from_float<T>(v[e]);
-    *reinterpret_cast<u32x2 *>(p) = u.raw;
-  }
-}
 
 // ---------------------------------------------------------------------------------------------------------
 // sdd: C[z, blockid] = op(A)[z,h, i-th block-row, :K] . op(B)[z,h, :K, j-th block-col]
@@ -343,11 +369,11 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
   }
   T *cz = reinterpret_cast<T *>(g.c) + z * g.c_sz;
   const uint8_t *valid = g.valid ? g.valid + grp * (PACK * PACK) : nullptr;
-  auto store = [&](int m, int n, f32x4 v) {
+  auto store = [&](int m, int n, u32x4 v) {
     const int ent = (m / BLOCK) * PACK + n / BLOCK;
     if (valid && !valid[ent]) return;
     const int64_t bk = e[ent * 4 + 3];
-    store4<T>(cz + bk * (BLOCK * BLOCK) + (m % BLOCK) * BLOCK + n % BLOCK, v);
+    *reinterpret_cast<u32x4 *>(cz + bk * (BLOCK * BLOCK) + (m % BLOCK) * BLOCK + n % BLOCK) = v;
   };
   G::run(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
 }
@@ -374,7 +400,7 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK / SPLIT>::WG * SddShape<BL
   av.idx[0] = e[1]; av.off = (sub / SPLIT) * TT;
   bv.idx[0] = e[2]; bv.off = (sub % SPLIT) * TT;
   T *cb = reinterpret_cast<T *>(g.c) + z * g.c_sz + (int64_t)e[3] * (BLOCK * BLOCK) + av.off * BLOCK + bv.off;
-  auto store = [&](int m, int n, f32x4 v) { store4<T>(cb + m * BLOCK + n, v); };
+  auto store = [&](int m, int n, u32x4 v) { *reinterpret_cast<u32x4 *>(cb + m * BLOCK + n) = v; };
   G::run(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
 }
 
@@ -484,17 +510,18 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k
   T *oz = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh;
   const int NF = g.NF, n0 = nt * S::TN;
   const int64_t ldo = g.ldo;
-  auto store = [&](int m, int n, f32x4 v) {
-    if (n0 + n >= NF) return;
-    if constexpr (OUT_NCONTIG) store4<T>(oz + ((int64_t)column * BLOCK + m) * ldo + n0 + n, v);
-    else store4<T>(oz + (int64_t)(n0 + n) * ldo + column * BLOCK + m, v);
+  // r, c = (m, n) when the output has n contiguous, (n, m) otherwise; c is the first of a 16-byte chunk
+  auto store = [&](int r, int c, u32x4 v) {
+    if constexpr (OUT_NCONTIG) {
+      if (n0 + c < NF) *reinterpret_cast<u32x4 *>(oz + ((int64_t)column * BLOCK + r) * ldo + n0 + c) = v;
+    } else {
+      if (n0 + r < NF) *reinterpret_cast<u32x4 *>(oz + (int64_t)(n0 + r) * ldo + column * BLOCK + c) = v;
+    }
   };
   if (nblk == 0) {   // nothing to read (the views below assume at least one block): write the zeros and leave
-    const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
-    for (int i = threadIdx.x; i < BLOCK * S::TN / 4; i += 256) {
-      if constexpr (OUT_NCONTIG) store(i / (S::TN / 4), (i % (S::TN / 4)) * 4, zero);
-      else store((i % (BLOCK / 4)) * 4, i / (BLOCK / 4), zero);
-    }
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    constexpr int VE = 16 / (int)sizeof(T), CW = OUT_NCONTIG ? S::TN : BLOCK;   // chunks run along the contiguous index
+    for (int i = threadIdx.x; i < BLOCK * S::TN / VE; i += 256) store(i / (CW / VE), (i % (CW / VE)) * VE, zero);
     return;
   }
   G::run(sv, dv, (nblk * BLOCK + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
