@@ -117,6 +117,18 @@ def test_block128_sdd_one_or_four_workgroups_per_block(Z):
     run_case('sdd', False, True, 128, torch.bfloat16, Z=Z, H=2, M=1024, N=1024, K=48, layout=lay, seed=10, backward=False)
 
 
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+@pytest.mark.parametrize('mode,trans_a,trans_b', [('dsd', False, False), ('dsd', True, True), ('dds', False, True), ('dds', True, False)])
+def test_narrow_free_dimension(block, mode, trans_a, trans_b):
+    # free dimension of at most 64 (the head dimension of an attention product): the kernels use a 64-wide tile
+    # instead of their wide one; 48 leaves part of that tile empty
+    for free, dtype in ((64, torch.float16), (48, torch.float32)):
+        if mode == 'dsd':
+            run_case(mode, trans_a, trans_b, block, dtype, Z=2, H=2, M=256, N=free, K=384, seed=block + free, backward=False)
+        else:
+            run_case(mode, trans_a, trans_b, block, dtype, Z=2, H=2, M=free, N=256, K=384, seed=block + free, backward=False)
+
+
 def test_degenerate_layouts():
     # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
     lay = torch.zeros(2, 4, 6, dtype=torch.int64)

@@ -471,18 +471,22 @@ template <typename T, int BLOCK> struct DenseView {                   // element
   __device__ __forceinline__ int64_t scalar_r(const Step &st, int i) const { return ((int64_t)st.pos[i] + st.kin) * ld; }
 };
 
-template <int BLOCK> struct XsdShape {
+template <int BLOCK, bool WIDE> struct XsdShape {
   // Tile of the dense free dimension.  Wide tiles for block 32 and 128: a wavefront then reuses each fragment of the
   // sparse block for two or four MFMAs (LDS reads per MFMA are what bounds these kernels); measured +13 % at block 32.
-  static constexpr int TN = BLOCK == 64 ? 128 : BLOCK >= 32 ? 256 : 64;
-  static constexpr int WGM = BLOCK >= 64 ? 2 : 1;        // 32 -> 1x4 wavefronts of 32x64; 64 -> 2x2 of 32x64; 128 -> 2x2 of 64x128
+  // The narrow shape serves free dimensions up to 64 (the head dimension of an attention product), where a wide
+  // tile would be mostly padding.
+  static constexpr int TN = !WIDE ? 64 : BLOCK == 64 ? 128 : BLOCK >= 32 ? 256 : 64;
+  // wide: 32 -> 1x4 wavefronts of 32x64; 64 -> 2x2 of 32x64; 128 -> 2x2 of 64x128.  narrow: 16 -> 1x4 of 16x16;
+  // 32 -> 2x2 of 16x32; 64 -> 2x2 of 32x32; 128 -> 2x2 of 64x32
+  static constexpr int WGM = (WIDE ? BLOCK >= 64 : BLOCK >= 32) ? 2 : 1;
   static constexpr int WGN = 4 / WGM;
 };
 
 // (at least two wavefronts per SIMD: the 128 x 256 tile of block 128 would otherwise take 266 registers and run alone)
-template <typename T, int BLOCK, bool SP_TRANS, bool DN_KCONTIG, bool OUT_NCONTIG>
+template <typename T, int BLOCK, bool WIDE, bool SP_TRANS, bool DN_KCONTIG, bool OUT_NCONTIG>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_xsd(XsdArgs g) {
-  typedef XsdShape<BLOCK> S;
+  typedef XsdShape<BLOCK, WIDE> S;
   typedef TileGemm<T, BLOCK, S::TN, S::WGM, S::WGN, !SP_TRANS, DN_KCONTIG, OUT_NCONTIG> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int n_tiles = (g.NF + S::TN - 1) / S::TN;
@@ -576,14 +580,14 @@ template <typename T> int launch_sdd(const SddArgs &g, int block, int pack, bool
   return BSP_ERR_UNSUPPORTED;
 }
 
-template <typename T, int BLOCK> int launch_xsd_b(const XsdArgs &g, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
-  typedef XsdShape<BLOCK> S;
+template <typename T, int BLOCK, bool WIDE> int launch_xsd_bw(const XsdArgs &g, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+  typedef XsdShape<BLOCK, WIDE> S;
   const int64_t n_wg = (int64_t)g.width * ((g.NF + S::TN - 1) / S::TN) * g.Z;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   dim3 grid((unsigned)n_wg), blockdim(256);
 #define BSP_XSD_LAUNCH(ST, DK, ON)                                                                               \
-  hipLaunchKernelGGL((k_xsd<T, BLOCK, ST, DK, ON>), grid, blockdim,                                             \
+  hipLaunchKernelGGL((k_xsd<T, BLOCK, WIDE, ST, DK, ON>), grid, blockdim,                                       \
                      (TileGemm<T, BLOCK, S::TN, S::WGM, S::WGN, !ST, DK, ON>::SMEM_BYTES), st, g)
   const int key = (sp_trans ? 4 : 0) | (dn_kc ? 2 : 0) | (out_nc ? 1 : 0);
   switch (key) {
@@ -598,6 +602,11 @@ template <typename T, int BLOCK> int launch_xsd_b(const XsdArgs &g, bool sp_tran
   }
 #undef BSP_XSD_LAUNCH
   return BSP_OK;
+}
+
+template <typename T, int BLOCK> int launch_xsd_b(const XsdArgs &g, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+  if (g.NF > 64 && XsdShape<BLOCK, true>::TN > 64) return launch_xsd_bw<T, BLOCK, true>(g, sp_trans, dn_kc, out_nc, st);
+  return launch_xsd_bw<T, BLOCK, false>(g, sp_trans, dn_kc, out_nc, st);
 }
 
 template <typename T> int launch_xsd(const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
