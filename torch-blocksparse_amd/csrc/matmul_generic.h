@@ -191,7 +191,9 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
   static constexpr int SMEM_BYTES = 2 * (X_ELEMS + Y_ELEMS) * (int)sizeof(T);
 
   // ksteps = number of TK-wide reduction steps.  Store(m, n, vals): vals[4] run along n (OUT_NCONTIG) or m.
-  template <class XView, class YView, class Store>
+  // SUB > 0: the output consists of SUB x SUB blocks that are each contiguous in memory (the sparse result of sdd);
+  // the epilogue then writes block by block.  SUB == 0: the output is a matrix with long rows.
+  template <int SUB = 0, class XView, class YView, class Store>
   static __device__ __forceinline__ void run(const XView &xv, const YView &yv, int ksteps, T *smem, const Store &store) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave / WGN, wn = wave % WGN;
@@ -270,6 +272,41 @@ template <typename T, int TM, int TN, int WGM, int WGN, bool X_KCONTIG, bool Y_K
     // time through its own piece of LDS (free after the last barrier) and writes whole 16-byte chunks, consecutive
     // lanes along a row.  store(r, c, chunk): r = row (m if OUT_NCONTIG, else n), c = first of VE consecutive columns.
     constexpr int VE = 16 / (int)sizeof(T);
+    if constexpr (SUB > 0 && OUT_NCONTIG && TM * (TN + VE) * (int)sizeof(T) <= SMEM_BYTES) {
+      // Blocked output: the whole TM x TN tile is staged (all wavefronts, two barriers) and then written block by
+      // block, consecutive lanes on consecutive 16-byte chunks of one block: 512 contiguous bytes per 32 lanes at
+      // block 16, where row-wise stores would write 32-byte pieces.
+      constexpr int LDS_ROW = TN + VE, CPB = SUB * SUB / VE, BPR = TN / SUB, CHUNKS = TM * TN / VE;
+      const int cc = lane % MS;
+#pragma unroll
+      for (int i = 0; i < RM; i++)
+#pragma unroll
+        for (int j = 0; j < RN; j++)
+#pragma unroll
+          for (int g4 = 0; g4 < M::NACC / 4; g4++) {
+            const int rr = (MS == 16) ? 4 * (lane >> 4) : 8 * g4 + 4 * (lane >> 5);
+            T *dst = smem + ((wm * RM + i) * MS + cc) * LDS_ROW + (wn * RN + j) * MS + rr;
+            if constexpr (sizeof(T) == 4) {
+              *reinterpret_cast<f32x4 *>(dst) = f32x4{acc[i][j][4 * g4 + 0], acc[i][j][4 * g4 + 1], acc[i][j][4 * g4 + 2], acc[i][j][4 * g4 + 3]};
+            } else {
+              union { u32x2 raw; T e[4]; } u;
+#pragma unroll
+              for (int e = 0; e < 4; e++) u.e[e] = from_float<T>(acc[i][j][4 * g4 + e]);
+              *reinterpret_cast<u32x2 *>(dst) = u.raw;
+            }
+          }
+      __syncthreads();
+#pragma unroll
+      for (int it = 0; it < (CHUNKS + NT - 1) / NT; it++) {
+        const int idx = it * NT + tid;
+        if (CHUNKS % NT == 0 || idx < CHUNKS) {
+          const int blk = idx / CPB, within = idx % CPB;
+          const int m = (blk / BPR) * SUB + within / (SUB / VE), n = (blk % BPR) * SUB + (within % (SUB / VE)) * VE;
+          store(m, n, *reinterpret_cast<const u32x4 *>(smem + m * LDS_ROW + n));
+        }
+      }
+      return;
+    }
     constexpr int NR = OUT_NCONTIG ? RM : RN, NC = OUT_NCONTIG ? RN : RM;   // tiles along the row / contiguous index
     // tiles staged per pass: all NC of them if that fits the tile buffers, else half, a quarter ...
     constexpr int CG = stage_tiles(NC, MS, VE, (int)sizeof(T) * WGM * WGN, SMEM_BYTES);
@@ -375,7 +412,7 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
     const int64_t bk = e[ent * 4 + 3];
     *reinterpret_cast<u32x4 *>(cz + bk * (BLOCK * BLOCK) + (m % BLOCK) * BLOCK + n % BLOCK) = v;
   };
-  G::run(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
+  G::template run<BLOCK>(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
 }
 
 // sdd with SPLIT x SPLIT workgroups per block (pack 1): for layouts with so few blocks that one workgroup per block
