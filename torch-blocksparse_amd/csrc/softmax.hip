@@ -176,21 +176,16 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
     }
     const float sc = a.scale * unit;
-    if (a.kpm) {                                        // softmax.py:112-116, 122-124
+    const bool has_kpm = a.kpm != nullptr;
 #pragma unroll
-      for (int b = 0; b < NB; b++)
-        if (b < size) {
+    for (int b = 0; b < NB; b++)
+      if (b < size) {                                   // softmax.py:112-116, 122-124
 #pragma unroll
-          for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(px[b].e[e]), sc, kpm_s[b * BLOCK + u.col + e]);
-        }
-    } else {
-#pragma unroll
-      for (int b = 0; b < NB; b++)
-        if (b < size) {
-#pragma unroll
-          for (int e = 0; e < GE::EV; e++) fx[b][e] = to_float(px[b].e[e]) * sc;
-        }
-    }
+        for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(px[b].e[e]), sc, has_kpm ? kpm_s[b * BLOCK + u.col + e] : 0.f);
+        // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
+        // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
+        if constexpr (NB >= 16) __builtin_amdgcn_sched_barrier(0);
+      }
     if constexpr (EXTRA) {
       if (a.rpe) {                                      // :118-120
 #pragma unroll
@@ -417,7 +412,8 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
 
 // Register budget: a lane keeps NB * EV fp32 values (forward) or 2 * NB raw chunks (backward).
 template <typename T, int BLOCK> constexpr int max_nb_fwd() { return 128 / Geo<T, BLOCK>::EV > 32 ? 32 : 128 / Geo<T, BLOCK>::EV; }
-template <typename T, int BLOCK> constexpr int max_nb_bwd() { return 16; }
+// backward: 2 raw chunks per block; 8-byte chunks (block 16, 16-bit types) leave room for 32 blocks
+template <typename T, int BLOCK> constexpr int max_nb_bwd() { return Geo<T, BLOCK>::EV * (int)sizeof(T) <= 8 ? 32 : 16; }
 
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
   const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
@@ -449,6 +445,7 @@ template <typename T, int BLOCK> void launch_bwd(const BwdArgs &a, int maxlut, h
   else if (maxlut <= 7) launch_bwd_nb<T, BLOCK, 7>(a, st);
   else if (maxlut <= 8) launch_bwd_nb<T, BLOCK, 8>(a, st);
   else if (maxlut <= 16) launch_bwd_nb<T, BLOCK, 16>(a, st);
+  else if (maxlut <= 32 && max_nb_bwd<T, BLOCK>() >= 32) launch_bwd_nb<T, BLOCK, (max_nb_bwd<T, BLOCK>() >= 32 ? 32 : 0)>(a, st);
   else launch_bwd_nb<T, BLOCK, 0>(a, st);
 }
 
