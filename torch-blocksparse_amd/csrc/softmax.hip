@@ -245,13 +245,18 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
     const T *rz = reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + u.col;
     const T *az = reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + u.col;
     P px[CH], pk[CH], pr[NX], pa[NX];
-    int32_t bid[CH];
+    int32_t bid[CH], bcol[CH];
     auto load_chunk = [&](int b0) {
+#pragma unroll
+      for (int j = 0; j < CH; j++) {                    // table reads first, unconditional: one wait for all of them
+        const int bb = b0 + j < size ? b0 + j : b0;
+        bid[j] = core[4 * bb + 0];
+        bcol[j] = core[4 * bb + 1];
+      }
 #pragma unroll
       for (int j = 0; j < CH; j++)
         if (b0 + j < size) {
-          bid[j] = core[4 * (b0 + j) + 0];
-          const int64_t c0 = (int64_t)core[4 * (b0 + j) + 1] * BLOCK;   // first column of the block in the dense matrix
+          const int64_t c0 = (int64_t)bcol[j] * BLOCK;  // first column of the block in the dense matrix
           px[j].load(xb + (int64_t)bid[j] * (BLOCK * BLOCK));
           if (a.kpm) pk[j].load(kz + c0);
           if constexpr (EXTRA) {
@@ -346,10 +351,12 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
     P py[NB], pd[NB];
     int32_t bid[NB];
     float dot = 0.f;
+    // the table reads come first and unconditionally (one wait for all of them, not one round trip per block)
+#pragma unroll
+    for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
-        bid[b] = core[4 * b];
         const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
         py[b].load(yb + o);
         pd[b].load(db + o);
@@ -377,9 +384,10 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
     int64_t off[CH];
     auto load_chunk = [&](int b0) {
 #pragma unroll
+      for (int j = 0; j < CH; j++) off[j] = (int64_t)core[4 * (b0 + j < size ? b0 + j : b0)] * (BLOCK * BLOCK);
+#pragma unroll
       for (int j = 0; j < CH; j++)
         if (b0 + j < size) {
-          off[j] = (int64_t)core[4 * (b0 + j)] * (BLOCK * BLOCK);
           py[j].load(yb + off[j]);
           pd[j].load(db + off[j]);
         }
