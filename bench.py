@@ -273,19 +273,31 @@ def other_config(args):
         causal = torch.tril(torch.ones(L, L, dtype=torch.float16, device=dev))
         fl = 2.0 * B * dh * nnz * block * block
         xb = B * nnz * block * block * 2
+        do = torch.randn_like(q)
+        from torch_blocksparse.matmul import _sparse_matmul
+        fn, spd, t = _sparse_matmul.fn, lay.shape, [None]
+        sl, dl = sdd.make_lut(torch.float16, dev), dsd.make_lut(torch.float16, dev)   # (c, da, db) tables of each op
+        sm_lut, sm_maxlut = sm.make_lut(dev)
         with torch.no_grad():
             w = sdd(q, k)
+            dw = torch.randn_like(w)
             for name, f, flops, nbytes in (
                     ('sdd q.k^T', lambda: sdd(q, k), fl, xb + 2 * B * H * L * dh * 2),
                     ('softmax fwd, scale only', lambda: sm(w, scale=0.125), 0, 2 * xb),
                     ('softmax fwd, rpe + causal mask', lambda: sm(w, scale=0.125, rpe=rpe, attn_mask=causal, attn_mask_mode='mul'), 0, 2 * xb),   # x only: both masks are shared by batch and heads
-                    ('dsd p.v', lambda: dsd(w, v), fl, xb + 2 * B * H * L * dh * 2)):
+                    ('dsd p.v', lambda: dsd(w, v), fl, xb + 2 * B * H * L * dh * 2),
+                    # backward, in the order autograd runs it (the products of MatMul.backward are MatMul modes of their own)
+                    ('dsd p^T.do', lambda: fn['dsd'](w, do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t), fl, xb + 2 * B * H * L * dh * 2),
+                    ('sdd do.v^T', lambda: fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t), fl, xb + 2 * B * H * L * dh * 2),
+                    ('softmax bwd', lambda: _bwd_softmax(tb, w, dw, 0.125, sm_lut, sm_maxlut, spd, block), 0, 3 * xb),
+                    ('dds (q^T.ds)^T', lambda: fn['dds'](q, dw, True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t), fl, xb + 2 * B * H * L * dh * 2),
+                    ('dsd ds.k', lambda: fn['dsd'](dw, k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t), fl, xb + 2 * B * H * L * dh * 2)):
                 ms = timeit(f)
                 ent = {'launch': name, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)}
                 if flops:
                     ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
                 out.append(ent)
-        workload = 'BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, forward chain'
+        workload = 'BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, forward and backward launches'
     print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
                       'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic', 'config': {'workload': workload, 'config': args.config},
                       'launches': out}))

@@ -73,7 +73,10 @@ struct FwdArgs {
 template <typename T, int BLOCK> struct Unit {
   int z, hr, rxm, col;   // batch, head*R + block-row, row inside the block, lane's first column inside a block
   bool ok;
-  __device__ __forceinline__ Unit(int64_t n_units, int HR) {
+  // shared_masks: the launch reads a relative position embedding or an attention mask.  Their rows are the same for
+  // every head (and batch), so the units are then ordered block-row first, heads and batches inside: the wavefronts
+  // that need the same mask rows run at the same time on the same XCD and all but the first find them in its L2.
+  __device__ __forceinline__ Unit(int64_t n_units, int HR, bool shared_masks = false, int H = 1, int Z = 1) {
     typedef Geo<T, BLOCK> GE;
     const int64_t n_wg = (n_units + kWavesPerGroup - 1) / kWavesPerGroup;
     const int64_t wg = xcd_remap(blockIdx.x, n_wg);
@@ -86,8 +89,15 @@ template <typename T, int BLOCK> struct Unit {
     // Block-rows are taken from the last one down.  The matmul kernels on either side of this one walk a causal
     // layout from its longest rows (the last ones) to its shortest, so this order reads first what the producer wrote
     // last; measured in the attention chain it makes this kernel and its consumer 3-5 % faster than the ascending order.
-    hr = HR - 1 - (int)(t % HR);
-    z = (int)(t / HR);
+    if (shared_masks) {
+      const int R = HR / H;
+      z = (int)(t % Z);
+      const int64_t t2 = t / Z;
+      hr = (int)(t2 % H) * R + (R - 1 - (int)((t2 / H) % R));
+    } else {
+      hr = HR - 1 - (int)(t % HR);
+      z = (int)(t / HR);
+    }
     rxm = g * GE::RPW + lane / GE::LPR;
     col = (lane % GE::LPR) * GE::EV;
   }
@@ -110,7 +120,7 @@ template <typename T, int BLOCK, int NB, bool EXTRA>
 __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   typedef Geo<T, BLOCK> GE;
   const int HR = a.H * a.R;
-  Unit<T, BLOCK> u(a.n_units, HR);
+  Unit<T, BLOCK> u(a.n_units, HR, EXTRA, a.H, a.Z);
   if (!u.ok) return;
   const table_ptr lut = as_table(a.lut);
   const int size = lut[2 * u.hr + 0];                   // header (size, offset), softmax.py:30-32
