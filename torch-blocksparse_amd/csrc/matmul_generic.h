@@ -552,11 +552,12 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k
   const int NF = g.NF, n0 = nt * S::TN;
   const int64_t ldo = g.ldo;
   // r, c = (m, n) when the output has n contiguous, (n, m) otherwise; c is the first of a 16-byte chunk
+  // streaming stores: the dense result is not read again by the sparse chain and should not displace what is
   auto store = [&](int r, int c, u32x4 v) {
     if constexpr (OUT_NCONTIG) {
-      if (n0 + c < NF) *reinterpret_cast<u32x4 *>(oz + ((int64_t)column * BLOCK + r) * ldo + n0 + c) = v;
+      if (n0 + c < NF) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(oz + ((int64_t)column * BLOCK + r) * ldo + n0 + c));
     } else {
-      if (n0 + r < NF) *reinterpret_cast<u32x4 *>(oz + (int64_t)(n0 + r) * ldo + column * BLOCK + c) = v;
+      if (n0 + r < NF) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(oz + (int64_t)(n0 + r) * ldo + column * BLOCK + c));
     }
   };
   if (nblk == 0) {   // nothing to read (the views below assume at least one block): write the zeros and leave

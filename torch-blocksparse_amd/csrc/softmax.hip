@@ -28,6 +28,8 @@ template <typename T, int EV> struct Pack {
   union { raw_t raw; T e[EV]; };
   __device__ __forceinline__ void load(const T *p) { raw = *reinterpret_cast<const raw_t *>(p); }
   __device__ __forceinline__ void store(T *p) const { *reinterpret_cast<raw_t *>(p) = raw; }
+  // for data nobody reads again soon: leaves the caches to what the next kernels need
+  __device__ __forceinline__ void load_stream(const T *p) { raw = __builtin_nontemporal_load(reinterpret_cast<const raw_t *>(p)); }
 };
 
 // Geometry: LPR lanes share a row and each owns one chunk of EV consecutive columns of every block (16 bytes,
@@ -368,7 +370,7 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
     for (int b = 0; b < NB; b++)
       if (b < size) {
         const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
-        py[b].load(yb + o);
+        py[b].load_stream(yb + o);   // y is not read again after the backward pass
         pd[b].load(db + o);
       }
 #pragma unroll
@@ -398,7 +400,7 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
 #pragma unroll
       for (int j = 0; j < CH; j++)
         if (b0 + j < size) {
-          py[j].load(yb + off[j]);
+          py[j].load_stream(yb + off[j]);
           pd[j].load(db + off[j]);
         }
     };
