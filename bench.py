@@ -44,6 +44,8 @@ def main():
     ap.add_argument('--warmup', type=int, default=5)
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--batch', type=int, default=8)
+    ap.add_argument('--block', type=int, default=64, choices=[16, 32, 64],
+                    help='config 3 only: express the same attention mask in smaller blocks (64 = the headline workload)')
     ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
                     help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
     args = ap.parse_args()
@@ -58,10 +60,12 @@ def main():
     from torch_blocksparse.matmul import _sparse_matmul
     dev = torch.device('cuda:0')
     torch.manual_seed(0)
-    B, H, L, dh, block = args.batch, 16, 4096, 64, 64
+    B, H, L, dh, block = args.batch, 16, 4096, 64, args.block
     dtype = torch.float16
     scale = 0.125
-    lay = tb.sparse_transformer_layout(H, L // block, 4, 16, True)
+    lay = tb.sparse_transformer_layout(H, L // 64, 4, 16, True)
+    if block != 64:   # the same mask, every 64-block split into (64 / block)^2 blocks: same flops, same bytes
+        lay = lay.repeat_interleave(64 // block, 1).repeat_interleave(64 // block, 2)
     nnz = int(lay.sum())
     q, k, v, do = [torch.randn(B, H, L, dh, dtype=dtype, device=dev) for _ in range(4)]
     q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
@@ -162,7 +166,7 @@ def main():
     for name, _, flops, nbytes in launches:
         ms = sum(a.elapsed_time(b) for a, b in events[name]) / len(events[name])
         ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
-               'bytes': nbytes, 'traffic': TRAFFIC_BYTES.get(name) if B == 8 else None}
+               'bytes': nbytes, 'traffic': TRAFFIC_BYTES.get(name) if (B == 8 and block == 64) else None}
         if flops:
             ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
             ent['mfma_frac'] = round(flops / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)
@@ -173,12 +177,12 @@ def main():
                 'frac': kernels[dom]['hbm_frac'], 'traffic': kernels[dom]['traffic']}
 
     out = {
-        'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk64',
+        'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk%d' % block,
         'value': round(6 * flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f16', 'data': 'synthetic',
-        'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block 64, fixed '
-                               'layout (local 4 blocks + 1 global per 16, causal), scale 1/8, additive key-padding mask' % B,
+        'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block %d, fixed '
+                               'layout (local 4 blocks + 1 global per 16 at block 64, causal), scale 1/8, additive key-padding mask' % (B, block),
                    'nnz_blocks': nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
         'matmul_TFLOP/s_kernel_time_only': round(6 * flops_mm / sum(e['ms'] for n, e in kernels.items() if 'softmax' not in n) * 1e-9, 2),
         'softmax_GB/s': {'fwd': kernels['softmax_fwd']['GB/s'], 'bwd': kernels['softmax_bwd']['GB/s']},

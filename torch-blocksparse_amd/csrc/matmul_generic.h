@@ -365,7 +365,10 @@ struct SddArgs {
 };
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
-  const T *base; int64_t ld; int K; int idx[PACK];   // base doubles as the dummy address of out-of-range chunks
+  // idx is a vector, not an array: an array member makes the compiler keep the view in scratch memory and turn the
+  // selection in blk() into an indexed scratch load, a full memory round trip before a workgroup's first load
+  typedef int idx_t __attribute__((ext_vector_type(PACK == 1 ? 2 : PACK)));
+  const T *base; int64_t ld; int K; idx_t idx;   // base doubles as the dummy address of out-of-range chunks
   int off = 0;                                        // first row of the tile inside its block (tiles smaller than a block)
   static constexpr int NB = 1;
   struct Step { int k0; bool live[1]; int klim; };
@@ -406,10 +409,14 @@ __global__ void __launch_bounds__(64 * SddShape<BLOCK * PACK>::WG * SddShape<BLO
   }
   T *cz = reinterpret_cast<T *>(g.c) + z * g.c_sz;
   const uint8_t *valid = g.valid ? g.valid + grp * (PACK * PACK) : nullptr;
+  // The entry differs from lane to lane here, so the output block is looked up through an ordinary pointer (a vector
+  // load): through the constant address space the compiler fetches all PACK * PACK entries with scalar loads and
+  // indexes them per lane in scratch memory.
+  const int32_t *eg = g.lut + grp * (PACK * PACK * 4);
   auto store = [&](int m, int n, u32x4 v) {
     const int ent = (m / BLOCK) * PACK + n / BLOCK;
     if (valid && !valid[ent]) return;
-    const int64_t bk = e[ent * 4 + 3];
+    const int64_t bk = eg[ent * 4 + 3];
     *reinterpret_cast<u32x4 *>(cz + bk * (BLOCK * BLOCK) + (m % BLOCK) * BLOCK + n % BLOCK) = v;
   };
   G::template run<BLOCK>(av, bv, (g.K + G::TK - 1) / G::TK, reinterpret_cast<T *>(smem_raw), store);
