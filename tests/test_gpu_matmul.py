@@ -129,6 +129,24 @@ def test_narrow_free_dimension(block, mode, trans_a, trans_b):
             run_case(mode, trans_a, trans_b, block, dtype, Z=2, H=2, M=free, N=256, K=384, seed=block + free, backward=False)
 
 
+@pytest.mark.parametrize('block', [16, 32])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_small_block_row_groups(block, dtype):
+    # blocks of 16 and 32 with a free dimension of 64 or 128 (attention shapes) run on row-group kernels with one
+    # wavefront per member.  22 lines: the last group has two members; one empty block-row, one full block-column,
+    # one full block-row; forward and backward reach the plain and the transposed variant of dsd and of dds.
+    n = 22
+    lay = random_layout((3, n, n), 0.3, 77 + block)
+    lay[:, 5, :] = 0
+    lay[:, :, 7] = 1
+    lay[1, 9, :] = 1
+    lay[:, 5, :] = 0
+    for free in (64, 128):
+        run_case('dsd', False, False, block, dtype, Z=2, H=3, M=n * block, K=n * block, N=free, layout=lay, seed=block + free, dist='randn', scale=0.25)
+        run_case('dsd', True, False, block, dtype, Z=2, H=3, M=n * block, K=n * block, N=free, layout=lay, seed=block + free + 1, dist='randn', scale=0.25)
+        run_case('sdd', False, True, block, dtype, Z=2, H=3, M=n * block, N=n * block, K=free, layout=lay, seed=block + free + 2, dist='randn', scale=0.25)
+
+
 def test_degenerate_layouts():
     # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
     lay = torch.zeros(2, 4, 6, dtype=torch.int64)

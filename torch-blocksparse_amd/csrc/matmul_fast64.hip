@@ -15,6 +15,7 @@
 //                Four wavefronts per workgroup, each owning 16 output rows; global loads run four blocks
 //                ahead of the MFMAs in a register ring.
 #include "matmul_generic.h"
+#include <type_traits>
 
 namespace bsp {
 namespace {
@@ -587,11 +588,169 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// Row groups for blocks of 16 and 32 (16-bit types, 64-wide tile of the dense free dimension).  Same plan as the
+// block-64 kernel above, other division of labour: a line is only 16 or 32 rows, so each of the four wavefronts
+// takes one MEMBER of the group (all rows of its line), and an entry is one block of the reduction: its dense rows
+// (BLOCK x 64) go through LDS once for all four members, each wavefront fetches its own sparse block straight into
+// operand registers (through its own piece of LDS and the transposing read when the block is read transposed).
+// Against one workgroup per line this moves 2.5x fewer bytes between L2, LDS and the registers per line and
+// needs half the barriers.  Block 16 multiplies with the 16x16x16 MFMA (one block = one reduction step).
+// ---------------------------------------------------------------------------------------------------------
+template <typename T, int K> struct LineMma;
+template <typename T> struct LineMma<T, 32> : Mma16<T> {};
+template <> struct LineMma<f16, 16> {
+  typedef f16x4 frag_t;
+  static __device__ __forceinline__ f32x4 run(frag_t a, frag_t b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x16f16(a, b, c, 0, 0, 0); }
+};
+template <> struct LineMma<bf16, 16> {
+  typedef s16x4 frag_t;
+  static __device__ __forceinline__ f32x4 run(frag_t a, frag_t b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0); }
+};
+// operand of the line kernels from an LDS tile stored [k][column]: K consecutive reduction indices of this lane's column
+template <typename T, int K> __device__ __forceinline__ typename LineMma<T, K>::frag_t line_tr_frag(const T *tile, int ld, int col0, int lane) {
+  const int q = lane >> 4, t = lane & 15;
+  if constexpr (K == 32) {
+    const T *p = tile + (8 * q + (t >> 2)) * ld + col0 + 4 * (t & 3);
+    return tr_frag<T>(p, p + 4 * ld);
+  } else {
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+    const T *p = tile + (4 * q + (t >> 2)) * ld + col0 + 4 * (t & 3);
+    return __builtin_bit_cast(typename LineMma<T, K>::frag_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)p));
+  }
+}
+
+constexpr int kSmallRing = 4;
+
+template <typename T, int BLOCK, bool SP_TRANS>
+__global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
+  typedef LineMma<T, BLOCK> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int MT = BLOCK / 16;                 // 16-row tiles of a line
+  constexpr int XB = BLOCK * BLOCK * 2 / 64;     // bytes of a sparse block per lane: 8 (block 16) or 32
+  constexpr int NX = XB / 16 > 0 ? XB / 16 : 1;  // loads per lane: one of 8 bytes, or two of 16
+  typedef typename std::conditional<XB == 8, u32x2, u32x4>::type xreg_t;
+  constexpr int LDX = BLOCK + 8;
+  constexpr int YT = BLOCK * kLdsRow, XT = SP_TRANS ? BLOCK * LDX : 0;
+  __shared__ __attribute__((aligned(16))) T Ys[2][YT];
+  __shared__ __attribute__((aligned(16))) T Xs[4][XT > 0 ? XT : 8];
+  __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int z = blockIdx.x % g.Z;
+  const int64_t rest = blockIdx.x / g.Z;
+  const int n0 = (int)(rest % g.n_tiles) * 64;
+  const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
+  const int e0 = hd[0], ne = hd[1], depth = hd[2], code = hd[3];
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  // a chain (a long line on its own) is a group whose only member is member 0
+  const int line = code < 0 ? -(code + 1) + wave : (code & 0xffffff) * G + wave;
+  const bool mine = code < 0 ? wave == 0 : (line < g.lines && !(((code >> 24) >> wave) & 1));
+  const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
+  const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
+  const int64_t ldd = g.ldd;
+  const int yc = tid % (BLOCK * 8), yrow = yc >> 3, ycol = (yc & 7) * 8;   // this thread's 16-byte chunk of the dense rows
+  const bool ywrite = tid < BLOCK * 8;
+  const int q = lane >> 4, t = lane & 15;
+  struct Stage { u32x4 y; xreg_t x[NX]; };
+  Stage ring[kSmallRing];
+  // A fixed number of loads per stage whatever the entry holds (the wait in front of a stage is then exact): an
+  // absent block reads one line at the start of the sparse tensor.
+  auto issue = [&](Stage &st, int e) {
+    const table_ptr en = ent + (G + 1) * e;
+    st.y = *reinterpret_cast<const u32x4 *>(dn + ((int64_t)en[0] * BLOCK + yrow) * ldd + ycol);
+    const int bid = en[1 + wave];
+    const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * (BLOCK * BLOCK);
+#pragma unroll
+    for (int i = 0; i < NX; i++) {
+      const T *px;
+      if constexpr (SP_TRANS) px = blk + (XB == 8 ? lane * 4 : (64 * i + lane) * 8);        // as stored: consecutive lanes, consecutive chunks
+      else px = XB == 8 ? blk + t * BLOCK + 4 * q : blk + (16 * i + t) * BLOCK + 8 * q;   // operand layout
+      if (bid < 0) px = sp;
+      st.x[i] = *reinterpret_cast<const xreg_t *>(px);
+    }
+  };
+  f32x4 acc[MT][4];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (ne > 0) {
+    const int last = ne - 1;
+#pragma unroll
+    for (int u = 0; u < kSmallRing; u++) issue(ring[u], u < last ? u : last);
+    const int steps = (ne + kSmallRing - 1) / kSmallRing * kSmallRing;
+    for (int e0i = 0; e0i < steps; e0i += kSmallRing) {
+#pragma unroll
+      for (int u = 0; u < kSmallRing; u++) {
+        const int e = e0i + u;
+        const bool live = e < ne;
+        const int buf = e & 1;
+        Stage &st = ring[u];
+        const int bid0 = ent[(G + 1) * min(e, last) + 1 + wave];
+        const int bid = live ? bid0 : -1;
+        if (ywrite) *reinterpret_cast<u32x4 *>(&Ys[buf][yrow * kLdsRow + ycol]) = st.y;
+        frag_t xf[MT];
+        if constexpr (SP_TRANS) {
+#pragma unroll
+          for (int i = 0; i < NX; i++) {
+            const int c = 64 * i + lane;                       // chunk of xreg_t: row c / (chunks per row)
+            constexpr int CPR = BLOCK * 2 / (int)sizeof(xreg_t), CE = (int)sizeof(xreg_t) / 2;
+            *reinterpret_cast<xreg_t *>(&Xs[wave][(c / CPR) * LDX + (c % CPR) * CE]) = st.x[i];
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < MT; i++) xf[i] = __builtin_bit_cast(frag_t, st.x[i]);
+        }
+        __syncthreads();
+        if (bid >= 0) {
+          frag_t yf[4];
+#pragma unroll
+          for (int j = 0; j < 4; j++) yf[j] = line_tr_frag<T, BLOCK>(Ys[buf], kLdsRow, 16 * j, lane);
+          if constexpr (SP_TRANS) {
+#pragma unroll
+            for (int i = 0; i < MT; i++) xf[i] = line_tr_frag<T, BLOCK>(Xs[wave], LDX, 16 * i, lane);
+          }
+#pragma unroll
+          for (int i = 0; i < MT; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // rows n = 16j + 4*(lane/16) + e, column m = lane % 16
+        }
+        issue(st, e + kSmallRing < last ? e + kSmallRing : last);
+      }
+    }
+  }
+  if (mine) {
+    T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+      store_slice<T, true>(Cs[wave], po + ((int64_t)line * BLOCK + 16 * i) * g.ldo, g.ldo, acc[i], lane);
+  }
+}
+
 bool fast_ok_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc) {
   return block == 64 && pack == 1 && a_kc && b_kc && g.K % 64 == 0;
 }
 bool fast_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
   return block == 64 && !dn_kc && out_nc && g.NF % 64 == 0;
+}
+
+// The member-per-wavefront kernel pays while the free dimension is short; with many 64-wide tiles the general kernel's
+// 256-wide tile reuses each sparse block four times.
+bool small_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
+  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && !dn_kc && out_nc && g.NF % 64 == 0 && g.NF <= 128;
+}
+template <typename T> int xsd_small_t(const XsdArgs &g, int block, bool sp_trans, hipStream_t st) {
+  const int64_t n = (int64_t)g.n_pgroups * g.n_tiles * g.Z;
+  if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)n), wg(256);
+  if (block == 16) {
+    if (sp_trans) hipLaunchKernelGGL((k_xsd_rg_small<T, 16, true>), grid, wg, 0, st, g);
+    else hipLaunchKernelGGL((k_xsd_rg_small<T, 16, false>), grid, wg, 0, st, g);
+  } else {
+    if (sp_trans) hipLaunchKernelGGL((k_xsd_rg_small<T, 32, true>), grid, wg, 0, st, g);
+    else hipLaunchKernelGGL((k_xsd_rg_small<T, 32, false>), grid, wg, 0, st, g);
+  }
+  return BSP_OK;
 }
 
 template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
@@ -632,6 +791,10 @@ int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool
   return rc == BSP_OK ? 1 : rc;
 }
 int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+  if (dtype != BSP_F32 && small_ok_xsd(g, block, dn_kc, out_nc)) {
+    int rc = dtype == BSP_F16 ? xsd_small_t<f16>(g, block, sp_trans, st) : xsd_small_t<bf16>(g, block, sp_trans, st);
+    return rc == BSP_OK ? 1 : rc;
+  }
   if (dtype == BSP_F32 || !fast_ok_xsd(g, block, dn_kc, out_nc)) return 0;
   int rc = dtype == BSP_F16 ? xsd_fast_t<f16>(g, sp_trans, st) : xsd_fast_t<bf16>(g, sp_trans, st);
   return rc == BSP_OK ? 1 : rc;
