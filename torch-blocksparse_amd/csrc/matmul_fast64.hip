@@ -620,6 +620,103 @@ template <typename T, int K> __device__ __forceinline__ typename LineMma<T, K>::
   }
 }
 
+// A chain at blocks 16 / 32: the four wavefronts take every fourth entry of the line each, with their own dense rows
+// in their own piece of LDS (no workgroup barrier in the loop), and the four partial results are added through LDS at
+// the end, one 16-row tile at a time.  Ys: four tiles of BLOCK x kLdsRow, Xs: four sparse blocks (transposed variant),
+// red: 16 KiB for the reduction (may overlap Ys and Xs: used after a barrier that ends the loop).
+template <typename T, int BLOCK, bool SP_TRANS>
+__device__ __forceinline__ void xsd_chain_small(const XsdArgs &g, T *Ys, T *Xs, T *Cs, float *red, int z, int n0, int depth, int line,
+                                                table_ptr ent, int ne) {
+  typedef LineMma<T, BLOCK> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int MT = BLOCK / 16, LDX = BLOCK + 8, YT = BLOCK * kLdsRow, XT = BLOCK * LDX;
+  constexpr int NY = BLOCK / 8;                   // 16-byte loads per lane for BLOCK rows of 64 columns
+  constexpr int XB = BLOCK * BLOCK * 2 / 64;
+  constexpr int NX = XB / 16 > 0 ? XB / 16 : 1;
+  typedef typename std::conditional<XB == 8, u32x2, u32x4>::type xreg_t;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int q = lane >> 4, t = lane & 15;
+  const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
+  const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
+  const int64_t ldd = g.ldd;
+  T *Yw = Ys + wave * YT, *Xw = Xs + wave * XT;
+  const int lr = lane >> 3, lc = (lane & 7) * 8;
+  u32x4 y[NY];
+  xreg_t x[NX];
+  auto issue = [&](int e) {
+    const table_ptr en = ent + (G + 1) * e;
+    const T *py = dn + ((int64_t)en[0] * BLOCK + lr) * ldd + lc;
+#pragma unroll
+    for (int i = 0; i < NY; i++) y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)i * 8 * ldd);
+    const T *blk = sp + (int64_t)en[1] * (BLOCK * BLOCK);
+#pragma unroll
+    for (int i = 0; i < NX; i++) {
+      if constexpr (SP_TRANS) x[i] = *reinterpret_cast<const xreg_t *>(blk + (XB == 8 ? lane * 4 : (64 * i + lane) * 8));
+      else x[i] = *reinterpret_cast<const xreg_t *>(XB == 8 ? blk + t * BLOCK + 4 * q : blk + (16 * i + t) * BLOCK + 8 * q);
+    }
+  };
+  f32x4 acc[MT][4];
+#pragma unroll
+  for (int i = 0; i < MT; i++)
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  const int count = (ne - wave + 3) / 4;          // entries wave, wave + 4, ...
+  if (count > 0) issue(wave);
+  for (int k = 0; k < count; k++) {
+#pragma unroll
+    for (int i = 0; i < NY; i++) *reinterpret_cast<u32x4 *>(&Yw[(8 * i + lr) * kLdsRow + lc]) = y[i];
+    frag_t xf[MT];
+    if constexpr (SP_TRANS) {
+#pragma unroll
+      for (int i = 0; i < NX; i++) {
+        const int c = 64 * i + lane;
+        constexpr int CPR = BLOCK * 2 / (int)sizeof(xreg_t), CE = (int)sizeof(xreg_t) / 2;
+        *reinterpret_cast<xreg_t *>(&Xw[(c / CPR) * LDX + (c % CPR) * CE]) = x[i];
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < MT; i++) xf[i] = __builtin_bit_cast(frag_t, x[i]);
+    }
+    __builtin_amdgcn_wave_barrier();              // the LDS operations of one wavefront complete in order
+    frag_t yf[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) yf[j] = line_tr_frag<T, BLOCK>(Yw, kLdsRow, 16 * j, lane);
+    if constexpr (SP_TRANS) {
+#pragma unroll
+      for (int i = 0; i < MT; i++) xf[i] = line_tr_frag<T, BLOCK>(Xw, LDX, 16 * i, lane);
+    }
+    if (k + 1 < count) issue(wave + 4 * (k + 1));  // the registers of this entry are free again
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+      for (int j = 0; j < 4; j++) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);
+    __builtin_amdgcn_wave_barrier();
+  }
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    __syncthreads();                               // the loop's tiles (first round) or the previous sums are no longer read
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+#pragma unroll
+      for (int c = 0; c < 4; c++) red[((wave * 4 + j) * 4 + c) * 64 + lane] = acc[i][j][c];
+    __syncthreads();
+    if (wave == (i & 3)) {
+      f32x4 fin[4];
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+          float v = 0.f;
+#pragma unroll
+          for (int w = 0; w < 4; w++) v += red[((w * 4 + j) * 4 + c) * 64 + lane];
+          fin[j][c] = v;
+        }
+      store_slice<T, true>(Cs + wave * (16 * kLdsRow), po + ((int64_t)line * BLOCK + 16 * i) * g.ldo, g.ldo, fin, lane);
+    }
+  }
+}
+
 constexpr int kSmallRing = 4;
 
 template <typename T, int BLOCK, bool SP_TRANS>
@@ -632,9 +729,16 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
   typedef typename std::conditional<XB == 8, u32x2, u32x4>::type xreg_t;
   constexpr int LDX = BLOCK + 8;
   constexpr int YT = BLOCK * kLdsRow, XT = SP_TRANS ? BLOCK * LDX : 0;
-  __shared__ __attribute__((aligned(16))) T Ys[2][YT];
-  __shared__ __attribute__((aligned(16))) T Xs[4][XT > 0 ? XT : 8];
-  __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
+  // groups: two dense tiles (double buffer); chains: one per wavefront.  The chain's reduction buffer (16 KiB of
+  // floats) lies over the tiles (the front part is as large as the larger of the two) and is only used after a
+  // barrier that ends the chain's loop; the staging rows Cs follow.
+  constexpr int CT = 16 * kLdsRow;
+  constexpr int TILES = 4 * YT + 4 * XT, RED = 16 * 64 * 4 * (int)sizeof(float) / (int)sizeof(T);
+  constexpr int FRONT = TILES > RED ? TILES : RED;
+  __shared__ __attribute__((aligned(16))) T smem[FRONT + 4 * CT];
+  T (*Ys)[YT] = reinterpret_cast<T (*)[YT]>(smem);
+  T (*Xs)[XT > 0 ? XT : 8] = reinterpret_cast<T (*)[XT > 0 ? XT : 8]>(smem + 4 * YT);
+  T (*Cs)[CT] = reinterpret_cast<T (*)[CT]>(smem + FRONT);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int z = blockIdx.x % g.Z;
   const int64_t rest = blockIdx.x / g.Z;
@@ -642,9 +746,12 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
   const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
   const int e0 = hd[0], ne = hd[1], depth = hd[2], code = hd[3];
   const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
-  // a chain (a long line on its own) is a group whose only member is member 0
-  const int line = code < 0 ? -(code + 1) + wave : (code & 0xffffff) * G + wave;
-  const bool mine = code < 0 ? wave == 0 : (line < g.lines && !(((code >> 24) >> wave) & 1));
+  if (code < 0) {   // a chain: the line -(code + 1) on its own
+    xsd_chain_small<T, BLOCK, SP_TRANS>(g, smem, smem + 4 * YT, smem + FRONT, reinterpret_cast<float *>(smem), z, n0, depth, -(code + 1), ent, ne);
+    return;
+  }
+  const int line = (code & 0xffffff) * G + wave;
+  const bool mine = line < g.lines && !(((code >> 24) >> wave) & 1);
   const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;

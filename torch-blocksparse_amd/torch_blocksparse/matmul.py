@@ -197,9 +197,7 @@ class _sparse_matmul(torch.autograd.Function):
         _lib.check(rc, 'bsp_dxx_lut_build')
         lut = lut[:n.value]
         lut.plan = plan
-        # block 64: long lines become chains; blocks 16 and 32: every line stays in its group (their kernel gives a
-        # chain to a single wavefront)
-        lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=None if block == 64 else 0) if block in (16, 32, 64) else None
+        lut.gplan = GroupPlan.build(layout, trans, dev) if block in (16, 32, 64) else None
         return lut, num_locks.value, width.value, None
 
     @staticmethod
