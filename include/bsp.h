@@ -24,6 +24,7 @@ typedef enum { BSP_F16 = 0, BSP_BF16 = 1, BSP_F32 = 2 } bsp_dtype;
 
 typedef enum {
   BSP_OK = 0,
+  BSP_OK_WHOLE_LAYOUT = 1,   /* bsp_sdd_matmul only: the group plan was used, every block of the layout is written */
   BSP_ERR_ARG = -1,          /* null pointer, bad size, misaligned operand */
   BSP_ERR_UNSUPPORTED = -2,  /* block size / dtype / mode not built */
   BSP_ERR_CAPACITY = -3,     /* caller-provided table or workspace too small */
@@ -100,7 +101,9 @@ int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_ro
  * lda / ldb: row stride of the stored 2-D matrices.  n_groups = rows / (pack*pack).
  * d_gplan / n_plan_groups / plan_lines: optional group plan of the layout built with by_rows = 1, its number of
  * groups and the number of block-rows per head (NULL / 0 / 0 if none); when given, a kernel that shares operand
- * tiles inside each group may take the launch. */
+ * tiles inside each group may take the launch.  The plan describes the whole layout, not one pack level: if that
+ * kernel ran, the return value is BSP_OK_WHOLE_LAYOUT and the caller skips the remaining pack levels (pass the plan
+ * with the first level only). */
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
                    int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                    int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,

@@ -60,7 +60,7 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   hipStream_t st = as_stream(stream);
   int rc = generic_only() ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
   if (rc < 0) return rc;
-  if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
+  if (rc >= 1) { BSP_LAUNCH_CHECK(); return rc == 2 ? BSP_OK_WHOLE_LAYOUT : BSP_OK; }
   switch (dtype) {
     case BSP_F16: rc = sdd_generic_f16(g, block, pack, a_kc, b_kc, st); break;
     case BSP_BF16: rc = sdd_generic_bf16(g, block, pack, a_kc, b_kc, st); break;

@@ -834,6 +834,84 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
   }
 }
 
+// sdd at blocks 16 / 32, K = 64, both operands with the reduction contiguous: one wavefront per member of a row
+// group.  The member's rows of A stay in operand registers; per entry (a block-column that some member needs) the
+// BLOCK rows of B are fetched once by the whole workgroup with whole-line loads, pass through LDS (two buffers, one
+// barrier per entry) and serve all four members; a wavefront whose member has a block there multiplies and writes
+// it: a lane holds four consecutive columns of one row, so a 16 x 16 tile leaves as 512 contiguous bytes without a
+// detour through LDS.  (Fetching the rows of B straight into operand layout, one row per lane, was measured 15-55 %
+// slower than the general kernel: neighbouring lanes then never share a cache line.)
+template <typename T, int BLOCK>
+__global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int MT = BLOCK / 16;
+  constexpr int RING = 4;
+  constexpr int YT = BLOCK * kLdsRow;
+  __shared__ __attribute__((aligned(16))) T Ks[2][YT];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int z = blockIdx.x % g.Z;
+  const table_ptr hd = as_table(g.gplan) + 4 * (int64_t)(blockIdx.x / g.Z);
+  const int e0 = hd[0], ne = hd[1], h = hd[2], code = hd[3];
+  if (ne <= 0) return;
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  // (a plan with chains: a chain is a group whose only member is member 0)
+  const int line = code < 0 ? -(code + 1) + wave : (code & 0xffffff) * G + wave;
+  const bool mine = code < 0 ? wave == 0 : (line < g.lines && !(((code >> 24) >> wave) & 1));
+  const int t = lane & 15, q = lane >> 4;
+  const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
+  const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
+  frag_t xq[MT][2];
+#pragma unroll
+  for (int i = 0; i < MT; i++) {
+    const T *p = pa + ((int64_t)(mine ? line : 0) * BLOCK + 16 * i + t) * g.lda + 8 * q;
+    xq[i][0] = *reinterpret_cast<const frag_t *>(p);
+    xq[i][1] = *reinterpret_cast<const frag_t *>(p + 32);
+  }
+  const int yc = tid % (BLOCK * 8), yrow = yc >> 3, ycol = (yc & 7) * 8;   // this thread's 16-byte chunk of the B rows
+  const bool ywrite = tid < BLOCK * 8;
+  u32x4 ring[RING];
+  auto issue = [&](u32x4 &st, int e) {
+    st = *reinterpret_cast<const u32x4 *>(pb + ((int64_t)ent[(G + 1) * e] * BLOCK + yrow) * g.ldb + ycol);
+  };
+  const int last = ne - 1;
+#pragma unroll
+  for (int u = 0; u < RING; u++) issue(ring[u], u < last ? u : last);
+  const int steps = (ne + RING - 1) / RING * RING;
+  for (int e0i = 0; e0i < steps; e0i += RING) {
+#pragma unroll
+    for (int u = 0; u < RING; u++) {
+      const int e = e0i + u;
+      const int buf = e & 1;
+      const int bid0 = ent[(G + 1) * min(e, last) + 1 + wave];
+      const int bid = (e < ne && mine) ? bid0 : -1;
+      if (ywrite) *reinterpret_cast<u32x4 *>(&Ks[buf][yrow * kLdsRow + ycol]) = ring[u];
+      issue(ring[u], e + RING < last ? e + RING : last);
+      __syncthreads();
+      if (bid >= 0) {
+        T *ob = pc + (int64_t)bid * (BLOCK * BLOCK) + t * BLOCK + 4 * q;
+#pragma unroll
+        for (int j = 0; j < MT; j++) {
+          frag_t yf[2];
+#pragma unroll
+          for (int s2 = 0; s2 < 2; s2++) yf[s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + t) * kLdsRow + 32 * s2 + 8 * q]);
+#pragma unroll
+          for (int i = 0; i < MT; i++) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) acc = M::run(yf[s2], xq[i][s2], acc);   // rows n = 16j + 4q + c, column m = 16i + t
+            union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+            for (int c = 0; c < 4; c++) pk.e[c] = from_float<T>(acc[c]);
+            *reinterpret_cast<u32x2 *>(ob + 16 * i * BLOCK + 16 * j) = pk.raw;
+          }
+        }
+      }
+    }
+  }
+}
+
 bool fast_ok_sdd(const SddArgs &g, int block, int pack, bool a_kc, bool b_kc) {
   return block == 64 && pack == 1 && a_kc && b_kc && g.K % 64 == 0;
 }
@@ -857,6 +935,17 @@ template <typename T> int xsd_small_t(const XsdArgs &g, int block, bool sp_trans
     if (sp_trans) hipLaunchKernelGGL((k_xsd_rg_small<T, 32, true>), grid, wg, 0, st, g);
     else hipLaunchKernelGGL((k_xsd_rg_small<T, 32, false>), grid, wg, 0, st, g);
   }
+  return BSP_OK;
+}
+
+bool small_ok_sdd(const SddArgs &g, int block, bool a_kc, bool b_kc) {
+  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && a_kc && b_kc && g.K == 64;
+}
+template <typename T> int sdd_small_t(const SddArgs &g, int block, hipStream_t st) {
+  const int64_t n = (int64_t)g.n_pgroups * g.Z;
+  if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (block == 16) hipLaunchKernelGGL((k_sdd_rg_small<T, 16>), dim3((unsigned)n), dim3(256), 0, st, g);
+  else hipLaunchKernelGGL((k_sdd_rg_small<T, 32>), dim3((unsigned)n), dim3(256), 0, st, g);
   return BSP_OK;
 }
 
@@ -891,8 +980,13 @@ template <typename T> int xsd_fast_t(const XsdArgs &g, bool sp_trans, hipStream_
 
 }  // namespace
 
-// Returns 1 if a specialised kernel took the launch, 0 if the caller should use the general kernel, < 0 on error.
+// Returns 1 if a specialised kernel took the launch (2: through the group plan, which covers every pack level of the
+// layout), 0 if the caller should use the general kernel, < 0 on error.
 int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st) {
+  if (dtype != BSP_F32 && small_ok_sdd(g, block, a_kc, b_kc)) {
+    int rc = dtype == BSP_F16 ? sdd_small_t<f16>(g, block, st) : sdd_small_t<bf16>(g, block, st);
+    return rc == BSP_OK ? 2 : rc;
+  }
   if (dtype == BSP_F32 || !fast_ok_sdd(g, block, pack, a_kc, b_kc)) return 0;
   int rc = dtype == BSP_F16 ? sdd_fast_t<f16>(g, st) : sdd_fast_t<bf16>(g, st);
   return rc == BSP_OK ? 1 : rc;

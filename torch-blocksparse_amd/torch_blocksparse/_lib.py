@@ -16,6 +16,7 @@ F16, BF16, F32 = 0, 1, 2
 DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 
 OK = 0
+OK_WHOLE_LAYOUT = 1   # bsp_sdd_matmul: the group plan was used, every block of the layout is written
 ERR_CAPACITY = -3
 ERR_EMPTY_HEAD = -4
 ERR_ROW_TOO_LONG = -6

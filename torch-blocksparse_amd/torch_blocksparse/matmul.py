@@ -128,7 +128,7 @@ class _sparse_matmul(torch.autograd.Function):
             break
         luts, widths, out_packs = SddTables(), [], []
         luts.nnz = nnz
-        if block == 64:
+        if block in (16, 32, 64):
             luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0)
         done = 0
         for k in range(n_levels.value):
@@ -157,13 +157,18 @@ class _sparse_matmul(torch.autograd.Function):
         total_width = luts.nnz if isinstance(luts, SddTables) else sum(w * p * p for w, p in zip(widths, packs))
         c = torch.empty((AS0, total_width, block, block), dtype=a.dtype, device=a.device)
         timer = _Timer(bench, a.device)
-        gplan = GroupPlan.args(getattr(luts, 'gplan', None) if len(luts) == 1 else None)
+        # the group plan describes the whole layout: it goes with the first pack level, and if the library used it
+        # (status OK_WHOLE_LAYOUT) every block is written and the other levels are skipped
+        gplan = GroupPlan.args(getattr(luts, 'gplan', None))
         for lut, width, pack in zip(luts, widths, packs):
             rc = lib.bsp_sdd_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                     AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
                                     c.stride(0), block, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
                                     gplan[0], gplan[1], gplan[2], _lib.stream_ptr(a.device))
+            if rc == _lib.OK_WHOLE_LAYOUT:
+                break
             _lib.check(rc, 'bsp_sdd_matmul')
+            gplan = GroupPlan.args(None)
         time[0] = timer.done()
         return c
 
