@@ -277,12 +277,16 @@ template <typename T, bool STREAM = false> __device__ __forceinline__ void store
   __builtin_amdgcn_wave_barrier();
 }
 
-// sdd, K = 64: members = block-rows of A (their 16-row slices stay in registers), entries = block-columns (B tiles)
-template <typename T>
+// sdd, K = KD (64 or 128): members = block-rows of A (their 16-row slices stay in registers), entries = block-columns
+// (B tiles of 64 rows x KD)
+template <typename T, int KD>
 __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
-  constexpr int TILE = 64 * kLdsRow;
+  constexpr int NK = KD / 32;                    // MFMA steps along the reduction
+  constexpr int LDK = KD + 8;                    // LDS row of a B tile
+  constexpr int TILE = 64 * LDK;
+  constexpr int CPR = KD / 8, NL = 64 * CPR / 256;   // 16-byte chunks per row, loads per thread and tile
   __shared__ __attribute__((aligned(16))) T Ks[2][TILE];
   __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -294,23 +298,25 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
   const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
   T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
-  frag_t xq[G][2];
+  frag_t xq[G][NK];
 #pragma unroll
   for (int m = 0; m < G; m++) {
     const int row = lg * G + m;
     if (row < g.lines) {
       const T *p = pa + ((int64_t)row * 64 + wave * 16 + r) * g.lda + kq;
-      xq[m][0] = *reinterpret_cast<const frag_t *>(p);
-      xq[m][1] = *reinterpret_cast<const frag_t *>(p + 32);
+#pragma unroll
+      for (int s2 = 0; s2 < NK; s2++) xq[m][s2] = *reinterpret_cast<const frag_t *>(p + 32 * s2);
     }
   }
-  const int ck = tid >> 3, cc = (tid & 7) * 8;
-  struct Stage { u32x4 y[2]; };
+  struct Stage { u32x4 y[NL]; };
   Stage ring[kRing];
   auto issue = [&](Stage &st, int e) {
-    const T *py = pb + ((int64_t)ent[(G + 1) * e] * 64 + ck) * g.ldb + cc;
-    st.y[0] = *reinterpret_cast<const u32x4 *>(py);
-    st.y[1] = *reinterpret_cast<const u32x4 *>(py + 32 * g.ldb);
+    const T *py = pb + (int64_t)ent[(G + 1) * e] * 64 * g.ldb;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const int c = tid + 256 * i;
+      st.y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)(c / CPR) * g.ldb + (c % CPR) * 8);
+    }
   };
 #pragma unroll
   for (int u = 0; u < kRing; u++)
@@ -321,15 +327,18 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
       const int e = e0i + u;
       if (e < ne) {
         const int buf = e & 1;
-        *reinterpret_cast<u32x4 *>(&Ks[buf][ck * kLdsRow + cc]) = ring[u].y[0];
-        *reinterpret_cast<u32x4 *>(&Ks[buf][(ck + 32) * kLdsRow + cc]) = ring[u].y[1];
+#pragma unroll
+        for (int i = 0; i < NL; i++) {
+          const int c = tid + 256 * i;
+          *reinterpret_cast<u32x4 *>(&Ks[buf][(c / CPR) * LDK + (c % CPR) * 8]) = ring[u].y[i];
+        }
         if (e + kRing < ne) issue(ring[u], e + kRing);
         __syncthreads();
-        frag_t yf[4][2];
+        frag_t yf[4][NK];
 #pragma unroll
         for (int j = 0; j < 4; j++)
 #pragma unroll
-          for (int s2 = 0; s2 < 2; s2++) yf[j][s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + r) * kLdsRow + 32 * s2 + kq]);
+          for (int s2 = 0; s2 < NK; s2++) yf[j][s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + r) * LDK + 32 * s2 + kq]);
 #pragma unroll
         for (int m = 0; m < G; m++) {
           const int bid = ent[(G + 1) * e + 1 + m];
@@ -339,7 +348,7 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
             for (int j = 0; j < 4; j++) {
               acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-              for (int s2 = 0; s2 < 2; s2++) acc[j] = M::run(yf[j][s2], xq[m][s2], acc[j]);   // rows n = 16j + 4*(lane/16) + e, column m-row = lane%16
+              for (int s2 = 0; s2 < NK; s2++) acc[j] = M::run(yf[j][s2], xq[m][s2], acc[j]);   // rows n = 16j + 4*(lane/16) + e, column m-row = lane%16
             }
             store_slice<T>(Cs[wave], pc + (int64_t)bid * 4096 + wave * 1024, 64, acc, lane);
           }
@@ -834,20 +843,21 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
   }
 }
 
-// sdd at blocks 16 / 32, K = 64, both operands with the reduction contiguous: one wavefront per member of a row
+// sdd at blocks 16 / 32, K = 64 or 128, both operands with the reduction contiguous: one wavefront per member of a row
 // group.  The member's rows of A stay in operand registers; per entry (a block-column that some member needs) the
 // BLOCK rows of B are fetched once by the whole workgroup with whole-line loads, pass through LDS (two buffers, one
 // barrier per entry) and serve all four members; a wavefront whose member has a block there multiplies and writes
 // it: a lane holds four consecutive columns of one row, so a 16 x 16 tile leaves as 512 contiguous bytes without a
 // detour through LDS.  (Fetching the rows of B straight into operand layout, one row per lane, was measured 15-55 %
 // slower than the general kernel: neighbouring lanes then never share a cache line.)
-template <typename T, int BLOCK>
+template <typename T, int BLOCK, int KD>
 __global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
-  constexpr int MT = BLOCK / 16;
+  constexpr int MT = BLOCK / 16, NK = KD / 32;
   constexpr int RING = 4;
-  constexpr int YT = BLOCK * kLdsRow;
+  constexpr int LDK = KD + 8, YT = BLOCK * LDK;
+  constexpr int CPR = KD / 8, CHUNKS = BLOCK * CPR, NL = (CHUNKS + 255) / 256;   // 16-byte chunks per row and tile, loads per thread
   __shared__ __attribute__((aligned(16))) T Ks[2][YT];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int z = blockIdx.x % g.Z;
@@ -862,18 +872,22 @@ __global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
   const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
   const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
   T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
-  frag_t xq[MT][2];
+  frag_t xq[MT][NK];
 #pragma unroll
   for (int i = 0; i < MT; i++) {
     const T *p = pa + ((int64_t)(mine ? line : 0) * BLOCK + 16 * i + t) * g.lda + 8 * q;
-    xq[i][0] = *reinterpret_cast<const frag_t *>(p);
-    xq[i][1] = *reinterpret_cast<const frag_t *>(p + 32);
+#pragma unroll
+    for (int s2 = 0; s2 < NK; s2++) xq[i][s2] = *reinterpret_cast<const frag_t *>(p + 32 * s2);
   }
-  const int yc = tid % (BLOCK * 8), yrow = yc >> 3, ycol = (yc & 7) * 8;   // this thread's 16-byte chunk of the B rows
-  const bool ywrite = tid < BLOCK * 8;
-  u32x4 ring[RING];
-  auto issue = [&](u32x4 &st, int e) {
-    st = *reinterpret_cast<const u32x4 *>(pb + ((int64_t)ent[(G + 1) * e] * BLOCK + yrow) * g.ldb + ycol);
+  struct Stage { u32x4 y[NL]; };
+  Stage ring[RING];
+  auto issue = [&](Stage &st, int e) {
+    const T *py = pb + (int64_t)ent[(G + 1) * e] * BLOCK * g.ldb;
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      const int c = (tid + 256 * i) % CHUNKS;    // (threads beyond the tile repeat a chunk and do not write it)
+      st.y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)(c / CPR) * g.ldb + (c % CPR) * 8);
+    }
   };
   const int last = ne - 1;
 #pragma unroll
@@ -886,21 +900,25 @@ __global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
       const int buf = e & 1;
       const int bid0 = ent[(G + 1) * min(e, last) + 1 + wave];
       const int bid = (e < ne && mine) ? bid0 : -1;
-      if (ywrite) *reinterpret_cast<u32x4 *>(&Ks[buf][yrow * kLdsRow + ycol]) = ring[u];
+#pragma unroll
+      for (int i = 0; i < NL; i++) {
+        const int c = tid + 256 * i;
+        if (CHUNKS % 256 == 0 || c < CHUNKS) *reinterpret_cast<u32x4 *>(&Ks[buf][(c / CPR) * LDK + (c % CPR) * 8]) = ring[u].y[i];
+      }
       issue(ring[u], e + RING < last ? e + RING : last);
       __syncthreads();
       if (bid >= 0) {
         T *ob = pc + (int64_t)bid * (BLOCK * BLOCK) + t * BLOCK + 4 * q;
 #pragma unroll
         for (int j = 0; j < MT; j++) {
-          frag_t yf[2];
+          frag_t yf[NK];
 #pragma unroll
-          for (int s2 = 0; s2 < 2; s2++) yf[s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + t) * kLdsRow + 32 * s2 + 8 * q]);
+          for (int s2 = 0; s2 < NK; s2++) yf[s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + t) * LDK + 32 * s2 + 8 * q]);
 #pragma unroll
           for (int i = 0; i < MT; i++) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) acc = M::run(yf[s2], xq[i][s2], acc);   // rows n = 16j + 4q + c, column m = 16i + t
+            for (int s2 = 0; s2 < NK; s2++) acc = M::run(yf[s2], xq[i][s2], acc);   // rows n = 16j + 4q + c, column m = 16i + t
             union { u32x2 raw; T e[4]; } pk;
 #pragma unroll
             for (int c = 0; c < 4; c++) pk.e[c] = from_float<T>(acc[c]);
@@ -939,21 +957,25 @@ template <typename T> int xsd_small_t(const XsdArgs &g, int block, bool sp_trans
 }
 
 bool small_ok_sdd(const SddArgs &g, int block, bool a_kc, bool b_kc) {
-  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && a_kc && b_kc && g.K == 64;
+  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && a_kc && b_kc && (g.K == 64 || g.K == 128);
 }
 template <typename T> int sdd_small_t(const SddArgs &g, int block, hipStream_t st) {
   const int64_t n = (int64_t)g.n_pgroups * g.Z;
   if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
-  if (block == 16) hipLaunchKernelGGL((k_sdd_rg_small<T, 16>), dim3((unsigned)n), dim3(256), 0, st, g);
-  else hipLaunchKernelGGL((k_sdd_rg_small<T, 32>), dim3((unsigned)n), dim3(256), 0, st, g);
+  const dim3 grid((unsigned)n), wg(256);
+  if (block == 16 && g.K == 64) hipLaunchKernelGGL((k_sdd_rg_small<T, 16, 64>), grid, wg, 0, st, g);
+  else if (block == 16) hipLaunchKernelGGL((k_sdd_rg_small<T, 16, 128>), grid, wg, 0, st, g);
+  else if (g.K == 64) hipLaunchKernelGGL((k_sdd_rg_small<T, 32, 64>), grid, wg, 0, st, g);
+  else hipLaunchKernelGGL((k_sdd_rg_small<T, 32, 128>), grid, wg, 0, st, g);
   return BSP_OK;
 }
 
 template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
-  if (g.gplan && g.n_pgroups > 0 && g.K == 64 && !g.valid) {
+  if (g.gplan && g.n_pgroups > 0 && (g.K == 64 || g.K == 128) && !g.valid) {
     const int64_t n = (int64_t)g.n_pgroups * g.Z;
     if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
-    hipLaunchKernelGGL(k_sdd64_rg<T>, dim3((unsigned)n), dim3(256), 0, st, g);
+    if (g.K == 64) hipLaunchKernelGGL((k_sdd64_rg<T, 64>), dim3((unsigned)n), dim3(256), 0, st, g);
+    else hipLaunchKernelGGL((k_sdd64_rg<T, 128>), dim3((unsigned)n), dim3(256), 0, st, g);
     return BSP_OK;
   }
   const int64_t n_wg = (g.n_groups * g.Z + 3) / 4;
