@@ -470,11 +470,13 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
   constexpr int RING = XSD_RING;
-  // groups: two dense tiles (+ two sparse tiles when read transposed); chains: one of each per wavefront
-  __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 4) * TILE];
+  // groups: two dense tiles + two sparse tiles when read transposed, else a 16-row slice of each member's block per
+  // wavefront (4 x 4 quarter tiles); chains: one dense and one sparse tile per wavefront
+  __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 6) * TILE];
   T (*Ys)[TILE] = reinterpret_cast<T (*)[TILE]>(smem);
   T (*Xs)[TILE] = reinterpret_cast<T (*)[TILE]>(smem + 2 * TILE);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  T *Xw = smem + 2 * TILE + wave * TILE;   // untransposed groups: this wavefront's slices, member m at Xw + m * 16 * kLdsRow
   const int z = blockIdx.x % g.Z;
   const int64_t rest = blockIdx.x / g.Z;
   const int n0 = (int)(rest % g.n_tiles) * 64;
@@ -490,7 +492,7 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;
   const int ck = tid >> 3, cc = (tid & 7) * 8;
-  const int xr = wave * 16 + (lane & 15), xq = (lane >> 4) * 8;
+  const int xq = (lane >> 4) * 8;
   struct Stage { u32x4 y[2]; u32x4 x[G][2]; };
   Stage ring[RING];
   auto issue = [&](Stage &st, int e) {
@@ -507,7 +509,7 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
       const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * 4096;
       const T *p0, *p1;
       if constexpr (SP_TRANS) { p0 = blk + ck * 64 + cc; p1 = p0 + 32 * 64; }
-      else { p0 = blk + xr * 64 + xq; p1 = p0 + 32; }
+      else { p0 = blk + (wave * 16 + (lane >> 3)) * 64 + (lane & 7) * 8; p1 = p0 + 8 * 64; }   // whole rows: 8 lanes per 128-byte line
       if (bid < 0) { p0 = sp; p1 = sp; }
       st.x[m][0] = *reinterpret_cast<const u32x4 *>(p0);
       st.x[m][1] = *reinterpret_cast<const u32x4 *>(p1);
@@ -559,12 +561,24 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
           }
           if (!live) __syncthreads();   // a padding step still has to order its tile store against the next step
         } else {
+          // The wavefront's 16 rows of each block were fetched line by line (operand layout, one row per lane, costs
+          // 7 % of the launch: neighbouring lanes then never share a cache line); its own piece of LDS turns them into
+          // operand layout.  The LDS operations of one wavefront complete in order: no barrier of its own.
 #pragma unroll
-          for (int m = 0; m < G; m++) {
-            xf[m][0] = __builtin_bit_cast(frag_t, st.x[m][0]);
-            xf[m][1] = __builtin_bit_cast(frag_t, st.x[m][1]);
-          }
+          for (int m = 0; m < G; m++)
+            if (bid[m] >= 0) {
+              T *xm = Xw + m * 16 * kLdsRow;
+              *reinterpret_cast<u32x4 *>(xm + (lane >> 3) * kLdsRow + (lane & 7) * 8) = st.x[m][0];
+              *reinterpret_cast<u32x4 *>(xm + (8 + (lane >> 3)) * kLdsRow + (lane & 7) * 8) = st.x[m][1];
+            }
           __syncthreads();
+#pragma unroll
+          for (int m = 0; m < G; m++)
+            if (bid[m] >= 0) {
+              const T *xm = Xw + m * 16 * kLdsRow + (lane & 15) * kLdsRow + xq;
+              xf[m][0] = *reinterpret_cast<const frag_t *>(xm);
+              xf[m][1] = *reinterpret_cast<const frag_t *>(xm + 32);
+            }
         }
         frag_t yf[2][4];
 #pragma unroll
