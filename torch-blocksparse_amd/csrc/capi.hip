@@ -26,6 +26,7 @@ extern "C" int bsp_version(void) { return 1; }
 extern "C" const char *bsp_strerror(int status) {
   switch (status) {
     case BSP_OK: return "ok";
+    case BSP_OK_WHOLE_LAYOUT: return "ok, every block of the layout written (skip the remaining pack levels)";
     case BSP_ERR_ARG: return "invalid argument (null pointer, bad size or operand not 16-byte aligned)";
     case BSP_ERR_UNSUPPORTED: return "unsupported block size, dtype or problem size";
     case BSP_ERR_CAPACITY: return "caller-provided table or workspace too small";
