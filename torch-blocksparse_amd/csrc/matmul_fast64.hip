@@ -1,8 +1,15 @@
-// Bandwidth-oriented kernels for the attention shapes: block 64, fp16 / bf16, dense operands with a unit stride
-// along the head dimension.  At head_dim 64 every product of the sdd -> softmax -> dsd chain moves ~400 MB for
-// 17 GFLOP (43 flop/byte), i.e. it is bound by HBM, not by the matrix cores; these kernels are organised
-// around keeping many 16-byte loads in flight and touching every byte once.
+// Bandwidth-oriented kernels for the attention shapes: fp16 / bf16, dense operands with a unit stride along the
+// head dimension (64 or 128).  At head_dim 64 every product of the sdd -> softmax -> dsd chain moves ~400 MB for
+// 17 GFLOP (43 flop/byte), i.e. it is bound by HBM, not by the matrix cores; these kernels are organised around
+// keeping many 16-byte loads in flight and touching every byte once.  (The file began with block 64 only, hence its
+// name; blocks 16 and 32 have their own kernels below.)
 //
+//   row-group kernels (need a group plan, see bsp_group_plan_build):
+//   k_sdd64_rg, k_xsd64_rg        : block 64.  A workgroup owns 4 consecutive block-rows (or -columns) of a head; each
+//                                   wavefront computes 16 rows of every member; chains split over the wavefronts.
+//   k_sdd_rg_small, k_xsd_rg_small: blocks 16 and 32.  Same plan, one wavefront per member.
+//
+//   without a plan (block 64):
 //   k_sdd64_nt : C_blk = A[i-rows, :K] . B[j-rows, :K]^T.  One wavefront per output block.  Both operands
 //                have the reduction dimension contiguous, which is exactly the MFMA operand layout (a lane
 //                owns one row and 8 consecutive reduction indices), so they go from global memory straight
