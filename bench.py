@@ -30,10 +30,10 @@ MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
 # the same counter reads for the calibration copy of known size (profiles/attention_seq4096_fp16_blk64.txt).  None = not
 # measured for this build of the kernel.
 TRAFFIC_BYTES = {
-    'sdd_fwd  q.k^T': 140113965 + 268435464, 'sdd_bwd  do.v^T': 140113965 + 268435464,
-    'dsd_fwd  p.v': 342634560 + 67108864, 'dsd_bwd  ds.k': 342634560 + 67108864,
-    'dsd_bwd  p^T.do': 391909043 + 67108864, 'dds_bwd  (q^T.ds)^T': 391909043 + 67108864,
-    'softmax_fwd': 269818136 + 268435456, 'softmax_bwd': 538067580 + 268435456,
+    'sdd_fwd  q.k^T': 143501257 + 268435475, 'sdd_bwd  do.v^T': 143501257 + 268435475,
+    'dsd_fwd  p.v': 362576945 + 67108868, 'dsd_bwd  ds.k': 362576945 + 67108868,
+    'dsd_bwd  p^T.do': 403227301 + 67108864, 'dds_bwd  (q^T.ds)^T': 403227301 + 67108864,
+    'softmax_fwd': 269842570 + 268435456, 'softmax_bwd': 538083047 + 268435456,
 }
 
 
