@@ -255,9 +255,7 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
 // longest-first order.
 // ---------------------------------------------------------------------------------------------------------
 constexpr int G = BSP_GROUP;
-#ifndef XSD_RING
-#define XSD_RING 2
-#endif
+constexpr int kGroupRing = 2;   // register stages of k_xsd64_rg (three were measured 5-8 % slower)
 
 // STREAM: the slice belongs to a dense result, which nothing in the sparse chain reads again: written with streaming
 // stores it does not displace the sparse tensors that the next launches re-read from the memory-side cache
@@ -478,7 +476,7 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
-  constexpr int RING = XSD_RING;
+  constexpr int RING = kGroupRing;
   // groups: two dense tiles + two sparse tiles when read transposed, else a 16-row slice of each member's block per
   // wavefront (4 x 4 quarter tiles); chains: one dense and one sparse tile per wavefront
   __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 6) * TILE];
