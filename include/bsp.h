@@ -83,7 +83,8 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * descending for column groups.  thin_min > 0: a line with at least thin_min blocks leaves its group and becomes a
  * chain of its own (group index field = -(line + 1), member 0 = the line), whose entries bsp_dsd_matmul /
  * bsp_dds_matmul spread over the wavefronts of a workgroup; bits 24..27 of a group's index field mark the members
- * that left it (needs fewer than 2^24 groups per head).  Pass 0 for a plan given to bsp_sdd_matmul.
+ * that left it (needs fewer than 2^24 groups per head), bit 28 is the builder's hint that few groups want each
+ * dense tile (the kernels then fetch those tiles with streaming loads).  Pass 0 for a plan given to bsp_sdd_matmul.
  * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */
 #define BSP_GROUP 4
 int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);

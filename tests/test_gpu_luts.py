@@ -116,6 +116,10 @@ def test_group_plan(by_rows, thin_min):
             for line in range(L):
                 if thin[h, line]:
                     slots.append((-(line + 1), h, entries(h, [line, None, None, None])))
+        # bit 28 of every group's index field: at most 2.5 group entries per dense tile (streaming hint)
+        in_groups = sum(len(e) for code, h, e in slots if code >= 0)
+        hint = 1 if 2 * in_groups <= 5 * H * B else 0
+        slots = [(code | (hint << 28) if code >= 0 else code, h, e) for code, h, e in slots]
         slots.sort(key=lambda s: -len(s[2]))                        # stable: ties stay in slot order
         ng = len(slots)
         assert plan.n_groups == ng and plan.lines == L

@@ -385,7 +385,7 @@ __global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H,
 }
 __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *linecnt, const int32_t *cnt,
                              const int32_t *start, const int32_t *alive, int H, int R, int C, int by_rows, int thin_min,
-                             int64_t n_alive, int32_t *plan) {
+                             int64_t n_alive, int stream_hint, int32_t *plan) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
   const int64_t ng = (int64_t)H * NG, slots = ng + (int64_t)H * L;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
@@ -407,7 +407,7 @@ __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int3
     use[g] = chain ? g == 0 : (line < L && !thin);
     skip |= thin ? 1 << g : 0;
   }
-  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = chain ? -(first + 1) : (first / BSP_GROUP) | (skip << 24);
+  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = chain ? -(first + 1) : (first / BSP_GROUP) | (skip << 24) | (stream_hint << 28);
   for (int bb = 0; bb < B; bb++) {
     // Column groups list their positions from the last one down: the long lines of a causal layout (global
     // columns) then walk the dense operand's rows in step with each other and share them in L2 (measured: 12 % fewer
@@ -629,15 +629,21 @@ extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C
   hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.gcnt, ws + o.gstart, slots, (int32_t *)nullptr);
   hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.galive, ws + o.gapos, slots, (int32_t *)nullptr);
   BSP_LAUNCH_CHECK();
-  int32_t total = 0, n_alive = 0;
+  int32_t total = 0, n_alive = 0, in_groups = 0;
   BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.gstart + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
+  BSP_HIP_CHECK(hipMemcpyAsync(&in_groups, ws + o.gstart + ng, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipMemcpyAsync(&n_alive, ws + o.gapos + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   *n_groups = (int)n_alive;
   *plan_len = 4 * (int64_t)n_alive + (int64_t)(BSP_GROUP + 1) * total;
   if (*plan_len > plan_cap) return BSP_ERR_CAPACITY;
+  // Streaming hint (bit 28 of every group's index field): set when a dense tile is wanted by few groups (at most
+  // 2.5 group entries per tile of the other dimension).  The kernels then fetch the dense tiles with streaming loads,
+  // which keeps them out of the memory-side cache: measured 8 % faster on the fixed attention layout (1.0-1.4 entries
+  // per tile), 20-30 % slower on the long-context layout with random blocks (3.9-4.5), whose tiles come back later.
+  const int stream_hint = 2 * (int64_t)in_groups <= 5 * (int64_t)H * (by_rows ? C : R);
   hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, ws + o.rank, linecnt, ws + o.gcnt, ws + o.gstart,
-                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, d_plan);
+                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, stream_hint, d_plan);
   BSP_LAUNCH_CHECK();
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;

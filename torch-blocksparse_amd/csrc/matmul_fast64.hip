@@ -284,20 +284,20 @@ template <typename T, bool STREAM = false> __device__ __forceinline__ void store
 
 // sdd, K = KD (64 or 128): members = block-rows of A (their 16-row slices stay in registers), entries = block-columns
 // (B tiles of 64 rows x KD)
-template <typename T, int KD>
-__global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
+template <typename T, int KD, bool STREAM>
+__device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int NK = KD / 32;                    // MFMA steps along the reduction
   constexpr int LDK = KD + 8;                    // LDS row of a B tile
   constexpr int TILE = 64 * LDK;
   constexpr int CPR = KD / 8, NL = 64 * CPR / 256;   // 16-byte chunks per row, loads per thread and tile
-  __shared__ __attribute__((aligned(16))) T Ks[2][TILE];
-  __shared__ __attribute__((aligned(16))) T Cs[4][16 * kLdsRow];
+  T (*Ks)[TILE] = reinterpret_cast<T (*)[TILE]>(smem);                              // two B tiles
+  T (*Cs)[16 * kLdsRow] = reinterpret_cast<T (*)[16 * kLdsRow]>(smem + 2 * TILE);   // a 16-row staging slice per wavefront
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int z = blockIdx.x % g.Z;
   const table_ptr hd = as_table(g.gplan) + 4 * (int64_t)(blockIdx.x / g.Z);
-  const int e0 = hd[0], ne = hd[1], h = hd[2], lg = hd[3];
+  const int e0 = hd[0], ne = hd[1], h = hd[2], lg = hd[3] & 0xffffff;
   const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
   const int r = lane & 15, kq = (lane >> 4) * 8;
   const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
@@ -320,9 +320,11 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
 #pragma unroll
     for (int i = 0; i < NL; i++) {
       const int c = tid + 256 * i;
-      // streaming loads: the dense operands are small and shared through L2; kept out of the memory-side cache they
-      // leave it to the sparse result that the next launch reads (measured: 3-4 us per launch)
-      st.y[i] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(py + (int64_t)(c / CPR) * g.ldb + (c % CPR) * 8));
+      // streaming loads where the plan says so: tiles that few groups want, kept out of the memory-side cache, leave
+      // it to the sparse result that the next launch reads (measured: 3-4 us per launch on the fixed attention layout)
+      const u32x4 *pt = reinterpret_cast<const u32x4 *>(py + (int64_t)(c / CPR) * g.ldb + (c % CPR) * 8);
+      if constexpr (STREAM) st.y[i] = __builtin_nontemporal_load(pt);
+      else st.y[i] = *pt;
     }
   };
 #pragma unroll
@@ -363,6 +365,17 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
       }
     }
   }
+}
+
+// The streaming hint is a property of the whole plan (bit 28 of every group's index field), so all workgroups of a
+// launch take the same side of this branch.  Two copies of the body rather than a condition at the load: the
+// compiler merges two loads of one address that differ only in the hint, and drops the hint.
+template <typename T, int KD>
+__global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
+  __shared__ __attribute__((aligned(16))) T smem[2 * 64 * (KD + 8) + 4 * 16 * kLdsRow];
+  const int code = as_table(g.gplan)[4 * (int64_t)(blockIdx.x / g.Z) + 3];
+  if ((code >> 28) & 1) sdd64_rg_body<T, KD, true>(g, smem);
+  else sdd64_rg_body<T, KD, false>(g, smem);
 }
 
 // A chain = one output line with many blocks (the plan builder takes such lines out of their groups).  Walking its
@@ -471,15 +484,12 @@ __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int 
 }
 
 // dsd / dds: members = output lines (block-rows of the result), entries = positions of the reduction
-template <typename T, bool SP_TRANS>
-__global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
+template <typename T, bool SP_TRANS, bool STREAM>
+__device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
   constexpr int RING = kGroupRing;
-  // groups: two dense tiles + two sparse tiles when read transposed, else a 16-row slice of each member's block per
-  // wavefront (4 x 4 quarter tiles); chains: one dense and one sparse tile per wavefront
-  __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 6) * TILE];
   T (*Ys)[TILE] = reinterpret_cast<T (*)[TILE]>(smem);
   T (*Xs)[TILE] = reinterpret_cast<T (*)[TILE]>(smem + 2 * TILE);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -494,7 +504,7 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
     xsd_chain<T, SP_TRANS>(g, smem, z, n0, depth, -(code + 1), ent, ne);
     return;
   }
-  const int lg = code & 0xffffff, skip = code >> 24;   // members whose line is a chain are left to that chain
+  const int lg = code & 0xffffff, skip = (code >> 24) & 0xf;   // members whose line is a chain are left to that chain
   const T *sp = reinterpret_cast<const T *>(g.sp) + z * g.sp_sz;
   const T *dn = reinterpret_cast<const T *>(g.dn) + z * g.dn_sz + depth * g.dn_sh + n0;
   const int64_t ldd = g.ldd;
@@ -505,9 +515,11 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   auto issue = [&](Stage &st, int e) {
     const table_ptr en = ent + (G + 1) * e;
     const T *py = dn + ((int64_t)en[0] * 64 + ck) * ldd + cc;
-    // streaming loads for the dense tiles (shared through L2, kept out of the memory-side cache: 6 us per launch)
-    st.y[0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(py));
-    st.y[1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(py + 32 * ldd));
+    // streaming loads for the dense tiles where the plan says so (kept out of the memory-side cache: 6 us per launch
+    // on the fixed attention layout)
+    const u32x4 *q0 = reinterpret_cast<const u32x4 *>(py), *q1 = reinterpret_cast<const u32x4 *>(py + 32 * ldd);
+    if constexpr (STREAM) { st.y[0] = __builtin_nontemporal_load(q0); st.y[1] = __builtin_nontemporal_load(q1); }
+    else { st.y[0] = *q0; st.y[1] = *q1; }
     // A fixed number of loads per stage whatever the entry holds, so that the wait before a stage is consumed can
     // count exactly the loads issued after it (a data-dependent count would force a wait for everything in flight).
     // Absent members read one cache line at the start of the sparse tensor instead.
@@ -617,6 +629,17 @@ __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
     const int line = lg * G + m;
     if (line < g.lines && !((skip >> m) & 1)) store_slice<T, true>(cs, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, acc[m], lane);
   }
+}
+
+// (two copies of the body, chosen by the plan's streaming hint: see k_sdd64_rg)
+template <typename T, bool SP_TRANS>
+__global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
+  // groups: two dense tiles + two sparse tiles when read transposed, else a 16-row slice of each member's block per
+  // wavefront (4 x 4 quarter tiles); chains: one dense and one sparse tile per wavefront
+  __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 6) * 64 * kLdsRow];
+  const int code = as_table(g.gplan)[4 * ((int64_t)(blockIdx.x / g.Z) / g.n_tiles) + 3];
+  if (code >= 0 && ((code >> 28) & 1)) xsd64_rg_body<T, SP_TRANS, true>(g, smem);
+  else xsd64_rg_body<T, SP_TRANS, false>(g, smem);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -750,23 +773,27 @@ __device__ __forceinline__ void xsd_chain_small(const XsdArgs &g, T *Ys, T *Xs, 
 
 constexpr int kSmallRing = 4;
 
-template <typename T, int BLOCK, bool SP_TRANS>
-__global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
+// LDS of k_xsd_rg_small.  groups: two dense tiles (double buffer); chains: one per wavefront.  The chain's reduction
+// buffer (16 KiB of floats) lies over the tiles (the front part is as large as the larger of the two) and is only
+// used after a barrier that ends the chain's loop; the staging rows Cs follow.
+template <typename T, int BLOCK, bool SP_TRANS> struct SmallXsdLds {
+  static constexpr int LDX = BLOCK + 8;
+  static constexpr int YT = BLOCK * kLdsRow, XT = SP_TRANS ? BLOCK * LDX : 0, CT = 16 * kLdsRow;
+  static constexpr int TILES = 4 * YT + 4 * XT, RED = 16 * 64 * 4 * (int)sizeof(float) / (int)sizeof(T);
+  static constexpr int FRONT = TILES > RED ? TILES : RED;
+  static constexpr int ELEMS = FRONT + 4 * CT;
+};
+
+template <typename T, int BLOCK, bool SP_TRANS, bool STREAM>
+__device__ __forceinline__ void xsd_rg_small_body(const XsdArgs &g, T *smem) {
   typedef LineMma<T, BLOCK> M;
   typedef typename M::frag_t frag_t;
   constexpr int MT = BLOCK / 16;                 // 16-row tiles of a line
   constexpr int XB = BLOCK * BLOCK * 2 / 64;     // bytes of a sparse block per lane: 8 (block 16) or 32
   constexpr int NX = XB / 16 > 0 ? XB / 16 : 1;  // loads per lane: one of 8 bytes, or two of 16
   typedef typename std::conditional<XB == 8, u32x2, u32x4>::type xreg_t;
-  constexpr int LDX = BLOCK + 8;
-  constexpr int YT = BLOCK * kLdsRow, XT = SP_TRANS ? BLOCK * LDX : 0;
-  // groups: two dense tiles (double buffer); chains: one per wavefront.  The chain's reduction buffer (16 KiB of
-  // floats) lies over the tiles (the front part is as large as the larger of the two) and is only used after a
-  // barrier that ends the chain's loop; the staging rows Cs follow.
-  constexpr int CT = 16 * kLdsRow;
-  constexpr int TILES = 4 * YT + 4 * XT, RED = 16 * 64 * 4 * (int)sizeof(float) / (int)sizeof(T);
-  constexpr int FRONT = TILES > RED ? TILES : RED;
-  __shared__ __attribute__((aligned(16))) T smem[FRONT + 4 * CT];
+  typedef SmallXsdLds<T, BLOCK, SP_TRANS> LD;
+  constexpr int LDX = LD::LDX, YT = LD::YT, XT = LD::XT, CT = LD::CT, FRONT = LD::FRONT;
   T (*Ys)[YT] = reinterpret_cast<T (*)[YT]>(smem);
   T (*Xs)[XT > 0 ? XT : 8] = reinterpret_cast<T (*)[XT > 0 ? XT : 8]>(smem + 4 * YT);
   T (*Cs)[CT] = reinterpret_cast<T (*)[CT]>(smem + FRONT);
@@ -795,10 +822,11 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
   // absent block reads one line at the start of the sparse tensor.
   auto issue = [&](Stage &st, int e) {
     const table_ptr en = ent + (G + 1) * e;
-    // (streaming loads of the dense rows: 4-6 us less at block 32, 3-5 us more at block 16, where four times as many
-    // workgroups ask for each row)
+    // (streaming loads of the dense rows where the plan says so: 4-6 us less at block 32 on the fixed attention
+    // layout, 3-5 us more at block 16, where four times as many groups ask for each row)
     const u32x4 *py = reinterpret_cast<const u32x4 *>(dn + ((int64_t)en[0] * BLOCK + yrow) * ldd + ycol);
-    st.y = BLOCK == 32 ? __builtin_nontemporal_load(py) : *py;
+    if constexpr (STREAM) st.y = __builtin_nontemporal_load(py);
+    else st.y = *py;
     const int bid = en[1 + wave];
     const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * (BLOCK * BLOCK);
 #pragma unroll
@@ -866,6 +894,17 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
     for (int i = 0; i < MT; i++)
       store_slice<T, true>(Cs[wave], po + ((int64_t)line * BLOCK + 16 * i) * g.ldo, g.ldo, acc[i], lane);
   }
+}
+
+// (two copies of the body, chosen by the plan's streaming hint: see k_sdd64_rg)
+template <typename T, int BLOCK, bool SP_TRANS>
+__global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
+  __shared__ __attribute__((aligned(16))) T smem[SmallXsdLds<T, BLOCK, SP_TRANS>::ELEMS];
+  const int code = as_table(g.gplan)[4 * ((int64_t)(blockIdx.x / g.Z) / g.n_tiles) + 3];
+  // (block 16 ignores the hint: with four times as many groups per dense row as block 64, streaming loads were
+  // measured 3-15 % slower there whatever the plan says)
+  if (BLOCK != 16 && code >= 0 && ((code >> 28) & 1)) xsd_rg_small_body<T, BLOCK, SP_TRANS, true>(g, smem);
+  else xsd_rg_small_body<T, BLOCK, SP_TRANS, false>(g, smem);
 }
 
 // sdd at blocks 16 / 32, K = 64 or 128, both operands with the reduction contiguous: one wavefront per member of a row
