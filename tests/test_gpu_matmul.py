@@ -215,3 +215,48 @@ def test_linear_module():
     y.sum().backward()
     assert lin.weight.grad.shape == lin.weight.shape and x.grad.shape == x.shape
     assert_close(x.grad, torch.ones(5, 7, 384) @ wd.t(), torch.float16, 'linear dx')
+
+
+def test_random_attention_shapes_specialised_against_general(monkeypatch):
+    # 60 random layouts / block sizes / head dimensions / dtypes: the row-group kernels (blocks 16, 32, 64) must agree
+    # with the general kernels on the same inputs; covers ragged groups, empty and full lines, chains, one to three batches
+    import random
+    rnd = random.Random(7)
+    for it in range(60):
+        block = rnd.choice([16, 32, 64])
+        H, R, C = rnd.randint(1, 4), rnd.randint(1, 30), rnd.randint(1, 30)
+        lay = random_layout((H, R, C), rnd.choice([0.05, 0.2, 0.5, 0.9, 1.0]), it)
+        if rnd.random() < 0.3 and R > 2:
+            lay[:, rnd.randrange(R), :] = 1
+        if rnd.random() < 0.3 and C > 2:
+            lay[:, :, rnd.randrange(C)] = 1
+        lay[:, 0, 0] = 1                                  # no empty head
+        Z, free = rnd.randint(1, 3), rnd.choice([64, 128])
+        dtype = rnd.choice([torch.float16, torch.bfloat16])
+        mode = rnd.choice(['dsd', 'dsd_t', 'sdd', 'sdd_bwd'])
+        nnz = int(lay.sum())
+        g = torch.Generator().manual_seed(it)
+        mk = lambda *shape: torch.randn(*shape, generator=g).to(dtype).to(DEV)
+        if mode == 'dsd':
+            ops = (mk(Z, nnz, block, block), mk(Z, H, C * block, free))
+            f = lambda a, b: tb.MatMul(lay, block, 'dsd')(a, b)
+        elif mode == 'dsd_t':
+            ops = (mk(Z, nnz, block, block), mk(Z, H, R * block, free))
+            f = lambda a, b: tb.MatMul(lay, block, 'dsd', trans_a=True)(a, b)
+        else:
+            ops = (mk(Z, H, R * block, free), mk(Z, H, C * block, free), mk(Z, nnz, block, block))
+
+            def f(a, b, dc=None, bwd=(mode == 'sdd_bwd')):
+                a, b = a.clone().requires_grad_(bwd), b.clone().requires_grad_(bwd)
+                c = tb.MatMul(lay, block, 'sdd', trans_b=True)(a, b)
+                if not bwd:
+                    return c
+                c.backward(ops[2])
+                return torch.cat([a.grad.flatten(), b.grad.flatten()])
+        monkeypatch.delenv('BSP_GENERIC_ONLY', raising=False)
+        x = f(*ops[:2]).float()
+        monkeypatch.setenv('BSP_GENERIC_ONLY', '1')
+        y = f(*ops[:2]).float()
+        monkeypatch.delenv('BSP_GENERIC_ONLY', raising=False)
+        tol = (2e-2 if dtype == torch.bfloat16 else 4e-3) * (float(y.abs().max()) + 1e-6)
+        assert torch.isfinite(x).all() and float((x - y).abs().max()) <= tol, (it, mode, block, H, R, C, Z, free, dtype)
