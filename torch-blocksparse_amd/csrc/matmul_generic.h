@@ -83,11 +83,13 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   static constexpr int ITER = (NCH + NT - 1) / NT;
   static constexpr int CPR = TK / VE;    // chunks per row when the reduction is contiguous
   static constexpr int RCH = ROWS / VE;  // chunks per reduction index otherwise
-  // A 16-bit operand stored with the reduction dimension strided is kept in LDS as it lies in memory, [TK][ROWS + 8],
-  // and handed to the MFMA through the transposing LDS read; a 32-bit one is transposed while it is written.
-  static constexpr bool TR = !KCONTIG && sizeof(T) == 2;
+  // An operand stored with the reduction dimension strided is kept in LDS as it lies in memory, [TK][ROWS + 8].  A
+  // 16-bit one is handed to the MFMA through the transposing LDS read; a 32-bit one needs no transposition at all:
+  // its MFMA operand is a single element per lane, (row lane % MS, reduction index lane / MS), read where it lies.
+  static constexpr bool ASIS = !KCONTIG;
+  static constexpr bool TR = ASIS && sizeof(T) == 2;
   static constexpr int LDR = ROWS + 8;
-  static constexpr int ELEMS = TR ? TK * LDR : ROWS * LDK;
+  static constexpr int ELEMS = ASIS ? TK * LDR : ROWS * LDK;
   u32x4 reg[ITER];
   bool ok[ITER];
 
@@ -100,14 +102,8 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
         const u32x4 val = ok[it] ? reg[it] : z;
         if constexpr (KCONTIG) {
           *reinterpret_cast<u32x4 *>(S + (c / CPR) * LDK + (c % CPR) * VE) = val;
-        } else if constexpr (TR) {
-          *reinterpret_cast<u32x4 *>(S + (c / RCH) * LDR + (c % RCH) * VE) = val;
         } else {
-          union { u32x4 raw; T e[VE]; } u;
-          u.raw = val;
-          const int row0 = (c % RCH) * VE, k = c / RCH;
-#pragma unroll
-          for (int e = 0; e < VE; e++) S[(row0 + e) * LDK + k] = u.e[e];
+          *reinterpret_cast<u32x4 *>(S + (c / RCH) * LDR + (c % RCH) * VE) = val;
         }
       }
     }
@@ -125,6 +121,9 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
       typedef short s16x8 __attribute__((ext_vector_type(8)));
       s16x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       return __builtin_bit_cast(typename M::frag_t, v);
+    } else if constexpr (ASIS) {
+      static_assert(M::KV == 1, "32-bit operands: one element per lane");
+      return S[(kk * M::KSTEP + lane / MS) * LDR + row0 + lane % MS];
     } else {
       return *reinterpret_cast<const typename M::frag_t *>(S + (row0 + lane % MS) * LDK + (lane / MS) * M::KV + kk * M::KSTEP);
     }
