@@ -182,9 +182,14 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
           P p;
           p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
 #pragma unroll
-          for (int e = 0; e < GE::EV; e++) {
-            const float m = to_float(p.e[e]);
-            kpm_s[c * GE::EV + e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+          for (int e4 = 0; e4 < GE::EV; e4 += 4) {       // EV is 4 or 8: whole 16-byte LDS accesses
+            f32x4 add;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+              const float m = to_float(p.e[e4 + e]);
+              add[e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+            }
+            *reinterpret_cast<f32x4 *>(&kpm_s[c * GE::EV + e4]) = add;
           }
         }
       }
@@ -196,7 +201,12 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
     for (int b = 0; b < NB; b++)
       if (b < size) {                                   // softmax.py:112-116, 122-124
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(px[b].e[e]), sc, has_kpm ? kpm_s[b * BLOCK + u.col + e] : 0.f);
+        for (int e4 = 0; e4 < GE::EV; e4 += 4) {
+          const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+          const f32x4 add = has_kpm ? *reinterpret_cast<const f32x4 *>(&kpm_s[b * BLOCK + u.col + e4]) : zero4;
+#pragma unroll
+          for (int e = 0; e < 4; e++) fx[b][e4 + e] = fmaf(to_float(px[b].e[e4 + e]), sc, add[e]);
+        }
         // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
         // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
         if constexpr (NB >= 16) __builtin_amdgcn_sched_barrier(0);
