@@ -910,19 +910,22 @@ __global__ void __launch_bounds__(256) k_xsd_rg_small(XsdArgs g) {
 // sdd at blocks 16 / 32, K = 64 or 128, both operands with the reduction contiguous: one wavefront per member of a row
 // group.  The member's rows of A stay in operand registers; per entry (a block-column that some member needs) the
 // BLOCK rows of B are fetched once by the whole workgroup with whole-line loads, pass through LDS (two buffers, one
-// barrier per entry) and serve all four members; a wavefront whose member has a block there multiplies and writes
-// it: a lane holds four consecutive columns of one row, so a 16 x 16 tile leaves as 512 contiguous bytes without a
-// detour through LDS.  (Fetching the rows of B straight into operand layout, one row per lane, was measured 15-55 %
+// barrier per 64 rows: four entries at block 16, two at block 32) and serve all four members; a wavefront whose member has a block there multiplies and writes
+// it through its own piece of LDS, 16 bytes per lane in address order.  (Fetching the rows of B straight into operand layout, one row per lane, was measured 15-55 %
 // slower than the general kernel: neighbouring lanes then never share a cache line.)
 template <typename T, int BLOCK, int KD>
 __global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int MT = BLOCK / 16, NK = KD / 32;
-  constexpr int RING = 4;
-  constexpr int LDK = KD + 8, YT = BLOCK * LDK;
-  constexpr int CPR = KD / 8, CHUNKS = BLOCK * CPR, NL = (CHUNKS + 255) / 256;   // 16-byte chunks per row and tile, loads per thread
+  constexpr int EB = 64 / BLOCK;                 // entries per step: 64 rows of B per barrier, as at block 64
+  constexpr int RING = 2;
+  constexpr int LDK = KD + 8, YT = EB * BLOCK * LDK;
+  constexpr int CPR = KD / 8, CHUNKS = EB * BLOCK * CPR, NL = CHUNKS / 256;   // 16-byte chunks per row and step, loads per thread
+  static_assert(CHUNKS % 256 == 0, "a step's rows of B divide evenly among the threads");
+  constexpr int LDC = BLOCK + 8;                 // staging row of a result block
   __shared__ __attribute__((aligned(16))) T Ks[2][YT];
+  __shared__ __attribute__((aligned(16))) T Cs[4][EB * BLOCK * LDC];
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int z = blockIdx.x % g.Z;
   const table_ptr hd = as_table(g.gplan) + 4 * (int64_t)(blockIdx.x / g.Z);
@@ -945,51 +948,78 @@ __global__ void __launch_bounds__(256) k_sdd_rg_small(SddArgs g) {
   }
   struct Stage { u32x4 y[NL]; };
   Stage ring[RING];
-  auto issue = [&](Stage &st, int e) {
-    const T *py = pb + (int64_t)ent[(G + 1) * e] * BLOCK * g.ldb;
+  const int last = ne - 1;
+  // step s = entries EB * s ..; entries past the end repeat the last one (loaded, not used): a fixed number of loads
+  auto issue = [&](Stage &st, int s) {
 #pragma unroll
     for (int i = 0; i < NL; i++) {
-      const int c = (tid + 256 * i) % CHUNKS;    // (threads beyond the tile repeat a chunk and do not write it)
-      st.y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)(c / CPR) * g.ldb + (c % CPR) * 8);
+      const int c = tid + 256 * i, r = c / CPR;              // row of the step's EB * BLOCK rows
+      const int e = min(EB * s + r / BLOCK, last);
+      st.y[i] = *reinterpret_cast<const u32x4 *>(pb + ((int64_t)ent[(G + 1) * e] * BLOCK + r % BLOCK) * g.ldb + (c % CPR) * 8);
     }
   };
-  const int last = ne - 1;
+  const int nsteps = (ne + EB - 1) / EB, slast = nsteps - 1;
 #pragma unroll
-  for (int u = 0; u < RING; u++) issue(ring[u], u < last ? u : last);
-  const int steps = (ne + RING - 1) / RING * RING;
-  for (int e0i = 0; e0i < steps; e0i += RING) {
+  for (int u = 0; u < RING; u++) issue(ring[u], u < slast ? u : slast);
+  const int steps = (nsteps + RING - 1) / RING * RING;
+  for (int s0 = 0; s0 < steps; s0 += RING) {
 #pragma unroll
     for (int u = 0; u < RING; u++) {
-      const int e = e0i + u;
-      const int buf = e & 1;
-      const int bid0 = ent[(G + 1) * min(e, last) + 1 + wave];
-      const int bid = (e < ne && mine) ? bid0 : -1;
+      const int s = s0 + u;
+      const int buf = s & 1;
 #pragma unroll
       for (int i = 0; i < NL; i++) {
         const int c = tid + 256 * i;
-        if (CHUNKS % 256 == 0 || c < CHUNKS) *reinterpret_cast<u32x4 *>(&Ks[buf][(c / CPR) * LDK + (c % CPR) * 8]) = ring[u].y[i];
+        *reinterpret_cast<u32x4 *>(&Ks[buf][(c / CPR) * LDK + (c % CPR) * 8]) = ring[u].y[i];
       }
-      issue(ring[u], e + RING < last ? e + RING : last);
+      issue(ring[u], s + RING < slast ? s + RING : slast);
       __syncthreads();
-      if (bid >= 0) {
-        T *ob = pc + (int64_t)bid * (BLOCK * BLOCK) + t * BLOCK + 4 * q;
+      // The step's blocks of this member are computed into the wavefront's own piece of LDS (a lane holds 8 bytes of a
+      // row, neighbouring lanes different rows) and leave from there in address order, 1 KiB per store instruction:
+      // a block of 32 as two stores, two blocks of 16 as one (measured at block 32: 94 -> 77 us against storing from
+      // the accumulators).
+      int bids[EB];
 #pragma unroll
-        for (int j = 0; j < MT; j++) {
-          frag_t yf[NK];
+      for (int k = 0; k < EB; k++) {
+        const int e = EB * s + k;
+        const int bid0 = ent[(G + 1) * min(e, last) + 1 + wave];
+        bids[k] = (e < ne && mine) ? bid0 : -1;
+        if (bids[k] >= 0) {
+          T *cw = Cs[wave] + k * (BLOCK * LDC);
 #pragma unroll
-          for (int s2 = 0; s2 < NK; s2++) yf[s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + t) * LDK + 32 * s2 + 8 * q]);
+          for (int j = 0; j < MT; j++) {
+            frag_t yf[NK];
 #pragma unroll
-          for (int i = 0; i < MT; i++) {
-            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+            for (int s2 = 0; s2 < NK; s2++) yf[s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(k * BLOCK + 16 * j + t) * LDK + 32 * s2 + 8 * q]);
 #pragma unroll
-            for (int s2 = 0; s2 < NK; s2++) acc = M::run(yf[s2], xq[i][s2], acc);   // rows n = 16j + 4q + c, column m = 16i + t
-            union { u32x2 raw; T e[4]; } pk;
+            for (int i = 0; i < MT; i++) {
+              f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < 4; c++) pk.e[c] = from_float<T>(acc[c]);
-            *reinterpret_cast<u32x2 *>(ob + 16 * i * BLOCK + 16 * j) = pk.raw;
+              for (int s2 = 0; s2 < NK; s2++) acc = M::run(yf[s2], xq[i][s2], acc);   // rows n = 16j + 4q + c, column m = 16i + t
+              union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+              for (int c = 0; c < 4; c++) pk.e[c] = from_float<T>(acc[c]);
+              *reinterpret_cast<u32x2 *>(cw + (16 * i + t) * LDC + 16 * j + 4 * q) = pk.raw;
+            }
           }
         }
       }
+      __builtin_amdgcn_wave_barrier();                 // the LDS operations of one wavefront complete in order
+      constexpr int CPB = BLOCK * BLOCK / 8, RC = BLOCK / 8;   // 16-byte chunks per block and per row
+      constexpr int BPI = CPB >= 64 ? 1 : 64 / CPB;            // blocks per store instruction
+#pragma unroll
+      for (int k0 = 0; k0 < EB; k0 += BPI)
+#pragma unroll
+        for (int i = 0; i < (CPB * BPI) / 64; i++) {
+          const int c = lane + 64 * i;                  // chunk among the BPI blocks k0 ..
+          int bid = bids[k0];
+#pragma unroll
+          for (int p = 1; p < BPI; p++) bid = (c / CPB == p) ? bids[k0 + p] : bid;
+          const int cb = c % CPB;
+          const T *src = Cs[wave] + (k0 + c / CPB) * (BLOCK * LDC) + (cb / RC) * LDC + (cb % RC) * 8;
+          if (bid >= 0) *reinterpret_cast<u32x4 *>(pc + (int64_t)bid * (BLOCK * BLOCK) + cb * 8) = *reinterpret_cast<const u32x4 *>(src);
+        }
+      __builtin_amdgcn_wave_barrier();
     }
   }
 }
