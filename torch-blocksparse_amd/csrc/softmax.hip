@@ -207,31 +207,23 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
 #pragma unroll
           for (int e = 0; e < 4; e++) fx[b][e4 + e] = fmaf(to_float(px[b].e[e4 + e]), sc, add[e]);
         }
-        // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
-        // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
-        if constexpr (NB >= 16) __builtin_amdgcn_sched_barrier(0);
-      }
-    if constexpr (EXTRA) {
-      if (a.rpe) {                                      // :118-120
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-          if (b < size) {
+        if constexpr (EXTRA) {                          // all terms of a block in one place: its raw registers die here
+          if (a.rpe) {                                    // :118-120
 #pragma unroll
             for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(pr[b].e[e]), unit, fx[b][e]);
           }
-      }
-      if (a.attn) {                                     // :126-128, 'mul' mode :108-110
-#pragma unroll
-        for (int b = 0; b < NB; b++)
-          if (b < size) {
+          if (a.attn) {                                   // :126-128, 'mul' mode :108-110
 #pragma unroll
             for (int e = 0; e < GE::EV; e++) {
               const float m = to_float(pa[b].e[e]);
               fx[b][e] += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
             }
           }
+        }
+        // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
+        // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
+        if constexpr (NB >= 16 || (EXTRA && NB >= 8)) __builtin_amdgcn_sched_barrier(0);
       }
-    }
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
