@@ -145,6 +145,13 @@ def test_small_block_row_groups(block, dtype):
         run_case('dsd', False, False, block, dtype, Z=2, H=3, M=n * block, K=n * block, N=free, layout=lay, seed=block + free, dist='randn', scale=0.25)
         run_case('dsd', True, False, block, dtype, Z=2, H=3, M=n * block, K=n * block, N=free, layout=lay, seed=block + free + 1, dist='randn', scale=0.25)
         run_case('sdd', False, True, block, dtype, Z=2, H=3, M=n * block, N=n * block, K=free, layout=lay, seed=block + free + 2, dist='randn', scale=0.25)
+    # lines of 128 blocks and more become chains (split over the wavefronts): a full block-column of 132 and, seen from
+    # the transposed product, a full block-row
+    tall = random_layout((2, 132, 6), 0.2, 5 + block)
+    tall[:, :, 2] = 1
+    run_case('dsd', True, False, block, dtype, Z=2, H=2, M=6 * block, K=132 * block, N=64, layout=tall, seed=block + 3, dist='randn', scale=0.1)
+    wide = tall.transpose(1, 2).contiguous()
+    run_case('dsd', False, False, block, dtype, Z=2, H=2, M=6 * block, K=132 * block, N=64, layout=wide, seed=block + 4, dist='randn', scale=0.1)
 
 
 def test_degenerate_layouts():

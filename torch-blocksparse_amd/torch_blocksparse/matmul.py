@@ -50,12 +50,14 @@ class GroupPlan:
         self.table, self.n_groups, self.lines = table, n_groups, lines
 
     @staticmethod
-    def thin_min(layout, by_rows):
+    def thin_min(layout, by_rows, block=64):
         """Lines at least this long become chains: well above the average line, so that dense-ish layouts (whose
-        groups share every dense tile four times) keep their groups and only outliers such as global columns split."""
+        groups share every dense tile four times) keep their groups and only outliers such as global columns split.
+        The kernels for blocks 16 and 32 give a chain less than the block-64 kernel does (measured on the attention
+        mask: chains of 98 blocks of 32 cost 3 us, chains of 196 blocks of 16 save 15), so only very long lines split."""
         H, R, C = layout.shape
         mean = float((layout != 0).sum()) / max(1, H * (R if by_rows else C))
-        return max(16, int(2 * mean + 0.5))
+        return max(16 if block >= 64 else 128, int(2 * mean + 0.5))
 
     @staticmethod
     def build(layout, by_rows, device, thin_min=None):
@@ -202,7 +204,8 @@ class _sparse_matmul(torch.autograd.Function):
         _lib.check(rc, 'bsp_dxx_lut_build')
         lut = lut[:n.value]
         lut.plan = plan
-        lut.gplan = GroupPlan.build(layout, trans, dev) if block in (16, 32, 64) else None
+        lut.gplan = (GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block))
+                     if block in (16, 32, 64) else None)
         return lut, num_locks.value, width.value, None
 
     @staticmethod
