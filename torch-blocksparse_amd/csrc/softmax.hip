@@ -134,80 +134,83 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
   if (size <= 0) return;
   const table_ptr core = lut + offset;
   if constexpr (NB > 0) {
-    typedef Pack<T, GE::EV> P;
-    constexpr int NX = EXTRA ? NB : 1;
-    float fx[NB][GE::EV];
-    P px[NB], pr[NX], pa[NX];
-    int32_t bid[NB], bcol[NB];
-    float mx = -INFINITY;
+    if constexpr (NB >= 32) {
+      typedef Pack<T, GE::EV> P;
+      constexpr int NX = EXTRA ? NB : 1;
+      // Long rows are guarded GS blocks at a time: a guard per block costs a scalar compare, a mask and a branch in
+      // each of the five loops below (and the masks no longer fit the scalar registers at 32 blocks).  Inside a live
+      // group the blocks past the end of the row repeat the row's last block, so every access is valid, and get
+      // -inf added to their logits, so they contribute exp(-inf) = 0; they are not stored.
+      constexpr int GS = 4;
+      float fx[NB][GE::EV];
+      P px[NB], pr[NX], pa[NX];
+      int32_t bid[NB], bcol[NX];
+      float mx = -INFINITY;
+      const int last = size - 1;
 #pragma unroll
-    for (int b = 0; b < NB; b++) {
-      const int bb = b < size ? b : 0;                  // blocks past the end repeat the first one (never used, valid to read)
-      bid[b] = core[4 * bb + 0];
-      bcol[b] = core[4 * bb + 1];
-    }
-    // Every load of the row is issued before anything waits for one: the wavefront pays the memory latency once,
-    // not once per block.  (Loads and the arithmetic on them in one per-block branch end up serialised.)
-    const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
-    const int64_t grow = (int64_t)brow * BLOCK + u.rxm;  // row in the dense matrix
-#pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
-        px[b].load(xb + (int64_t)bid[b] * (BLOCK * BLOCK));
-        if constexpr (EXTRA) {
-          const int64_t gcol = (int64_t)bcol[b] * BLOCK + u.col;   // lane's first column in the dense matrix
-          if (a.rpe)                                               // address: softmax.py:50-55
-            pr[b].load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
-          if (a.attn) pa[b].load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);   // :67-70
-        }
+      for (int b = 0; b < NB; b++) {
+        const int bb = b < last ? b : last;               // blocks past the end repeat the last one
+        bid[b] = core[4 * bb + 0];
+        if constexpr (EXTRA) bcol[b] = core[4 * bb + 1];
       }
-    // All rows of a wavefront need the same BLOCK key-padding values per block.  The wavefront fetches them once
-    // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
-    // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
-    // the CU, and of the conversions, compared with every row reading the mask itself.
-    __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
-    float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
-    const float unit = logit_unit<T>();
-    if (a.kpm) {
-      const int lane = threadIdx.x & 63;
-      const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz;
-      constexpr int CH = NB * GE::LPR;                  // chunks of EV values
+      // keeps the table reads here, all in flight together: left alone, each one sinks to just before its block's load
 #pragma unroll
-      for (int c0 = 0; c0 < CH; c0 += 64) {
-        const int c = c0 + lane, b = c / GE::LPR;
-        int col = bcol[0];
+      for (int b = 0; b < NB; b++) asm volatile("" : "+s"(bid[b]));
+      // Every load of the row is issued before anything waits for one: the wavefront pays the memory latency once,
+      // not once per block.  (Loads and the arithmetic on them in one per-block branch end up serialised.)
+      const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
+      const int64_t grow = (int64_t)brow * BLOCK + u.rxm;  // row in the dense matrix
 #pragma unroll
-        for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
-        if (CH % 64 == 0 || c < CH) {
-          P p;
-          p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
+      for (int g = 0; g < NB; g += GS)
+        if (g < size) {
 #pragma unroll
-          for (int e4 = 0; e4 < GE::EV; e4 += 4) {       // EV is 4 or 8: whole 16-byte LDS accesses
-            f32x4 add;
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-              const float m = to_float(p.e[e4 + e]);
-              add[e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+          for (int b = g; b < g + GS; b++) {
+            px[b].load(xb + (int64_t)bid[b] * (BLOCK * BLOCK));
+            if constexpr (EXTRA) {
+              const int64_t gcol = (int64_t)bcol[b] * BLOCK + u.col;   // lane's first column in the dense matrix
+              if (a.rpe)                                               // address: softmax.py:50-55
+                pr[b].load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
+              if (a.attn) pa[b].load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);   // :67-70
             }
-            *reinterpret_cast<f32x4 *>(&kpm_s[c * GE::EV + e4]) = add;
           }
         }
-      }
-      __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
-    }
-    const float sc = a.scale * unit;
-    const bool has_kpm = a.kpm != nullptr;
+      // All rows of a wavefront need the same BLOCK key-padding values per block.  The wavefront fetches them once
+      // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
+      // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
+      // the CU, and of the conversions, compared with every row reading the mask itself.
+      __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
+      float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
+      const float unit = logit_unit<T>();
+      const bool has_kpm = a.kpm != nullptr;
+      if (has_kpm) {
+        const int lane = threadIdx.x & 63;
+        const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz;
+        constexpr int CH = NB * GE::LPR;                  // chunks of EV values
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {                                   // softmax.py:112-116, 122-124
+        for (int c0 = 0; c0 < CH; c0 += 64) {
+          const int c = c0 + lane, b = c / GE::LPR;
+          if ((CH % 64 == 0 || c < CH) && c0 / GE::LPR / GS * GS < size) {
+            const int col = a.lut[offset + 4 * (b < last ? b : last) + 1];   // the lane's block: a vector load of the table
+            P p;
+            p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
 #pragma unroll
-        for (int e4 = 0; e4 < GE::EV; e4 += 4) {
-          const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
-          const f32x4 add = has_kpm ? *reinterpret_cast<const f32x4 *>(&kpm_s[b * BLOCK + u.col + e4]) : zero4;
+            for (int e4 = 0; e4 < GE::EV; e4 += 4) {       // EV is 4 or 8: whole 16-byte LDS accesses
+              f32x4 add;
 #pragma unroll
-          for (int e = 0; e < 4; e++) fx[b][e4 + e] = fmaf(to_float(px[b].e[e4 + e]), sc, add[e]);
+              for (int e = 0; e < 4; e++) {
+                const float m = to_float(p.e[e4 + e]);
+                add[e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+                if (b >= size) add[e] = -INFINITY;
+              }
+              *reinterpret_cast<f32x4 *>(&kpm_s[c * GE::EV + e4]) = add;
+            }
+          }
         }
-        if constexpr (EXTRA) {                          // all terms of a block in one place: its raw registers die here
+        __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
+      }
+      const float sc = a.scale * unit;
+      auto extra_terms = [&](int b) {                     // all terms of a block in one place: its raw registers die here
+        if constexpr (EXTRA) {
           if (a.rpe) {                                    // :118-120
 #pragma unroll
             for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(pr[b].e[e]), unit, fx[b][e]);
@@ -223,30 +226,176 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
         // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
         // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
         if constexpr (NB >= 16 || (EXTRA && NB >= 8)) __builtin_amdgcn_sched_barrier(0);
+      };
+#pragma unroll
+      for (int g = 0; g < NB; g += GS)
+        if (g < size) {                                   // softmax.py:112-116, 122-124
+          float add[GS][GE::EV];
+          if (has_kpm) {
+#pragma unroll
+            for (int b = g; b < g + GS; b++) {
+#pragma unroll
+              for (int e4 = 0; e4 < GE::EV; e4 += 4)
+                *reinterpret_cast<f32x4 *>(&add[b - g][e4]) = *reinterpret_cast<const f32x4 *>(&kpm_s[b * BLOCK + u.col + e4]);
+            }
+          } else {
+#pragma unroll
+            for (int b = g; b < g + GS; b++) {
+#pragma unroll
+              for (int e = 0; e < GE::EV; e++) add[b - g][e] = b >= size ? -INFINITY : 0.f;
+            }
+          }
+#pragma unroll
+          for (int b = g; b < g + GS; b++) {
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(px[b].e[e]), sc, add[b - g][e]);
+            extra_terms(b);
+          }
+        }
+#pragma unroll
+      for (int g = 0; g < NB; g += GS)
+        if (g < size) {
+#pragma unroll
+          for (int b = g; b < g + GS; b++) {
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[b][e]);
+          }
+        }
+      mx = row_max<GE::LPR>(mx);                          // :130
+      float sum = 0.f;
+#pragma unroll
+      for (int g = 0; g < NB; g += GS)
+        if (g < size) {
+#pragma unroll
+          for (int b = g; b < g + GS; b++) {
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
+          }
+        }
+      sum = row_sum<GE::LPR>(sum);
+      const float inv = 1.f / sum;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
+          fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
+        }
+    } else {
+      typedef Pack<T, GE::EV> P;
+      constexpr int NX = EXTRA ? NB : 1;
+      float fx[NB][GE::EV];
+      P px[NB], pr[NX], pa[NX];
+      int32_t bid[NB], bcol[NB];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int b = 0; b < NB; b++) {
+        const int bb = b < size ? b : 0;                  // blocks past the end repeat the first one (never used, valid to read)
+        bid[b] = core[4 * bb + 0];
+        bcol[b] = core[4 * bb + 1];
       }
+      // Every load of the row is issued before anything waits for one: the wavefront pays the memory latency once,
+      // not once per block.  (Loads and the arithmetic on them in one per-block branch end up serialised.)
+      const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
+      const int64_t grow = (int64_t)brow * BLOCK + u.rxm;  // row in the dense matrix
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+          px[b].load(xb + (int64_t)bid[b] * (BLOCK * BLOCK));
+          if constexpr (EXTRA) {
+            const int64_t gcol = (int64_t)bcol[b] * BLOCK + u.col;   // lane's first column in the dense matrix
+            if (a.rpe)                                               // address: softmax.py:50-55
+              pr[b].load(reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + gcol);
+            if (a.attn) pa[b].load(reinterpret_cast<const T *>(a.attn) + grow * a.attn_sr + gcol);   // :67-70
+          }
+        }
+      // All rows of a wavefront need the same BLOCK key-padding values per block.  The wavefront fetches them once
+      // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
+      // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
+      // the CU, and of the conversions, compared with every row reading the mask itself.
+      __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
+      float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
+      const float unit = logit_unit<T>();
+      if (a.kpm) {
+        const int lane = threadIdx.x & 63;
+        const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz;
+        constexpr int CH = NB * GE::LPR;                  // chunks of EV values
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[b][e]);
+        for (int c0 = 0; c0 < CH; c0 += 64) {
+          const int c = c0 + lane, b = c / GE::LPR;
+          int col = bcol[0];
+#pragma unroll
+          for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
+          if (CH % 64 == 0 || c < CH) {
+            P p;
+            p.load(kz + (int64_t)col * BLOCK + (c % GE::LPR) * GE::EV);
+#pragma unroll
+            for (int e4 = 0; e4 < GE::EV; e4 += 4) {       // EV is 4 or 8: whole 16-byte LDS accesses
+              f32x4 add;
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                const float m = to_float(p.e[e4 + e]);
+                add[e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+              }
+              *reinterpret_cast<f32x4 *>(&kpm_s[c * GE::EV + e4]) = add;
+            }
+          }
+        }
+        __builtin_amdgcn_wave_barrier();                  // LDS operations of one wavefront complete in order
       }
-    mx = row_max<GE::LPR>(mx);                          // :130
-    float sum = 0.f;
+      const float sc = a.scale * unit;
+      const bool has_kpm = a.kpm != nullptr;
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
+      for (int b = 0; b < NB; b++)
+        if (b < size) {                                   // softmax.py:112-116, 122-124
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
-      }
-    sum = row_sum<GE::LPR>(sum);
-    const float inv = 1.f / sum;
+          for (int e4 = 0; e4 < GE::EV; e4 += 4) {
+            const f32x4 zero4 = {0.f, 0.f, 0.f, 0.f};
+            const f32x4 add = has_kpm ? *reinterpret_cast<const f32x4 *>(&kpm_s[b * BLOCK + u.col + e4]) : zero4;
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
+            for (int e = 0; e < 4; e++) fx[b][e4 + e] = fmaf(to_float(px[b].e[e4 + e]), sc, add[e]);
+          }
+          if constexpr (EXTRA) {                          // all terms of a block in one place: its raw registers die here
+            if (a.rpe) {                                    // :118-120
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
-        fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
-      }
+              for (int e = 0; e < GE::EV; e++) fx[b][e] = fmaf(to_float(pr[b].e[e]), unit, fx[b][e]);
+            }
+            if (a.attn) {                                   // :126-128, 'mul' mode :108-110
+#pragma unroll
+              for (int e = 0; e < GE::EV; e++) {
+                const float m = to_float(pa[b].e[e]);
+                fx[b][e] += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+              }
+            }
+          }
+          // In the large buckets the scheduler is kept from interleaving blocks: the raw registers of a block then die as
+          // its logits are born (a quarter fewer registers, one more wavefront per SIMD where there were two).
+          if constexpr (NB >= 16 || (EXTRA && NB >= 8)) __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) mx = fmaxf(mx, fx[b][e]);
+        }
+      mx = row_max<GE::LPR>(mx);                          // :130
+      float sum = 0.f;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) { fx[b][e] = exp_sub<T>(fx[b][e], mx); sum += fx[b][e]; }   // :131-132
+        }
+      sum = row_sum<GE::LPR>(sum);
+      const float inv = 1.f / sum;
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
+          fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
+        }
+    }
   } else {
     // Rows with more blocks than the register variant holds: two passes over x, kChunk blocks at a time with all loads
     // of a chunk in flight together.  Pass 1 keeps a running maximum and a running sum per lane (the sum is rescaled
@@ -365,35 +514,79 @@ __global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
   const T *yb = reinterpret_cast<const T *>(a.y) + (int64_t)u.z * a.y_sz + u.rxm * BLOCK + u.col;
   T *db = reinterpret_cast<T *>(a.dy) + (int64_t)u.z * a.dy_sz + u.rxm * BLOCK + u.col;
   if constexpr (NB > 0) {
-    P py[NB], pd[NB];
-    int32_t bid[NB];
-    float dot = 0.f;
-    // the table reads come first and unconditionally (one wait for all of them, not one round trip per block)
+    if constexpr (NB >= 32) {
+      P py[NB], pd[NB];
+      int32_t bid[NB];
+      float dot = 0.f;
+      // the long-row bucket is guarded four blocks at a time, like the forward kernel's: blocks past the end of the row
+      // repeat its last block (valid to read), stay out of the dot product and are not stored
+      const int last = size - 1;
 #pragma unroll
-    for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
+      for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < last ? b : last)];
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
-        const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
-        py[b].load_stream(yb + o);   // y is not read again after the backward pass
-        pd[b].load(db + o);
-      }
+      for (int b = 0; b < NB; b++) asm volatile("" : "+s"(bid[b]));   // all table reads in flight together, here
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
+      for (int g = 0; g < NB; g += 4)
+        if (g < size) {
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++) dot += to_float(py[b].e[e]) * to_float(pd[b].e[e]);   // softmax.py:187-188
-      }
-    dot = row_sum<GE::LPR>(dot);
+          for (int b = g; b < g + 4; b++) {
+            const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
+            py[b].load_stream(yb + o);   // y is not read again after the backward pass
+            pd[b].load(db + o);
+          }
+        }
 #pragma unroll
-    for (int b = 0; b < NB; b++)
-      if (b < size) {
-        P out;
+      for (int g = 0; g < NB; g += 4)
+        if (g < size) {
 #pragma unroll
-        for (int e = 0; e < GE::EV; e++)
-          out.e[e] = from_float<T>(to_float(py[b].e[e]) * (to_float(pd[b].e[e]) - dot) * a.scale);   // :189
-        out.store(db + (int64_t)bid[b] * (BLOCK * BLOCK));
-      }
+          for (int b = g; b < g + 4; b++) {
+            float part = 0.f;
+#pragma unroll
+            for (int e = 0; e < GE::EV; e++) part += to_float(py[b].e[e]) * to_float(pd[b].e[e]);   // softmax.py:187-188
+            dot += b < size ? part : 0.f;
+          }
+        }
+      dot = row_sum<GE::LPR>(dot);
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+          P out;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++)
+            out.e[e] = from_float<T>(to_float(py[b].e[e]) * (to_float(pd[b].e[e]) - dot) * a.scale);   // :189
+          out.store(db + (int64_t)bid[b] * (BLOCK * BLOCK));
+        }
+    } else {
+      P py[NB], pd[NB];
+      int32_t bid[NB];
+      float dot = 0.f;
+      // the table reads come first and unconditionally (one wait for all of them, not one round trip per block)
+#pragma unroll
+      for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+          const int64_t o = (int64_t)bid[b] * (BLOCK * BLOCK);
+          py[b].load_stream(yb + o);   // y is not read again after the backward pass
+          pd[b].load(db + o);
+        }
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++) dot += to_float(py[b].e[e]) * to_float(pd[b].e[e]);   // softmax.py:187-188
+        }
+      dot = row_sum<GE::LPR>(dot);
+#pragma unroll
+      for (int b = 0; b < NB; b++)
+        if (b < size) {
+          P out;
+#pragma unroll
+          for (int e = 0; e < GE::EV; e++)
+            out.e[e] = from_float<T>(to_float(py[b].e[e]) * (to_float(pd[b].e[e]) - dot) * a.scale);   // :189
+          out.store(db + (int64_t)bid[b] * (BLOCK * BLOCK));
+        }
+    }
   } else {
     // longer rows: two passes, kChunk blocks at a time with all loads of a chunk in flight together
     constexpr int CH = kChunk;
