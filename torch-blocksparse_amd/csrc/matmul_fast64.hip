@@ -771,8 +771,6 @@ __device__ __forceinline__ void xsd_chain_small(const XsdArgs &g, T *Ys, T *Xs, 
   }
 }
 
-constexpr int kSmallRing = 4;
-
 // LDS of k_xsd_rg_small.  groups: two dense tiles (double buffer); chains: one per wavefront.  The chain's reduction
 // buffer (16 KiB of floats) lies over the tiles (the front part is as large as the larger of the two) and is only
 // used after a barrier that ends the chain's loop; the staging rows Cs follow.
@@ -817,7 +815,11 @@ __device__ __forceinline__ void xsd_rg_small_body(const XsdArgs &g, T *smem) {
   const bool ywrite = tid < BLOCK * 8;
   const int q = lane >> 4, t = lane & 15;
   struct Stage { u32x4 y; xreg_t x[NX]; };
-  Stage ring[kSmallRing];
+  // Stages in flight (even: a stage's LDS buffer is its parity).  Measured: the untransposed products are 3-6 % faster
+  // with 2 than with 4 (fewer registers, one more workgroup per CU), the transposed ones at block 32 6-8 % slower;
+  // 6 and 8 are 5-20 % slower everywhere.
+  constexpr int RING = (!SP_TRANS || BLOCK == 16) ? 2 : 4;
+  Stage ring[RING];
   // A fixed number of loads per stage whatever the entry holds (the wait in front of a stage is then exact): an
   // absent block reads one line at the start of the sparse tensor.
   auto issue = [&](Stage &st, int e) {
@@ -846,11 +848,11 @@ __device__ __forceinline__ void xsd_rg_small_body(const XsdArgs &g, T *smem) {
   if (ne > 0) {
     const int last = ne - 1;
 #pragma unroll
-    for (int u = 0; u < kSmallRing; u++) issue(ring[u], u < last ? u : last);
-    const int steps = (ne + kSmallRing - 1) / kSmallRing * kSmallRing;
-    for (int e0i = 0; e0i < steps; e0i += kSmallRing) {
+    for (int u = 0; u < RING; u++) issue(ring[u], u < last ? u : last);
+    const int steps = (ne + RING - 1) / RING * RING;
+    for (int e0i = 0; e0i < steps; e0i += RING) {
 #pragma unroll
-      for (int u = 0; u < kSmallRing; u++) {
+      for (int u = 0; u < RING; u++) {
         const int e = e0i + u;
         const bool live = e < ne;
         const int buf = e & 1;
@@ -884,7 +886,7 @@ __device__ __forceinline__ void xsd_rg_small_body(const XsdArgs &g, T *smem) {
 #pragma unroll
             for (int j = 0; j < 4; j++) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // rows n = 16j + 4*(lane/16) + e, column m = lane % 16
         }
-        issue(st, e + kSmallRing < last ? e + kSmallRing : last);
+        issue(st, e + RING < last ? e + RING : last);
       }
     }
   }
