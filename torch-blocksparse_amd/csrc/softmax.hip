@@ -13,7 +13,14 @@
 namespace bsp {
 namespace {
 
-constexpr int kWavesPerGroup = 4;
+// Wavefronts per workgroup by bucket (NB as in the kernels below).  A workgroup starts only when every one of its
+// wavefronts has a slot, and a wavefront of the 32-block bucket takes a third of a SIMD's registers: with 4 per
+// workgroup the CUs ran 1.7 wavefronts per SIMD on average where 3 fit.  Measured (forward / backward, us):
+// 32-block bucket (block 16, rows of 28 blocks) 117 / 137 with 4, 97 / 122 with 2, 89 / 119 with 1; 16-block bucket
+// (block 32, 14 blocks) 88 / 121 with 4, 85 / 118 with 2, 86 / 120 with 1; 7 blocks at block 64: 80 / 116 with 4,
+// 80.5 / 115 with 2, 82 / 116 with 1, 86 / 126 with 8.
+template <int NB> constexpr int waves_per_group_fwd() { return NB >= 32 ? 1 : NB >= 16 ? 2 : 4; }
+template <int NB> constexpr int waves_per_group_bwd() { return NB >= 32 ? 1 : NB > 0 ? 2 : 4; }
 constexpr int kChunk = 8;           // blocks per step of the streaming variants
 
 template <typename T, int EV> struct RawVec;
@@ -81,12 +88,12 @@ template <typename T, int BLOCK> struct Unit {
   // shared_masks: the launch reads a relative position embedding or an attention mask.  Their rows are the same for
   // every head (and batch), so the units are then ordered block-row first, heads and batches inside: the wavefronts
   // that need the same mask rows run at the same time on the same XCD and all but the first find them in its L2.
-  __device__ __forceinline__ Unit(int64_t n_units, int HR, bool shared_masks = false, int H = 1, int Z = 1) {
+  __device__ __forceinline__ Unit(int64_t n_units, int HR, int wpg, bool shared_masks = false, int H = 1, int Z = 1) {
     typedef Geo<T, BLOCK> GE;
-    const int64_t n_wg = (n_units + kWavesPerGroup - 1) / kWavesPerGroup;
+    const int64_t n_wg = (n_units + wpg - 1) / wpg;
     const int64_t wg = xcd_remap(blockIdx.x, n_wg);
     // the wavefront index is uniform: as a scalar it keeps row sizes, block ids and base addresses out of the VALU
-    const int64_t u = wg * kWavesPerGroup + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t u = wg * wpg + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     ok = u < n_units;
     const int lane = threadIdx.x & 63;
     const int g = (int)(u % GE::G);
@@ -122,10 +129,11 @@ __device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<T, BLOCK>
 // position embedding or an attention mask is present (their values are kept beside x until the logits are built; the
 // plain variant does not pay registers for them).
 template <typename T, int BLOCK, int NB, bool EXTRA>
-__global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
+__global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(FwdArgs a) {
   typedef Geo<T, BLOCK> GE;
+  constexpr int WPG = waves_per_group_fwd<NB>();
   const int HR = a.H * a.R;
-  Unit<T, BLOCK> u(a.n_units, HR, EXTRA, a.H, a.Z);
+  Unit<T, BLOCK> u(a.n_units, HR, WPG, EXTRA, a.H, a.Z);
   if (!u.ok) return;
   const table_ptr lut = as_table(a.lut);
   const int size = lut[2 * u.hr + 0];                   // header (size, offset), softmax.py:30-32
@@ -178,7 +186,7 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
       // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
       // the CU, and of the conversions, compared with every row reading the mask itself.
-      __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
+      __shared__ __attribute__((aligned(16))) float kpm_lds[WPG * NB * BLOCK];
       float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
       const float unit = logit_unit<T>();
       const bool has_kpm = a.kpm != nullptr;
@@ -313,7 +321,7 @@ __global__ void __launch_bounds__(256) k_softmax_fwd(FwdArgs a) {
       // (one chunk per lane), turns them into the term that is added to the logits (softmax.py:104-106, 122-124) and
       // keeps that in its own piece of LDS: 1/RPW of the load instructions, of the bytes moved between the caches and
       // the CU, and of the conversions, compared with every row reading the mask itself.
-      __shared__ __attribute__((aligned(16))) float kpm_lds[kWavesPerGroup * NB * BLOCK];
+      __shared__ __attribute__((aligned(16))) float kpm_lds[WPG * NB * BLOCK];
       float *kpm_s = kpm_lds + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) * (NB * BLOCK);
       const float unit = logit_unit<T>();
       if (a.kpm) {
@@ -500,11 +508,11 @@ struct BwdArgs {
 };
 
 template <typename T, int BLOCK, int NB>
-__global__ void __launch_bounds__(256) k_softmax_bwd(BwdArgs a) {
+__global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(BwdArgs a) {
   typedef Geo<T, BLOCK> GE;
   typedef Pack<T, GE::EV> P;
   const int HR = a.H * a.R;
-  Unit<T, BLOCK> u(a.n_units, HR);
+  Unit<T, BLOCK> u(a.n_units, HR, waves_per_group_bwd<NB>());
   if (!u.ok) return;
   const table_ptr lut = as_table(a.lut);
   const int size = lut[2 * u.hr + 0];
@@ -634,13 +642,15 @@ template <typename T, int BLOCK> constexpr int max_nb_fwd() { return 128 / Geo<T
 template <typename T, int BLOCK> constexpr int max_nb_bwd() { return Geo<T, BLOCK>::EV * (int)sizeof(T) <= 8 ? 32 : 16; }
 
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
-  const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
-  if (a.rpe || a.attn) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
-  else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+  constexpr int WPG = waves_per_group_fwd<NB>();
+  const int64_t n_wg = (a.n_units + WPG - 1) / WPG;
+  if (a.rpe || a.attn) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
 }
 template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hipStream_t st) {
-  const int64_t n_wg = (a.n_units + kWavesPerGroup - 1) / kWavesPerGroup;
-  hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(256), 0, st, a);
+  constexpr int WPG = waves_per_group_bwd<NB>();
+  const int64_t n_wg = (a.n_units + WPG - 1) / WPG;
+  hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
 }
 
 template <typename T, int BLOCK> void launch_fwd(const FwdArgs &a, int maxlut, hipStream_t st) {
@@ -728,7 +738,7 @@ extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
   a.Z = Z; a.H = H; a.R = R; a.x_sz = x_stride_z;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
-  if (a.n_units <= 0 || a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 31) - 1) return BSP_ERR_UNSUPPORTED;
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_fwd<f16>(a, block, maxlut, as_stream(stream)); break;
@@ -751,7 +761,7 @@ extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, 
   a.y = y; a.dy = dy; a.scale = scale; a.lut = d_lut;
   a.Z = Z; a.H = H; a.R = R; a.y_sz = y_stride_z; a.dy_sz = dy_stride_z;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
-  if (a.n_units <= 0 || a.n_units / 4 + 1 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 31) - 1) return BSP_ERR_UNSUPPORTED;
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_bwd<f16>(a, block, maxlut, as_stream(stream)); break;
