@@ -547,7 +547,6 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
     const int last = ne - 1;
 #pragma unroll
     for (int u = 0; u < RING; u++) issue(ring[u], u < last ? u : last);
-    int xb = 0;
     const int steps = (ne + RING - 1) / RING * RING;
     for (int e0i = 0; e0i < steps; e0i += RING) {
 #pragma unroll
@@ -564,22 +563,26 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
         *reinterpret_cast<u32x4 *>(&Ys[buf][(ck + 32) * kLdsRow + cc]) = st.y[1];
         frag_t xf[G][2];
         if constexpr (SP_TRANS) {
+          // Two barriers per step: one tile per member, all written, then all read.  The first barrier keeps this
+          // step's tile stores behind the previous step's reads (the dense tile has two buffers for that, the four
+          // sparse tiles have not), the second one orders the stores before the reads.
+          __syncthreads();
 #pragma unroll
-          for (int m = 0; m < G; m++) {
-            const u32x4 x0 = st.x[m][0], x1 = st.x[m][1];
+          for (int m = 0; m < G; m++)
             if (bid[m] >= 0) {
-              *reinterpret_cast<u32x4 *>(&Xs[xb][ck * kLdsRow + cc]) = x0;
-              *reinterpret_cast<u32x4 *>(&Xs[xb][(ck + 32) * kLdsRow + cc]) = x1;
-              __syncthreads();
+              *reinterpret_cast<u32x4 *>(&Xs[m][ck * kLdsRow + cc]) = st.x[m][0];
+              *reinterpret_cast<u32x4 *>(&Xs[m][(ck + 32) * kLdsRow + cc]) = st.x[m][1];
+            }
+          __syncthreads();
+#pragma unroll
+          for (int m = 0; m < G; m++)
+            if (bid[m] >= 0) {
 #pragma unroll
               for (int s2 = 0; s2 < 2; s2++) {
-                const T *xrow = &Xs[xb][(32 * s2 + tr_row) * kLdsRow + 16 * wave + tr_col];
+                const T *xrow = &Xs[m][(32 * s2 + tr_row) * kLdsRow + 16 * wave + tr_col];
                 xf[m][s2] = tr_frag<T>(xrow, xrow + 4 * kLdsRow);
               }
-              xb ^= 1;
             }
-          }
-          if (!live) __syncthreads();   // a padding step still has to order its tile store against the next step
         } else {
           // The wavefront's 16 rows of each block were fetched line by line (operand layout, one row per lane, costs
           // 7 % of the launch: neighbouring lanes then never share a cache line); its own piece of LDS turns them into
