@@ -85,11 +85,14 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * bsp_dds_matmul spread over the wavefronts of a workgroup; bits 24..27 of a group's index field mark the members
  * that left it (needs fewer than 2^24 groups per head), bit 28 is the builder's hint that few groups want each
  * dense tile (the kernels then fetch those tiles with streaming loads).  Pass 0 for a plan given to bsp_sdd_matmul.
+ * order_buckets > 0 sorts the header by entries in units of 1/order_buckets of the largest group instead of exactly
+ * (equal keys head by head: better L2 reuse of the dense rows when one head's share of them is small); 0 = exact.
  * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */
 #define BSP_GROUP 4
 int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);
-int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int32_t *d_plan,
-                         int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len, void *stream);
+int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int order_buckets,
+                         int32_t *d_plan, int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len,
+                         void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Matmul launchers.  Strides are in elements; the innermost stride of every operand is 1 and rows start on

@@ -74,11 +74,14 @@ def test_group_plan(by_rows, thin_min):
     # our own work list for the row-group kernels: 4 consecutive lines per group, one entry per position where any
     # member has a block (positions ascending for row groups, descending for column groups); lines with at least
     # thin_min blocks leave their group (bit 24 + member of its index field) and become chains (index field
-    # -(line + 1)); header sorted by decreasing number of entries, groups before chains at equal length
+    # -(line + 1)); header sorted by decreasing number of entries (exactly, or in eighths of the largest group),
+    # groups before chains at equal length
     from torch_blocksparse.matmul import GroupPlan
-    for lay in (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64),
-                torch.ones(2, 7, 9, dtype=torch.int64)):
-        plan = GroupPlan.build(lay, by_rows, DEV, thin_min=thin_min)
+    import itertools
+    lays = (tb.sparse_transformer_layout(3, 18, 4, 8, True), random_layout((2, 9, 13), 0.4, 77), torch.ones(1, 4, 4, dtype=torch.int64),
+            torch.ones(2, 7, 9, dtype=torch.int64))
+    for lay, buckets in itertools.product(lays, (0, 8)):            # exact order, coarse order
+        plan = GroupPlan.build(lay, by_rows, DEV, thin_min=thin_min, order_buckets=buckets)
         t = plan.table.cpu().tolist()
         H, R, C = lay.shape
         L, B = (R, C) if by_rows else (C, R)
@@ -120,7 +123,9 @@ def test_group_plan(by_rows, thin_min):
         in_groups = sum(len(e) for code, h, e in slots if code >= 0)
         hint = 1 if 2 * in_groups <= 5 * H * B else 0
         slots = [(code | (hint << 28) if code >= 0 else code, h, e) for code, h, e in slots]
-        slots.sort(key=lambda s: -len(s[2]))                        # stable: ties stay in slot order
+        mx = max([len(e) for code, h, e in slots if code >= 0] + [0])   # the largest group (chains do not count)
+        key = (lambda n: n * buckets // (mx + 1)) if buckets else (lambda n: n)
+        slots.sort(key=lambda s: -key(len(s[2])))                   # stable: ties stay in slot order
         ng = len(slots)
         assert plan.n_groups == ng and plan.lines == L
         total = 0

@@ -385,15 +385,28 @@ __global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H,
 }
 __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *linecnt, const int32_t *cnt,
                              const int32_t *start, const int32_t *alive, int H, int R, int C, int by_rows, int thin_min,
-                             int64_t n_alive, int stream_hint, int32_t *plan) {
+                             int64_t n_alive, int stream_hint, int order_buckets, int32_t *plan) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
   const int64_t ng = (int64_t)H * NG, slots = ng + (int64_t)H * L;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (i >= slots || !alive[i]) return;
-  // position in the sorted header: more entries first, ties in slot order
+  // Position in the sorted header: more entries first, ties in slot order (head by head).  With order_buckets > 0 the
+  // key is the number of entries in units of 1/order_buckets of the largest group (chains not counted for the scale):
+  // the long groups still start first, but the many short ones behind them run head by head, so that the workgroups
+  // on the chip at one time want the dense rows of a few heads only and find them in L2.
   const int mine = cnt[i];
   int64_t pos = 0;
-  for (int64_t j = 0; j < slots; j++) pos += alive[j] && ((cnt[j] > mine) || (cnt[j] == mine && j < i));
+  if (order_buckets > 0) {
+    int mx = 0;
+    for (int64_t j = 0; j < ng; j++) mx = alive[j] && cnt[j] > mx ? cnt[j] : mx;
+    const int64_t km = (int64_t)mine * order_buckets / (mx + 1);
+    for (int64_t j = 0; j < slots; j++) {
+      const int64_t kj = (int64_t)cnt[j] * order_buckets / (mx + 1);
+      pos += alive[j] && ((kj > km) || (kj == km && j < i));
+    }
+  } else {
+    for (int64_t j = 0; j < slots; j++) pos += alive[j] && ((cnt[j] > mine) || (cnt[j] == mine && j < i));
+  }
   int32_t *hd = plan + 4 * pos;
   int32_t *e = plan + 4 * n_alive + (int64_t)(BSP_GROUP + 1) * start[i];
   const bool chain = i >= ng;
@@ -607,12 +620,13 @@ extern "C" int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_r
   return 4 * ((int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (int64_t)H * L) + (BSP_GROUP + 1) * nnz;
 }
 
-extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int32_t *d_plan,
+extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int order_buckets,
+                                    int32_t *d_plan,
                                     int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len,
                                     void *stream) {
   int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
   if (rc != BSP_OK) return rc;
-  if (!d_plan || !n_groups || !plan_len || thin_min < 0) return BSP_ERR_ARG;
+  if (!d_plan || !n_groups || !plan_len || thin_min < 0 || order_buckets < 0) return BSP_ERR_ARG;
   hipStream_t st = as_stream(stream);
   Ws o(H, R, C);
   int32_t *ws = (int32_t *)d_ws;
@@ -643,7 +657,7 @@ extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C
   // per tile), 20-30 % slower on the long-context layout with random blocks (3.9-4.5), whose tiles come back later.
   const int stream_hint = 2 * (int64_t)in_groups <= 5 * (int64_t)H * (by_rows ? C : R);
   hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, ws + o.rank, linecnt, ws + o.gcnt, ws + o.gstart,
-                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, stream_hint, d_plan);
+                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, stream_hint, order_buckets, d_plan);
   BSP_LAUNCH_CHECK();
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;

@@ -37,7 +37,7 @@ SIGNATURES = {
     'bsp_dxx_lut_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _pi64, _pi, _pi, _vp]),
     'bsp_sdd_lut_build': (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _i64, _vp, _i64, _pi, _pi, _pi64, _pi64, _pi, _vp]),
     'bsp_group_plan_cap': (_i64, [_i, _i, _i, _i64, _i]),
-    'bsp_group_plan_build': (_i, [_vp, _i, _i, _i, _i, _i, _vp, _i64, _vp, _i64, _pi, _pi64, _vp]),
+    'bsp_group_plan_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _i64, _pi, _pi64, _vp]),
     'bsp_sdd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _i, _vp, _vp,
                             _i64, _vp, _i, _i, _vp]),
     'bsp_dsd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
