@@ -76,7 +76,7 @@ def test_long_rows_streaming_variant(block, cols):
     run_case(1, 1, 2, cols, block, torch.float32, 0.95, cols + 1, scale=0.5)
 
 
-@pytest.mark.parametrize('longest', [1, 2, 3, 4, 5, 6, 7, 8, 9, 16, 17, 32, 33])
+@pytest.mark.parametrize('longest', [1, 2, 3, 4, 5, 6, 7, 8, 9, 16, 17, 18, 19, 22, 27, 30, 32, 33])
 def test_every_row_length_bucket(longest):
     # one kernel instantiation per bucket of "blocks kept in registers": the longest row decides which one runs, the
     # other rows (1 block, longest - 1 blocks, none) exercise its partially filled and empty paths
