@@ -738,7 +738,7 @@ extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
   a.Z = Z; a.H = H; a.R = R; a.x_sz = x_stride_z;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
-  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 31) - 1) return BSP_ERR_UNSUPPORTED;
+  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 26)) return BSP_ERR_UNSUPPORTED;   // one wavefront per unit: 2^32 threads per launch at most
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_fwd<f16>(a, block, maxlut, as_stream(stream)); break;
@@ -761,7 +761,7 @@ extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, 
   a.y = y; a.dy = dy; a.scale = scale; a.lut = d_lut;
   a.Z = Z; a.H = H; a.R = R; a.y_sz = y_stride_z; a.dy_sz = dy_stride_z;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
-  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 31) - 1) return BSP_ERR_UNSUPPORTED;
+  if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 26)) return BSP_ERR_UNSUPPORTED;   // one wavefront per unit: 2^32 threads per launch at most
   int rc;
   switch (dtype) {
     case BSP_F16: rc = dispatch_bwd<f16>(a, block, maxlut, as_stream(stream)); break;
