@@ -55,11 +55,15 @@ int bsp_softmax_lut_build(const int32_t *d_layout, int H, int R, int C, int32_t 
 /* dsd/dds table: replaces _sparse_matmul.make_dxx_lut + load_balance (matmul.py:221-267, 372-458).
  * d_lut receives 6*width header ints (offset, segment length, column, depth, lockid, maxid), then the
  * 2*nnz*(block/step) interleaved pointer increments and two trailing zeros -- bit-identical to the reference.
- * d_plan (int32 [2*nnz]) receives, per block in table order, (offset of the block in the dense operand's
- * reduction dimension, storage index of the block): the absolute positions the increments are differences
- * of; the matmul launchers below read them instead of re-summing the increments.
+ * d_plan (int32, at least bsp_dxx_plan_cap(...) ints; no counterpart in the reference) receives first the order
+ * in which the launchers dispatch the segments (width ints: head by head, inside a head the longest first), then,
+ * from int bsp_dxx_plan_pairs_offset(width) on, per block in table order (offset of the block in the dense
+ * operand's reduction dimension, storage index of the block): the absolute positions the increments are
+ * differences of; the matmul launchers below read them instead of re-summing the increments.
  * lut_cap >= bsp_dxx_lut_cap(...). */
 int64_t bsp_dxx_lut_cap(int H, int R, int C, int64_t nnz, int block, int step, int trans);
+int64_t bsp_dxx_plan_cap(int H, int R, int C, int64_t nnz, int trans);
+int64_t bsp_dxx_plan_pairs_offset(int width);
 int bsp_dxx_lut_build(const int32_t *d_layout, int H, int R, int C, int block, int step, int trans,
                       int32_t *d_lut, int64_t lut_cap, int32_t *d_plan, void *d_ws, int64_t ws_bytes,
                       int64_t *lut_len, int *width, int *num_locks, void *stream);

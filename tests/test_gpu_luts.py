@@ -28,6 +28,10 @@ def check_all_tables(lay, blocks=((16, 16), (16, 8), (32, 16), (64, 16), (128, 8
             # the per-block positions are what the increments are differences of
             nz = lay.nonzero() if trans else lay.transpose(1, 2).nonzero()
             assert lut.plan[:len(nz), 0].cpu().tolist() == (nz[:, 2] * block).tolist()
+            # dispatch order of the segments (ours): head by head, the longest first inside a head, ties in table order
+            hdr = elut[:6 * ewidth].reshape(ewidth, 6)
+            exp_order = sorted(range(ewidth), key=lambda i: (hdr[i, 3], -hdr[i, 1], i))
+            assert lut.planbuf[:width].cpu().tolist() == exp_order
     for block in (16, 32, 64, 128):
         luts, _, widths, packs = _sparse_matmul.make_sdd_lut(lay, block, torch.float16, DEV)
         exp = O.sdd_segment(layn, max(1, 64 // block))

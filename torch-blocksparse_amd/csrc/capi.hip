@@ -104,7 +104,7 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.sp = a; g.dn = b; g.out = c; g.Z = Z; g.NF = N;
   g.sp_sz = a_stride_z; g.dn_sz = b_stride_z; g.dn_sh = b_stride_h; g.ldd = ldb;
   g.out_sz = c_stride_z; g.out_sh = c_stride_h; g.ldo = ldc;
-  g.lut = d_lut; g.plan = d_plan; g.width = width;
+  g.lut = d_lut; g.order = d_plan; g.plan = d_plan + bsp_dxx_plan_pairs_offset(width); g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));   // step of the table: 8 for fp32, 16 otherwise (matmul.py:617)
   g.n_tiles = (N + 63) / 64;
   g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
@@ -128,7 +128,7 @@ extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, 
   g.sp = b; g.dn = a; g.out = c; g.Z = Z; g.NF = M;
   g.sp_sz = b_stride_z; g.dn_sz = a_stride_z; g.dn_sh = a_stride_h; g.ldd = lda;
   g.out_sz = c_stride_z; g.out_sh = c_stride_h; g.ldo = ldc;
-  g.lut = d_lut; g.plan = d_plan; g.width = width;
+  g.lut = d_lut; g.order = d_plan; g.plan = d_plan + bsp_dxx_plan_pairs_offset(width); g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));
   g.n_tiles = (M + 63) / 64;
   g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;

@@ -214,6 +214,21 @@ __global__ void k_dxx_plan(const int32_t *lay, const int32_t *rank, const int32_
   }
 }
 
+// order[p] = the p-th segment to dispatch: head by head (the launch order of the general kernels keeps the segments
+// of a head together for the dense operand's sake), inside a head the longest first, so that the workgroups that
+// start last are the short ones (no counterpart in the reference)
+__global__ void k_dxx_order(const int32_t *lut, int64_t width, int32_t *order) {
+  int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
+  if (i >= width) return;
+  const int len = lut[6 * i + 1], head = lut[6 * i + 3];
+  int64_t pos = 0;
+  for (int64_t j = 0; j < width; j++) {
+    const int lj = lut[6 * j + 1], hj = lut[6 * j + 3];
+    pos += hj < head || (hj == head && (lj > len || (lj == len && j < i)));
+  }
+  order[pos] = (int32_t)i;
+}
+
 __global__ void k_dxx_incs(const int32_t *plan, int64_t nnz, int block, int step, int trans, int64_t width, int32_t *lut) {
   int64_t t = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (t >= nnz) return;
@@ -516,6 +531,12 @@ extern "C" int64_t bsp_dxx_lut_cap(int H, int R, int C, int64_t nnz, int block, 
   return 6 * 2 * lines + 2 * nnz * (block / step) + 2;   // every line yields at most two segments
 }
 
+extern "C" int64_t bsp_dxx_plan_cap(int H, int R, int C, int64_t nnz, int trans) {
+  const int64_t lines = (int64_t)H * (trans ? R : C);
+  return 2 * lines + 2 + 2 * nnz;                        // at most two segments per line, then a pair per block
+}
+extern "C" int64_t bsp_dxx_plan_pairs_offset(int width) { return ((int64_t)width + 1) & ~(int64_t)1; }
+
 extern "C" int bsp_dxx_lut_build(const int32_t *d_layout, int H, int R, int C, int block, int step, int trans, int32_t *d_lut,
                                  int64_t lut_cap, int32_t *d_plan, void *d_ws, int64_t ws_bytes, int64_t *lut_len, int *width,
                                  int *num_locks, void *stream) {
@@ -555,9 +576,11 @@ extern "C" int bsp_dxx_lut_build(const int32_t *d_layout, int H, int R, int C, i
   *lut_len = need; *width = (int)w; *num_locks = 1;   // max(1, lockid.max()) with lockid == 0 everywhere (matmul.py:457)
   if (need > lut_cap) return BSP_ERR_CAPACITY;
   hipLaunchKernelGGL(k_dxx_header, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, ws + o.segstart, blkstart, H, L, block, step, d_lut);
-  hipLaunchKernelGGL(k_dxx_plan, dim3(cdiv(lines, T)), dim3(T), 0, st, d_layout, ws + o.rank, blkstart, H, R, C, block, trans, d_plan);
-  hipLaunchKernelGGL(k_dxx_incs, dim3(cdiv(nnz, T)), dim3(T), 0, st, d_plan, nnz, block, step, trans, w, d_lut);
-  hipLaunchKernelGGL(k_dxx_fix, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, ws + o.segstart, blkstart, d_plan, H, L, block, step, d_lut);
+  int32_t *pairs = d_plan + bsp_dxx_plan_pairs_offset((int)w);   // the dispatch order comes first
+  hipLaunchKernelGGL(k_dxx_plan, dim3(cdiv(lines, T)), dim3(T), 0, st, d_layout, ws + o.rank, blkstart, H, R, C, block, trans, pairs);
+  hipLaunchKernelGGL(k_dxx_incs, dim3(cdiv(nnz, T)), dim3(T), 0, st, pairs, nnz, block, step, trans, w, d_lut);
+  hipLaunchKernelGGL(k_dxx_fix, dim3(cdiv(lines, T)), dim3(T), 0, st, sizes, ws + o.headmax, ws + o.segstart, blkstart, pairs, H, L, block, step, d_lut);
+  hipLaunchKernelGGL(k_dxx_order, dim3(cdiv(w, T)), dim3(T), 0, st, d_lut, w, d_plan);
   BSP_LAUNCH_CHECK();
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;

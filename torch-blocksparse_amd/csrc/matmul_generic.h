@@ -458,6 +458,7 @@ struct XsdArgs {
   int Z, NF;                            // batch, size of the dense free dimension
   int64_t sp_sz, dn_sz, dn_sh, ldd, out_sz, out_sh, ldo;
   const int32_t *lut; const int32_t *plan; int width; int div2;   // div2 = 2 * block / step of the table
+  const int32_t *order;                 // order[p] = segment dispatched p-th (head by head, longest first inside a head), or null
   int n_tiles;                          // 64-wide tiles of the free dimension (specialised kernels)
   const int32_t *gplan; int n_pgroups; int lines;   // optional group plan, its groups, lines (block-rows or -columns) per head
 };
@@ -539,7 +540,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k
   // segment index fastest: consecutive workgroups (same XCD after the re-numbering) walk the segments of a head
   // against one slab of TN columns of the dense operand, which then stays in L2 between its uses
   const int nt = (int)((w % per_z) / g.width);
-  const int seg = (int)((w % per_z) % g.width);
+  const int seg0 = (int)((w % per_z) % g.width);
+  const int seg = g.order ? as_table(g.order)[seg0] : seg0;   // longest first only where the launch is short (see the dispatcher)
   const table_ptr hd = as_table(g.lut) + 6 * (int64_t)seg;
   const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];
   const int nblk = seglen / BLOCK;
@@ -624,11 +626,17 @@ template <typename T> int launch_sdd(const SddArgs &g, int block, int pack, bool
   return BSP_ERR_UNSUPPORTED;
 }
 
-template <typename T, int BLOCK, bool WIDE> int launch_xsd_bw(const XsdArgs &g, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+template <typename T, int BLOCK, bool WIDE> int launch_xsd_bw(const XsdArgs &g0, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
   typedef XsdShape<BLOCK, WIDE> S;
-  const int64_t n_wg = (int64_t)g.width * ((g.NF + S::TN - 1) / S::TN) * g.Z;
+  const int64_t n_wg = (int64_t)g0.width * ((g0.NF + S::TN - 1) / S::TN) * g0.Z;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  // Longest segments first only in short launches (a few workgroups per CU), where the last workgroups to start
+  // decide when the launch ends: 7 % on an 8192 x 4096 x 4096 linear layer at block 128 and 10 % density (1024
+  // workgroups).  A long launch balances by itself and reads the sparse blocks in storage order without it (1 %
+  // faster at 65536 workgroups).
+  XsdArgs g = g0;
+  if (n_wg > 16 * 256) g.order = nullptr;
   dim3 grid((unsigned)n_wg), blockdim(256);
 #define BSP_XSD_LAUNCH(ST, DK, ON)                                                                               \
   hipLaunchKernelGGL((k_xsd<T, BLOCK, WIDE, ST, DK, ON>), grid, blockdim,                                       \

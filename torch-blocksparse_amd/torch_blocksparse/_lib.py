@@ -34,6 +34,8 @@ SIGNATURES = {
     'bsp_layout_nnz': (_i, [_vp, _i, _i, _i, _vp, _i64, _pi64, _vp]),
     'bsp_softmax_lut_build': (_i, [_vp, _i, _i, _i, _vp, _i64, _vp, _i64, _pi64, _pi, _vp]),
     'bsp_dxx_lut_cap': (_i64, [_i, _i, _i, _i64, _i, _i, _i]),
+    'bsp_dxx_plan_cap': (_i64, [_i, _i, _i, _i64, _i]),
+    'bsp_dxx_plan_pairs_offset': (_i64, [_i]),
     'bsp_dxx_lut_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _pi64, _pi, _pi, _vp]),
     'bsp_sdd_lut_build': (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _i64, _vp, _i64, _pi, _pi, _pi64, _pi64, _pi, _vp]),
     'bsp_group_plan_cap': (_i64, [_i, _i, _i, _i64, _i]),

@@ -193,7 +193,8 @@ class _sparse_matmul(torch.autograd.Function):
         """-> (lut, num_locks, width, None) as the reference (matmul.py:372-458); built on `device`.
 
         The table tensor carries `.plan`: per block, in table order, (position in the dense operand's reduction
-        dimension, storage index) -- the absolute values the table's increments are differences of.
+        dimension, storage index) -- the absolute values the table's increments are differences of -- and
+        `.planbuf`, the buffer the launchers take: the order in which they dispatch the segments, then `.plan`.
         """
         lib = _lib.load()
         dev = torch.device(device)
@@ -203,18 +204,20 @@ class _sparse_matmul(torch.autograd.Function):
         nnz = int((layout != 0).sum())
         cap = lib.bsp_dxx_lut_cap(H, R, C, nnz, block, step, int(bool(trans)))
         lut = torch.empty((cap,), dtype=torch.int32, device=dev)
-        plan = torch.empty((max(nnz, 1), 2), dtype=torch.int32, device=dev)
+        planbuf = torch.empty((lib.bsp_dxx_plan_cap(H, R, C, max(nnz, 1), int(bool(trans))),), dtype=torch.int32, device=dev)
         n = ctypes.c_int64(0)
         width = ctypes.c_int(0)
         num_locks = ctypes.c_int(0)
-        rc = lib.bsp_dxx_lut_build(_lib.ptr(lay), H, R, C, block, step, int(bool(trans)), _lib.ptr(lut), cap, _lib.ptr(plan),
+        rc = lib.bsp_dxx_lut_build(_lib.ptr(lay), H, R, C, block, step, int(bool(trans)), _lib.ptr(lut), cap, _lib.ptr(planbuf),
                                    _lib.ptr(ws), ws_bytes, ctypes.byref(n), ctypes.byref(width), ctypes.byref(num_locks),
                                    _lib.stream_ptr(dev))
         if rc == _lib.ERR_EMPTY_HEAD:
             raise RuntimeError('block-sparse layout has a head without any nonzero block')
         _lib.check(rc, 'bsp_dxx_lut_build')
         lut = lut[:n.value]
-        lut.plan = plan
+        first = lib.bsp_dxx_plan_pairs_offset(width.value)
+        lut.planbuf = planbuf
+        lut.plan = planbuf[first:first + 2 * nnz].view(nnz, 2)
         lut.gplan = (GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block),
                                      order_buckets=GroupPlan.order_buckets(layout, trans, block))
                      if block in (16, 32, 64) else None)
@@ -243,7 +246,7 @@ class _sparse_matmul(torch.autograd.Function):
         timer = _Timer(bench, a.device)
         rc = _lib.load().bsp_dds_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), a.size(0), M, a.stride(0), a.stride(1), a.stride(2), b_sz, c.stride(0),
-                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
+                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
                                         *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(a.device))
         _lib.check(rc, 'bsp_dds_matmul')
         time[0] = timer.done()
@@ -265,7 +268,7 @@ class _sparse_matmul(torch.autograd.Function):
         timer = _Timer(bench, b.device)
         rc = _lib.load().bsp_dsd_matmul(_lib.DTYPES[b.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), b.size(0), N, a_sz, b.stride(0), b.stride(1), b.stride(2), c.stride(0),
-                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.plan), width,
+                                        c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
                                         *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(b.device))
         _lib.check(rc, 'bsp_dsd_matmul')
         time[0] = timer.done()
