@@ -89,6 +89,12 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * bsp_dds_matmul spread over the wavefronts of a workgroup; bits 24..27 of a group's index field mark the members
  * that left it (needs fewer than 2^24 groups per head), bit 28 is the builder's hint that few groups want each
  * dense tile (the kernels then fetch those tiles with streaming loads).  Pass 0 for a plan given to bsp_sdd_matmul.
+ * Plans over tiles (blocks of 16, for bsp_dsd_matmul / bsp_dds_matmul): the plan of the layout coarsened to 64 x 64
+ * tiles (a tile is present if any of its 4 x 4 blocks is), whose entries carry, after the BSP_GROUP+1 ints above (the
+ * ids there number the tiles), the ids of the 16 blocks of each member's tile, row by row, -1 where absent:
+ * 1 + BSP_GROUP + 16*BSP_GROUP ints per entry.  The caller assembles it from the coarse layout's plan and passes it
+ * with a NEGATIVE plan_lines (minus the tile lines per head); the launchers then run the block-64 row-group kernels
+ * and gather each tile from its blocks.
  * order_buckets > 0 sorts the header by entries in units of 1/order_buckets of the largest group instead of exactly
  * (equal keys head by head: better L2 reuse of the dense rows when one head's share of them is small); 0 = exact.
  * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */
@@ -120,7 +126,8 @@ int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a
 /* dense = sparse x dense: replaces _sparse_matmul._dsd_matmul + the DSD branch (matmul.py:507-552, 56-82).
  * C[z, h] = op(A_sparse)[h] . op(B)[z, h], written transposed when trans_c.  N = free dimension of op(B).
  * a_stride_z = 0 shares one sparse operand over the batch.  d_lut / d_plan / width from bsp_dxx_lut_build
- * with trans = !trans_a; d_gplan (optional) from bsp_group_plan_build with by_rows = !trans_a. */
+ * with trans = !trans_a; d_gplan (optional) from bsp_group_plan_build with by_rows = !trans_a; plan_lines < 0: a
+ * plan over tiles (see bsp_group_plan_build). */
 int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                    int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,

@@ -140,3 +140,38 @@ def test_group_plan(by_rows, thin_min):
             assert got == exp
             total += count
         assert len(t) == 4 * ng + 5 * total
+
+
+@pytest.mark.parametrize('by_rows', [True, False])
+def test_group_plan_over_tiles(by_rows):
+    # plan of a block-16 layout over 64 x 64 tiles: header and (position, tile ids) of the plan of the coarsened layout,
+    # every entry followed by the ids of the 4 x 4 small blocks of each member's tile (-1 where absent)
+    from torch_blocksparse.matmul import GroupPlan
+    lay = random_layout((2, 24, 36), 0.15, 99)
+    lay[:, 4:8, :] = 0
+    lay[1, :, 8] = 1
+    S, G = 4, 4
+    H, R, C = lay.shape
+    coarse = lay.view(H, R // S, S, C // S, S).amax((2, 4))
+    ref = GroupPlan.build(coarse, by_rows, DEV, thin_min=GroupPlan.thin_min(coarse, by_rows, 64),
+                          order_buckets=GroupPlan.order_buckets(coarse, by_rows, 64))
+    plan = GroupPlan.build_coarse(lay, 16, by_rows, DEV)
+    assert plan.coarse and plan.n_groups == ref.n_groups and plan.lines == ref.lines
+    ng = ref.n_groups
+    t, r = plan.table.cpu(), ref.table.cpu()
+    assert t[:4 * ng].tolist() == r[:4 * ng].tolist()
+    ent, rent = t[4 * ng:].view(-1, 1 + G + G * S * S), r[4 * ng:].view(-1, 1 + G)
+    assert ent[:, :1 + G].tolist() == rent.tolist()
+    rank = (torch.cumsum(lay.reshape(-1), 0) - 1).reshape(lay.shape)
+    fine = torch.where(lay != 0, rank, torch.full_like(rank, -1))
+    tiles = coarse.nonzero()                                         # tile id -> (head, tile row, tile column)
+    for e in range(ent.shape[0]):
+        for m in range(G):
+            tid = int(ent[e, 1 + m])
+            got = ent[e, 1 + G + m * S * S:1 + G + (m + 1) * S * S].view(S, S)
+            if tid < 0:
+                assert bool((got == -1).all())
+            else:
+                h, tr, tc = tiles[tid].tolist()
+                assert got.tolist() == fine[h, tr * S:(tr + 1) * S, tc * S:(tc + 1) * S].tolist()
+    assert GroupPlan.build_coarse(random_layout((1, 6, 9), 0.5, 1), 16, by_rows, DEV) is None   # sides must divide by 4

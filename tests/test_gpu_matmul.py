@@ -154,6 +154,29 @@ def test_small_block_row_groups(block, dtype):
     run_case('dsd', False, False, block, dtype, Z=2, H=2, M=6 * block, K=132 * block, N=64, layout=wide, seed=block + 4, dist='randn', scale=0.1)
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_block16_products_on_64x64_tiles(dtype):
+    # a block-16 layout whose sides divide by 4: dsd / dds run the block-64 row-group kernels on 64 x 64 tiles gathered
+    # from 4 x 4 small blocks (absent ones read as zeros).  Sparse tiles with 1 .. 16 blocks, an empty tile row, a full
+    # tile column and a full tile row (20 tiles: a chain), free dimension 64, 128 and 192; forward and backward reach
+    # the plain and the transposed product of dsd and, through sdd's backward, of dds (written transposed).
+    n = 80                                                           # 20 x 20 tiles
+    lay = random_layout((2, n, n), 0.12, 4242)
+    lay[:, 8:12, :] = 0                                              # tile row 2 empty
+    lay[:, :, 28:32] = (torch.rand(2, n, 4) < 0.5).long()            # tile column 7: present in every tile row ...
+    lay[:, ::4, 28] = 1
+    lay[:, 8:12, :] = 0                                              # ... but the empty one
+    lay[1, 36:40, :] = (torch.rand(n) < 0.6).long()                  # tile row 9 of head 1: every tile, partly filled
+    lay[1, 36, ::4] = 1
+    lay[0, 0:4, 0:4] = 1                                             # one full tile
+    for free in (64, 128, 192):
+        run_case('dsd', False, False, 16, dtype, Z=2, H=2, M=n * 16, K=n * 16, N=free, layout=lay, seed=free, dist='randn', scale=0.25)
+        run_case('dsd', True, False, 16, dtype, Z=2, H=2, M=n * 16, K=n * 16, N=free, layout=lay, seed=free + 1, dist='randn', scale=0.25)
+    run_case('sdd', False, True, 16, dtype, Z=2, H=2, M=n * 16, N=n * 16, K=64, layout=lay, seed=9, dist='randn', scale=0.25)
+    run_case('dds', False, False, 16, dtype, Z=2, H=2, M=64, K=n * 16, N=n * 16, layout=lay, seed=10, dist='randn', scale=0.25)
+    run_case('dds', False, True, 16, dtype, Z=2, H=2, M=128, K=n * 16, N=n * 16, layout=lay, seed=11, dist='randn', scale=0.25)
+
+
 def test_degenerate_layouts():
     # rows / columns without blocks must come out as zeros (the output buffer is uninitialised memory)
     lay = torch.zeros(2, 4, 6, dtype=torch.int64)

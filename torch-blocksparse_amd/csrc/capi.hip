@@ -95,7 +95,7 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
                               const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
                               void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || N <= 0 || width < 0) return BSP_ERR_ARG;
-  if (d_gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
+  if (d_gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   const int u = elems16(dtype);
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
@@ -119,7 +119,7 @@ extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, 
                               const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
                               void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || M <= 0 || width < 0) return BSP_ERR_ARG;
-  if (d_gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
+  if (d_gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   const int u = elems16(dtype);
   if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;

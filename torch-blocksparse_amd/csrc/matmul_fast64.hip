@@ -378,12 +378,29 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   else sdd64_rg_body<T, KD, false>(g, smem);
 }
 
+// Plans over 64 x 64 tiles of a block-16 / block-32 layout (SUBS = 64 / block per side): an entry is (position, G tile
+// flags, G x SUBS*SUBS ids of the small blocks, -1 where absent).  The kernels below then fetch a tile's rows from the
+// small blocks that hold them: `ids` = the SUBS ids of one row of small blocks (scalar), sc = the lane's column of
+// small blocks, (r_in, c_in) = the element inside the small block.  An absent block reads zeros.
+__device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0u, 0u, 0u, 0u};
+template <int SUBS> constexpr int plan_entry_ints() { return SUBS == 1 ? G + 1 : 1 + G + G * SUBS * SUBS; }
+template <typename T, int SUBS>
+__device__ __forceinline__ const T *sub_block_ptr(const T *sp, table_ptr ids, int sc, int r_in, int c_in) {
+  constexpr int BLKF = 64 / SUBS;
+  int id = ids[0];
+#pragma unroll
+  for (int k = 1; k < SUBS; k++) id = sc == k ? ids[k] : id;
+  const T *p = sp + (int64_t)id * (BLKF * BLKF) + r_in * BLKF + c_in;
+  return id >= 0 ? p : reinterpret_cast<const T *>(kZeroChunk);
+}
+
 // A chain = one output line with many blocks (the plan builder takes such lines out of their groups).  Walking its
 // entries one after the other would make this workgroup the last to finish by far, so the four wavefronts split
 // the reduction instead: wavefront w takes entries w, w+4, ... and computes all 64 rows of the line for them, in its
 // own piece of LDS and without workgroup barriers; the four partial results are added through LDS at the end.
-template <typename T, bool SP_TRANS>
+template <typename T, bool SP_TRANS, int SUBS = 1>
 __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int n0, int depth, int line, table_ptr ent, int ne) {
+  constexpr int ENT = plan_entry_ints<SUBS>(), BLKF = 64 / SUBS;
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
@@ -396,15 +413,29 @@ __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int 
   const int lr = lane >> 3, lc = (lane & 7) * 8;  // a lane's row (of 8) and 16-byte column chunk in a 64 x 64 tile
   u32x4 y[8], x[8];
   auto issue = [&](int e) {
-    const table_ptr en = ent + (G + 1) * e;
+    const table_ptr en = ent + ENT * e;
     const T *py = dn + ((int64_t)en[0] * 64 + lr) * ldd + lc;
 #pragma unroll
     for (int i = 0; i < 8; i++) y[i] = *reinterpret_cast<const u32x4 *>(py + (int64_t)i * 8 * ldd);
-    const T *blk = sp + (int64_t)en[1] * 4096;
+    if constexpr (SUBS == 1) {
+      const T *blk = sp + (int64_t)en[1] * 4096;
 #pragma unroll
-    for (int i = 0; i < 8; i++) {
-      if constexpr (SP_TRANS) x[i] = *reinterpret_cast<const u32x4 *>(blk + (i * 8 + lr) * 64 + lc);   // as stored, [k][m]
-      else x[i] = *reinterpret_cast<const u32x4 *>(blk + ((i >> 1) * 16 + (lane & 15)) * 64 + 32 * (i & 1) + (lane >> 4) * 8);   // operand layout
+      for (int i = 0; i < 8; i++) {
+        if constexpr (SP_TRANS) x[i] = *reinterpret_cast<const u32x4 *>(blk + (i * 8 + lr) * 64 + lc);   // as stored, [k][m]
+        else x[i] = *reinterpret_cast<const u32x4 *>(blk + ((i >> 1) * 16 + (lane & 15)) * 64 + 32 * (i & 1) + (lane >> 4) * 8);   // operand layout
+      }
+    } else {
+      const table_ptr ids = en + 1 + G;            // member 0 = the line
+#pragma unroll
+      for (int i = 0; i < 8; i++) {
+        // the same elements of the tile as above (whole rows of 8 lanes when transposed: 256 contiguous bytes per small
+        // block and load; else the operand layout, which walks a small block with consecutive lanes); the row of
+        // small blocks is the same for all lanes of a load
+        const int row0 = SP_TRANS ? i * 8 : (i >> 1) * 16;                       // the part of the row all lanes share
+        const int row = SP_TRANS ? row0 + lr : row0 + (lane & 15);
+        const int col = SP_TRANS ? lc : 32 * (i & 1) + (lane >> 4) * 8;
+        x[i] = *reinterpret_cast<const u32x4 *>(sub_block_ptr<T, SUBS>(sp, ids + (row0 / BLKF) * SUBS, col / BLKF, row % BLKF, col % BLKF));
+      }
     }
   };
   f32x4 acc[4][4];
@@ -484,11 +515,12 @@ __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int 
 }
 
 // dsd / dds: members = output lines (block-rows of the result), entries = positions of the reduction
-template <typename T, bool SP_TRANS, bool STREAM>
+template <typename T, bool SP_TRANS, bool STREAM, int SUBS = 1>
 __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   constexpr int TILE = 64 * kLdsRow;
+  constexpr int ENT = plan_entry_ints<SUBS>(), BLKF = 64 / SUBS;
   constexpr int RING = kGroupRing;
   T (*Ys)[TILE] = reinterpret_cast<T (*)[TILE]>(smem);
   T (*Xs)[TILE] = reinterpret_cast<T (*)[TILE]>(smem + 2 * TILE);
@@ -499,9 +531,9 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
   const int n0 = (int)(rest % g.n_tiles) * 64;
   const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
   const int e0 = hd[0], ne = hd[1], depth = hd[2], code = hd[3];
-  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)ENT * e0;
   if (code < 0) {   // a chain: the line -(code + 1) on its own
-    xsd_chain<T, SP_TRANS>(g, smem, z, n0, depth, -(code + 1), ent, ne);
+    xsd_chain<T, SP_TRANS, SUBS>(g, smem, z, n0, depth, -(code + 1), ent, ne);
     return;
   }
   const int lg = code & 0xffffff, skip = (code >> 24) & 0xf;   // members whose line is a chain are left to that chain
@@ -513,7 +545,7 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
   struct Stage { u32x4 y[2]; u32x4 x[G][2]; };
   Stage ring[RING];
   auto issue = [&](Stage &st, int e) {
-    const table_ptr en = ent + (G + 1) * e;
+    const table_ptr en = ent + ENT * e;
     const T *py = dn + ((int64_t)en[0] * 64 + ck) * ldd + cc;
     // streaming loads for the dense tiles where the plan says so (kept out of the memory-side cache: 6 us per launch
     // on the fixed attention layout)
@@ -526,10 +558,25 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
 #pragma unroll
     for (int m = 0; m < G; m++) {
       const int bid = en[1 + m];
-      const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * 4096;
       const T *p0, *p1;
-      if constexpr (SP_TRANS) { p0 = blk + ck * 64 + cc; p1 = p0 + 32 * 64; }
-      else { p0 = blk + (wave * 16 + (lane >> 3)) * 64 + (lane & 7) * 8; p1 = p0 + 8 * 64; }   // whole rows: 8 lanes per 128-byte line
+      if constexpr (SUBS == 1) {
+        const T *blk = sp + (int64_t)(bid >= 0 ? bid : 0) * 4096;
+        if constexpr (SP_TRANS) { p0 = blk + ck * 64 + cc; p1 = p0 + 32 * 64; }
+        else { p0 = blk + (wave * 16 + (lane >> 3)) * 64 + (lane & 7) * 8; p1 = p0 + 8 * 64; }   // whole rows: 8 lanes per 128-byte line
+      } else {
+        // the same elements of the tile, from the small blocks that hold them (8 rows of a small block are 256
+        // contiguous bytes at block 16); the row of small blocks is the same for a wavefront
+        const table_ptr ids = en + 1 + G + m * (SUBS * SUBS);
+        if constexpr (SP_TRANS) {
+          const int r0 = __builtin_amdgcn_readfirstlane(ck / BLKF);
+          p0 = sub_block_ptr<T, SUBS>(sp, ids + r0 * SUBS, cc / BLKF, ck % BLKF, cc % BLKF);
+          p1 = sub_block_ptr<T, SUBS>(sp, ids + (r0 + 32 / BLKF) * SUBS, cc / BLKF, ck % BLKF, cc % BLKF);
+        } else {
+          const int c = (lane & 7) * 8;
+          p0 = sub_block_ptr<T, SUBS>(sp, ids + ((wave * 16) / BLKF) * SUBS, c / BLKF, (wave * 16) % BLKF + (lane >> 3), c % BLKF);
+          p1 = p0 + (p0 == reinterpret_cast<const T *>(kZeroChunk) ? 0 : 8 * BLKF);
+        }
+      }
       if (bid < 0) { p0 = sp; p1 = sp; }
       st.x[m][0] = *reinterpret_cast<const u32x4 *>(p0);
       st.x[m][1] = *reinterpret_cast<const u32x4 *>(p1);
@@ -555,7 +602,7 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
         const bool live = e < ne;
         const int buf = e & 1;
         Stage &st = ring[u];
-        const table_ptr en = ent + (G + 1) * (live ? e : last);
+        const table_ptr en = ent + ENT * (live ? e : last);
         int bid[G];
 #pragma unroll
         for (int m = 0; m < G; m++) bid[m] = live ? en[1 + m] : -1;
@@ -635,14 +682,14 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
 }
 
 // (two copies of the body, chosen by the plan's streaming hint: see k_sdd64_rg)
-template <typename T, bool SP_TRANS>
+template <typename T, bool SP_TRANS, int SUBS = 1>
 __global__ void __launch_bounds__(256) k_xsd64_rg(XsdArgs g) {
   // groups: two dense tiles + two sparse tiles when read transposed, else a 16-row slice of each member's block per
   // wavefront (4 x 4 quarter tiles); chains: one dense and one sparse tile per wavefront
   __shared__ __attribute__((aligned(16))) T smem[(SP_TRANS ? 8 : 6) * 64 * kLdsRow];
   const int code = as_table(g.gplan)[4 * ((int64_t)(blockIdx.x / g.Z) / g.n_tiles) + 3];
-  if (code >= 0 && ((code >> 28) & 1)) xsd64_rg_body<T, SP_TRANS, true>(g, smem);
-  else xsd64_rg_body<T, SP_TRANS, false>(g, smem);
+  if (code >= 0 && ((code >> 28) & 1)) xsd64_rg_body<T, SP_TRANS, true, SUBS>(g, smem);
+  else xsd64_rg_body<T, SP_TRANS, false, SUBS>(g, smem);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -798,7 +845,7 @@ __device__ __forceinline__ void xsd_rg_small_body(const XsdArgs &g, T *smem) {
   constexpr int NX = XB / 16 > 0 ? XB / 16 : 1;  // loads per lane: one of 8 bytes, or two of 16
   typedef typename std::conditional<XB == 8, u32x2, u32x4>::type xreg_t;
   typedef SmallXsdLds<T, BLOCK, SP_TRANS> LD;
-  constexpr int LDX = LD::LDX, YT = LD::YT, XT = LD::XT, CT = LD::CT, FRONT = LD::FRONT;
+  constexpr int LDX = LD::LDX, YT = LD::YT, XT = LD::XT, CT = LD::CT;
   T (*Ys)[YT] = reinterpret_cast<T (*)[YT]>(smem);
   T (*Xs)[XT > 0 ? XT : 8] = reinterpret_cast<T (*)[XT > 0 ? XT : 8]>(smem + 4 * YT);
   T (*Cs)[CT] = reinterpret_cast<T (*)[CT]>(smem);
@@ -1117,7 +1164,24 @@ int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool
   int rc = dtype == BSP_F16 ? sdd_fast_t<f16>(g, st) : sdd_fast_t<bf16>(g, st);
   return rc == BSP_OK ? 1 : rc;
 }
-int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+// a plan over 64 x 64 tiles of a block-16 / block-32 layout (negative line count): the block-64 row-group kernel,
+// gathering each tile from its small blocks
+template <typename T, int SUBS> int xsd_coarse_t(const XsdArgs &g, bool sp_trans, hipStream_t st) {
+  const int64_t n = (int64_t)g.n_pgroups * g.n_tiles * g.Z;
+  if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  if (sp_trans) hipLaunchKernelGGL((k_xsd64_rg<T, true, SUBS>), dim3((unsigned)n), dim3(256), 0, st, g);
+  else hipLaunchKernelGGL((k_xsd64_rg<T, false, SUBS>), dim3((unsigned)n), dim3(256), 0, st, g);
+  return BSP_OK;
+}
+int xsd_fast64(int dtype, const XsdArgs &g0, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
+  XsdArgs g = g0;
+  if (g.gplan && g.lines < 0) {
+    const bool ok = dtype != BSP_F32 && block == 16 && g.n_pgroups > 0 && !dn_kc && out_nc && g.NF % 64 == 0;
+    if (!ok) return 0;                              // such a plan serves nothing else: the general kernels take the launch
+    g.lines = -g.lines;
+    const int rc = dtype == BSP_F16 ? xsd_coarse_t<f16, 4>(g, sp_trans, st) : xsd_coarse_t<bf16, 4>(g, sp_trans, st);
+    return rc == BSP_OK ? 1 : rc;
+  }
   if (dtype != BSP_F32 && small_ok_xsd(g, block, dn_kc, out_nc)) {
     int rc = dtype == BSP_F16 ? xsd_small_t<f16>(g, block, sp_trans, st) : xsd_small_t<bf16>(g, block, sp_trans, st);
     return rc == BSP_OK ? 1 : rc;

@@ -89,10 +89,40 @@ class GroupPlan:
         return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C)
 
     @staticmethod
+    def build_coarse(layout, block, by_rows, device):
+        """Plan of a block-16 / block-32 layout over 64 x 64 tiles, for the dsd / dds launchers: the groups, chains and
+        order of `build` on the layout coarsened to 64 (a tile is present if any of its S x S blocks is, S = 64 / block),
+        with entries that carry the ids of the small blocks: (position, 4 tile flags, 4 x S*S block ids, -1 where
+        absent).  The launchers are told by a negative line count.  None if the layout does not divide into tiles."""
+        S = 64 // block
+        H, R, C = layout.shape
+        if R % S or C % S:
+            return None
+        dev = torch.device(device)
+        lay = (layout != 0)
+        coarse = lay.reshape(H, R // S, S, C // S, S).any(4).any(2).to(torch.int64)
+        plan = GroupPlan.build(coarse, by_rows, dev, thin_min=GroupPlan.thin_min(coarse, by_rows, 64),
+                               order_buckets=GroupPlan.order_buckets(coarse, by_rows, 64))
+        ng, G = plan.n_groups, 4
+        table = plan.table
+        header, entries = table[:4 * ng], table[4 * ng:].view(-1, G + 1)
+        # ids of the small blocks of every present tile, tiles in nonzero() order like the plan's tile ids
+        layd = lay.to(dev)
+        fine = torch.where(layd, torch.cumsum(layd.reshape(-1).to(torch.int64), 0).reshape(layd.shape) - 1,
+                           torch.full((), -1, dtype=torch.int64, device=dev)).to(torch.int32)
+        tiles = fine.reshape(H, R // S, S, C // S, S).permute(0, 1, 3, 2, 4)[coarse.to(dev).bool()].reshape(-1, S * S)
+        ids = entries[:, 1:].to(torch.int64)                                    # [entries, G] tile ids or -1
+        sub = torch.where((ids >= 0).unsqueeze(2), tiles[ids.clamp(min=0)], torch.full((), -1, dtype=torch.int32, device=dev))
+        wide = torch.cat([entries, sub.reshape(entries.shape[0], G * S * S)], 1).to(torch.int32)
+        out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines)
+        out.coarse = True
+        return out
+
+    @staticmethod
     def args(plan):
         if plan is None:
             return ctypes.c_void_p(0), 0, 0
-        return _lib.ptr(plan.table), plan.n_groups, plan.lines
+        return _lib.ptr(plan.table), plan.n_groups, (-plan.lines if getattr(plan, 'coarse', False) else plan.lines)
 
 
 class SddTables(list):
@@ -218,9 +248,10 @@ class _sparse_matmul(torch.autograd.Function):
         first = lib.bsp_dxx_plan_pairs_offset(width.value)
         lut.planbuf = planbuf
         lut.plan = planbuf[first:first + 2 * nnz].view(nnz, 2)
-        lut.gplan = (GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block),
-                                     order_buckets=GroupPlan.order_buckets(layout, trans, block))
-                     if block in (16, 32, 64) else None)
+        lut.gplan = GroupPlan.build_coarse(layout, block, trans, dev) if block == 16 else None
+        if lut.gplan is None and block in (16, 32, 64):
+            lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block),
+                                        order_buckets=GroupPlan.order_buckets(layout, trans, block))
         return lut, num_locks.value, width.value, None
 
     @staticmethod
