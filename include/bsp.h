@@ -89,12 +89,12 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * bsp_dds_matmul spread over the wavefronts of a workgroup; bits 24..27 of a group's index field mark the members
  * that left it (needs fewer than 2^24 groups per head), bit 28 is the builder's hint that few groups want each
  * dense tile (the kernels then fetch those tiles with streaming loads).  Pass 0 for a plan given to bsp_sdd_matmul.
- * Plans over tiles (blocks of 16, for bsp_dsd_matmul / bsp_dds_matmul): the plan of the layout coarsened to 64 x 64
+ * Plans over tiles (blocks of 16, for all three launchers): the plan of the layout coarsened to 64 x 64
  * tiles (a tile is present if any of its 4 x 4 blocks is), whose entries carry, after the BSP_GROUP+1 ints above (the
  * ids there number the tiles), the ids of the 16 blocks of each member's tile, row by row, -1 where absent:
  * 1 + BSP_GROUP + 16*BSP_GROUP ints per entry.  The caller assembles it from the coarse layout's plan and passes it
  * with a NEGATIVE plan_lines (minus the tile lines per head); the launchers then run the block-64 row-group kernels
- * and gather each tile from its blocks.
+ * and gather each tile from its blocks (bsp_sdd_matmul: scatter each result tile to the blocks present).
  * order_buckets > 0 sorts the header by entries in units of 1/order_buckets of the largest group instead of exactly
  * (equal keys head by head: better L2 reuse of the dense rows when one head's share of them is small); 0 = exact.
  * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */

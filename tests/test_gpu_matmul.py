@@ -156,8 +156,8 @@ def test_small_block_row_groups(block, dtype):
 
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 def test_block16_products_on_64x64_tiles(dtype):
-    # a block-16 layout whose sides divide by 4: dsd / dds run the block-64 row-group kernels on 64 x 64 tiles gathered
-    # from 4 x 4 small blocks (absent ones read as zeros).  Sparse tiles with 1 .. 16 blocks, an empty tile row, a full
+    # a block-16 layout whose sides divide by 4: sdd / dsd / dds run the block-64 row-group kernels on 64 x 64 tiles
+    # gathered from (scattered to) 4 x 4 small blocks (absent ones read as zeros, are not written).  Sparse tiles with 1 .. 16 blocks, an empty tile row, a full
     # tile column and a full tile row (20 tiles: a chain), free dimension 64, 128 and 192; forward and backward reach
     # the plain and the transposed product of dsd and, through sdd's backward, of dds (written transposed).
     n = 80                                                           # 20 x 20 tiles
@@ -172,7 +172,9 @@ def test_block16_products_on_64x64_tiles(dtype):
     for free in (64, 128, 192):
         run_case('dsd', False, False, 16, dtype, Z=2, H=2, M=n * 16, K=n * 16, N=free, layout=lay, seed=free, dist='randn', scale=0.25)
         run_case('dsd', True, False, 16, dtype, Z=2, H=2, M=n * 16, K=n * 16, N=free, layout=lay, seed=free + 1, dist='randn', scale=0.25)
+    # sdd scatters its 64 x 64 result tiles to the blocks present (reduction 64 and 128)
     run_case('sdd', False, True, 16, dtype, Z=2, H=2, M=n * 16, N=n * 16, K=64, layout=lay, seed=9, dist='randn', scale=0.25)
+    run_case('sdd', False, True, 16, dtype, Z=2, H=2, M=n * 16, N=n * 16, K=128, layout=lay, seed=12, dist='randn', scale=0.25)
     run_case('dds', False, False, 16, dtype, Z=2, H=2, M=64, K=n * 16, N=n * 16, layout=lay, seed=10, dist='randn', scale=0.25)
     run_case('dds', False, True, 16, dtype, Z=2, H=2, M=128, K=n * 16, N=n * 16, layout=lay, seed=11, dist='randn', scale=0.25)
 

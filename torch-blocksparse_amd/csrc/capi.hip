@@ -55,7 +55,7 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.b_sz = b_stride_z; g.b_sh = b_stride_h; g.ldb = ldb; g.c_sz = c_stride_z;
   g.lut = d_lut; g.valid = d_valid; g.n_groups = n_groups;
   g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
-  if (g.gplan && (n_plan_groups <= 0 || plan_lines <= 0)) return BSP_ERR_ARG;
+  if (g.gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);

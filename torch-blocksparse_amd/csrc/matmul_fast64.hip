@@ -257,6 +257,22 @@ __global__ void __launch_bounds__(256) k_xsd64(XsdArgs g) {
 constexpr int G = BSP_GROUP;
 constexpr int kGroupRing = 2;   // register stages of k_xsd64_rg (three were measured 5-8 % slower)
 
+// Plans over 64 x 64 tiles of a block-16 / block-32 layout (SUBS = 64 / block per side): an entry is (position, G tile
+// flags, G x SUBS*SUBS ids of the small blocks, -1 where absent).  The kernels below then fetch a tile's rows from the
+// small blocks that hold them: `ids` = the SUBS ids of one row of small blocks (scalar), sc = the lane's column of
+// small blocks, (r_in, c_in) = the element inside the small block.  An absent block reads zeros.
+__device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0u, 0u, 0u, 0u};
+template <int SUBS> constexpr int plan_entry_ints() { return SUBS == 1 ? G + 1 : 1 + G + G * SUBS * SUBS; }
+template <typename T, int SUBS>
+__device__ __forceinline__ const T *sub_block_ptr(const T *sp, table_ptr ids, int sc, int r_in, int c_in) {
+  constexpr int BLKF = 64 / SUBS;
+  int id = ids[0];
+#pragma unroll
+  for (int k = 1; k < SUBS; k++) id = sc == k ? ids[k] : id;
+  const T *p = sp + (int64_t)id * (BLKF * BLKF) + r_in * BLKF + c_in;
+  return id >= 0 ? p : reinterpret_cast<const T *>(kZeroChunk);
+}
+
 // STREAM: the slice belongs to a dense result, which nothing in the sparse chain reads again: written with streaming
 // stores it does not displace the sparse tensors that the next launches re-read from the memory-side cache
 // (measured on the attention step: 8-9 us less for two of the four dsd/dds launches, 1-2 us for the others; the same
@@ -282,12 +298,38 @@ template <typename T, bool STREAM = false> __device__ __forceinline__ void store
   __builtin_amdgcn_wave_barrier();
 }
 
+// The same slice scattered to the four small blocks (16 x 16) of one row of a tile: ids = their block ids (-1: absent,
+// nothing stored); a store instruction writes 8 rows = 256 contiguous bytes of each.
+template <typename T> __device__ __forceinline__ void store_slice_sub16(T *cs, T *c, table_ptr ids, const f32x4 (&acc)[4], int lane) {
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk.e[e] = from_float<T>(acc[j][e]);
+    *reinterpret_cast<u32x2 *>(cs + (lane & 15) * kLdsRow + 16 * j + 4 * (lane >> 4)) = pk.raw;
+  }
+  __builtin_amdgcn_wave_barrier();
+  const int sc = (lane & 7) >> 1;
+  int id = ids[0];
+#pragma unroll
+  for (int k = 1; k < 4; k++) id = sc == k ? ids[k] : id;
+  const T *rs = cs + (lane >> 3) * kLdsRow + (lane & 7) * 8;
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(rs + i * 8 * kLdsRow);
+    if (id >= 0) *reinterpret_cast<u32x4 *>(c + (int64_t)id * 256 + ((lane >> 3) + 8 * i) * 16 + (lane & 1) * 8) = v;
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
 // sdd, K = KD (64 or 128): members = block-rows of A (their 16-row slices stay in registers), entries = block-columns
 // (B tiles of 64 rows x KD)
-template <typename T, int KD, bool STREAM>
+template <typename T, int KD, bool STREAM, int SUBS = 1>
 __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
+  constexpr int ENT = plan_entry_ints<SUBS>();   // SUBS = 4: a plan over 64 x 64 tiles of a block-16 layout, the result tile is scattered
+  static_assert(SUBS == 1 || SUBS == 4, "tiles of whole blocks or of 4 x 4 blocks of 16");
   constexpr int NK = KD / 32;                    // MFMA steps along the reduction
   constexpr int LDK = KD + 8;                    // LDS row of a B tile
   constexpr int TILE = 64 * LDK;
@@ -298,7 +340,7 @@ __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
   const int z = blockIdx.x % g.Z;
   const table_ptr hd = as_table(g.gplan) + 4 * (int64_t)(blockIdx.x / g.Z);
   const int e0 = hd[0], ne = hd[1], h = hd[2], lg = hd[3] & 0xffffff;
-  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * e0;
+  const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)ENT * e0;
   const int r = lane & 15, kq = (lane >> 4) * 8;
   const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
   const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
@@ -316,7 +358,7 @@ __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
   struct Stage { u32x4 y[NL]; };
   Stage ring[kRing];
   auto issue = [&](Stage &st, int e) {
-    const T *py = pb + (int64_t)ent[(G + 1) * e] * 64 * g.ldb;
+    const T *py = pb + (int64_t)ent[ENT * e] * 64 * g.ldb;
 #pragma unroll
     for (int i = 0; i < NL; i++) {
       const int c = tid + 256 * i;
@@ -350,7 +392,7 @@ __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
           for (int s2 = 0; s2 < NK; s2++) yf[j][s2] = *reinterpret_cast<const frag_t *>(&Ks[buf][(16 * j + r) * LDK + 32 * s2 + kq]);
 #pragma unroll
         for (int m = 0; m < G; m++) {
-          const int bid = ent[(G + 1) * e + 1 + m];
+          const int bid = ent[ENT * e + 1 + m];
           if (bid >= 0) {
             f32x4 acc[4];
 #pragma unroll
@@ -359,7 +401,8 @@ __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
 #pragma unroll
               for (int s2 = 0; s2 < NK; s2++) acc[j] = M::run(yf[j][s2], xq[m][s2], acc[j]);   // rows n = 16j + 4*(lane/16) + e, column m-row = lane%16
             }
-            store_slice<T>(Cs[wave], pc + (int64_t)bid * 4096 + wave * 1024, 64, acc, lane);
+            if constexpr (SUBS == 1) store_slice<T>(Cs[wave], pc + (int64_t)bid * 4096 + wave * 1024, 64, acc, lane);
+            else store_slice_sub16<T>(Cs[wave], pc, ent + ENT * e + 1 + G + m * 16 + wave * 4, acc, lane);
           }
         }
       }
@@ -370,28 +413,12 @@ __device__ __forceinline__ void sdd64_rg_body(const SddArgs &g, T *smem) {
 // The streaming hint is a property of the whole plan (bit 28 of every group's index field), so all workgroups of a
 // launch take the same side of this branch.  Two copies of the body rather than a condition at the load: the
 // compiler merges two loads of one address that differ only in the hint, and drops the hint.
-template <typename T, int KD>
+template <typename T, int KD, int SUBS = 1>
 __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
   __shared__ __attribute__((aligned(16))) T smem[2 * 64 * (KD + 8) + 4 * 16 * kLdsRow];
   const int code = as_table(g.gplan)[4 * (int64_t)(blockIdx.x / g.Z) + 3];
-  if ((code >> 28) & 1) sdd64_rg_body<T, KD, true>(g, smem);
-  else sdd64_rg_body<T, KD, false>(g, smem);
-}
-
-// Plans over 64 x 64 tiles of a block-16 / block-32 layout (SUBS = 64 / block per side): an entry is (position, G tile
-// flags, G x SUBS*SUBS ids of the small blocks, -1 where absent).  The kernels below then fetch a tile's rows from the
-// small blocks that hold them: `ids` = the SUBS ids of one row of small blocks (scalar), sc = the lane's column of
-// small blocks, (r_in, c_in) = the element inside the small block.  An absent block reads zeros.
-__device__ __attribute__((aligned(16))) const uint32_t kZeroChunk[4] = {0u, 0u, 0u, 0u};
-template <int SUBS> constexpr int plan_entry_ints() { return SUBS == 1 ? G + 1 : 1 + G + G * SUBS * SUBS; }
-template <typename T, int SUBS>
-__device__ __forceinline__ const T *sub_block_ptr(const T *sp, table_ptr ids, int sc, int r_in, int c_in) {
-  constexpr int BLKF = 64 / SUBS;
-  int id = ids[0];
-#pragma unroll
-  for (int k = 1; k < SUBS; k++) id = sc == k ? ids[k] : id;
-  const T *p = sp + (int64_t)id * (BLKF * BLKF) + r_in * BLKF + c_in;
-  return id >= 0 ? p : reinterpret_cast<const T *>(kZeroChunk);
+  if ((code >> 28) & 1) sdd64_rg_body<T, KD, true, SUBS>(g, smem);
+  else sdd64_rg_body<T, KD, false, SUBS>(g, smem);
 }
 
 // A chain = one output line with many blocks (the plan builder takes such lines out of their groups).  Walking its
@@ -1155,7 +1182,26 @@ template <typename T> int xsd_fast_t(const XsdArgs &g, bool sp_trans, hipStream_
 
 // Returns 1 if a specialised kernel took the launch (2: through the group plan, which covers every pack level of the
 // layout), 0 if the caller should use the general kernel, < 0 on error.
-int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st) {
+int sdd_fast64(int dtype, const SddArgs &g0, int block, int pack, bool a_kc, bool b_kc, hipStream_t st) {
+  SddArgs g = g0;
+  if (g.gplan && g.lines < 0) {
+    // a plan over 64 x 64 tiles of a block-16 layout: the block-64 row-group kernel, scattering each result tile to
+    // its small blocks; covers the whole layout
+    const bool ok = dtype != BSP_F32 && block == 16 && g.n_pgroups > 0 && a_kc && b_kc && (g.K == 64 || g.K == 128);
+    if (!ok) return 0;
+    g.lines = -g.lines;
+    const int64_t n = (int64_t)g.n_pgroups * g.Z;
+    if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+    const dim3 grid((unsigned)n), wg(256);
+    if (dtype == BSP_F16) {
+      if (g.K == 64) hipLaunchKernelGGL((k_sdd64_rg<f16, 64, 4>), grid, wg, 0, st, g);
+      else hipLaunchKernelGGL((k_sdd64_rg<f16, 128, 4>), grid, wg, 0, st, g);
+    } else {
+      if (g.K == 64) hipLaunchKernelGGL((k_sdd64_rg<bf16, 64, 4>), grid, wg, 0, st, g);
+      else hipLaunchKernelGGL((k_sdd64_rg<bf16, 128, 4>), grid, wg, 0, st, g);
+    }
+    return 2;
+  }
   if (dtype != BSP_F32 && small_ok_sdd(g, block, a_kc, b_kc)) {
     int rc = dtype == BSP_F16 ? sdd_small_t<f16>(g, block, st) : sdd_small_t<bf16>(g, block, st);
     return rc == BSP_OK ? 2 : rc;

@@ -89,11 +89,12 @@ class GroupPlan:
         return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C)
 
     @staticmethod
-    def build_coarse(layout, block, by_rows, device):
-        """Plan of a block-16 / block-32 layout over 64 x 64 tiles, for the dsd / dds launchers: the groups, chains and
-        order of `build` on the layout coarsened to 64 (a tile is present if any of its S x S blocks is, S = 64 / block),
-        with entries that carry the ids of the small blocks: (position, 4 tile flags, 4 x S*S block ids, -1 where
-        absent).  The launchers are told by a negative line count.  None if the layout does not divide into tiles."""
+    def build_coarse(layout, block, by_rows, device, for_sdd=False):
+        """Plan of a block-16 layout over 64 x 64 tiles: the groups, chains and order of `build` on the layout coarsened
+        to 64 (a tile is present if any of its S x S blocks is, S = 64 / block), with entries that carry the ids of the
+        small blocks: (position, 4 tile ids, 4 x S*S block ids, -1 where absent).  The launchers are told by a
+        negative line count.  for_sdd: no chains, exact order (the plan bsp_sdd_matmul takes).  None if the layout
+        does not divide into tiles."""
         S = 64 // block
         H, R, C = layout.shape
         if R % S or C % S:
@@ -101,8 +102,8 @@ class GroupPlan:
         dev = torch.device(device)
         lay = (layout != 0)
         coarse = lay.reshape(H, R // S, S, C // S, S).any(4).any(2).to(torch.int64)
-        plan = GroupPlan.build(coarse, by_rows, dev, thin_min=GroupPlan.thin_min(coarse, by_rows, 64),
-                               order_buckets=GroupPlan.order_buckets(coarse, by_rows, 64))
+        plan = GroupPlan.build(coarse, by_rows, dev, thin_min=0 if for_sdd else GroupPlan.thin_min(coarse, by_rows, 64),
+                               order_buckets=0 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64))
         ng, G = plan.n_groups, 4
         table = plan.table
         header, entries = table[:4 * ng], table[4 * ng:].view(-1, G + 1)
@@ -172,7 +173,9 @@ class _sparse_matmul(torch.autograd.Function):
         luts, widths, out_packs = SddTables(), [], []
         luts.nnz = nnz
         if block in (16, 32, 64):
-            luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0)
+            luts.gplan = GroupPlan.build_coarse(layout, block, True, dev, for_sdd=True) if block == 16 else None
+            if luts.gplan is None:
+                luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0)
         done = 0
         for k in range(n_levels.value):
             p, r = int(packs[k]), int(rows[k])
