@@ -93,8 +93,10 @@ class GroupPlan:
         """Plan of a block-16 layout over 64 x 64 tiles: the groups, chains and order of `build` on the layout coarsened
         to 64 (a tile is present if any of its S x S blocks is, S = 64 / block), with entries that carry the ids of the
         small blocks: (position, 4 tile ids, 4 x S*S block ids, -1 where absent).  The launchers are told by a
-        negative line count.  for_sdd: no chains, exact order (the plan bsp_sdd_matmul takes).  None if the layout
-        does not divide into tiles."""
+        negative line count.  for_sdd: the plan bsp_sdd_matmul takes: no chains, and the longer half of the groups before
+        the shorter half, head by head in each (measured on the attention mask: the sdd and the softmax that reads
+        its result 2-3 us faster each than with the exact longest-first order).  None if the layout does not divide
+        into tiles."""
         S = 64 // block
         H, R, C = layout.shape
         if R % S or C % S:
@@ -103,7 +105,7 @@ class GroupPlan:
         lay = (layout != 0)
         coarse = lay.reshape(H, R // S, S, C // S, S).any(4).any(2).to(torch.int64)
         plan = GroupPlan.build(coarse, by_rows, dev, thin_min=0 if for_sdd else GroupPlan.thin_min(coarse, by_rows, 64),
-                               order_buckets=0 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64))
+                               order_buckets=2 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64))
         ng, G = plan.n_groups, 4
         table = plan.table
         header, entries = table[:4 * ng], table[4 * ng:].view(-1, G + 1)
