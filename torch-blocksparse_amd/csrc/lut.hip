@@ -221,10 +221,13 @@ __global__ void k_dxx_order(const int32_t *lut, int64_t width, int32_t *order) {
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
   if (i >= width) return;
   const int len = lut[6 * i + 1], head = lut[6 * i + 3];
-  int64_t pos = 0;
-  for (int64_t j = 0; j < width; j++) {
-    const int lj = lut[6 * j + 1], hj = lut[6 * j + 3];
-    pos += hj < head || (hj == head && (lj > len || (lj == len && j < i)));
+  int64_t lo = i, hi = i + 1;                      // the segments of a head are neighbours in the table
+  while (lo > 0 && lut[6 * (lo - 1) + 3] == head) lo--;
+  while (hi < width && lut[6 * hi + 3] == head) hi++;
+  int64_t pos = lo;
+  for (int64_t j = lo; j < hi; j++) {
+    const int lj = lut[6 * j + 1];
+    pos += lj > len || (lj == len && j < i);
   }
   order[pos] = (int32_t)i;
 }
