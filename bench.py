@@ -8,33 +8,66 @@ One step = sdd(q, k^T) -> softmax -> dsd(p, v), then the backward pass (softmax 
 Prints one JSON line.  `value` is the effective matmul throughput of the whole step: the FLOPs of the six
 block-sparse products over their nonzero blocks (2*Z*64*nnz*64^2 each, the reference's formula,
 tests/test_matmul.py:82-84) divided by the wall time of the full step, softmax included.  `kernels` lists every
-launch of the step with its own HIP-event time, effective TFLOP/s or GB/s and roofline fractions; `roofline`
-repeats the entry of the launch that takes the largest share of the step.  `cpu_baseline` is the same chain
-computed by the fp32 dense-masked oracle on the host cores, on a slice of the batch.
+launch of the step with its own HIP-event time, effective TFLOP/s or GB/s and roofline fractions; `roofline` is the
+kernel that takes the largest share of the step (all its launches together).  `other_configs` holds the per-launch
+figures of the other benchmark configurations (block-32 dsd/dds round trip, long-context BigBird attention,
+block-128 sparse linear layer).  `cpu_baseline` is the same chain computed by the fp32 dense-masked oracle on the host
+cores, on a slice of the batch.
+
+Other modes:  --config N        one of the other configurations alone (one JSON line, not the headline)
+              --calibrate       what this box streams: read / write / copy / in-place / 1r:2w probes at 4 GiB and at the
+                                step's 268 MB footprint, and the step's launches with the caches flushed before each
+              --record-traffic  turn two rocprofv3 --pmc runs of this script (FETCH_SIZE, WRITE_SIZE) into the file that
+                                `traffic` in the JSON line is read from
 """
 import argparse
+import ctypes
+import glob
+import hashlib
 import json
 import os
 import sys
 import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
-for p in (ROOT, os.path.join(ROOT, 'torch-blocksparse_amd')):
+PKG = os.path.join(ROOT, 'torch-blocksparse_amd')
+for p in (ROOT, PKG):
     if p not in sys.path:
         sys.path.insert(0, p)
 
 HBM_PEAK_GBS = 8000.0       # MI355X HBM3E
 MFMA_PEAK_TFLOPS = 2500.0   # dense fp16 MFMA
+FP32_PEAK_TFLOPS = 157.3    # fp32 matrix
 
-# HBM bytes per launch at batch 8, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per dispatch), each scaled by what
-# the same counter reads for the calibration copy of known size (profiles/attention_seq4096_fp16_blk64.txt).  None = not
-# measured for this build of the kernel.
-TRAFFIC_BYTES = {
-    'sdd_fwd  q.k^T': 143501257 + 268435475, 'sdd_bwd  do.v^T': 143501257 + 268435475,
-    'dsd_fwd  p.v': 362576945 + 67108868, 'dsd_bwd  ds.k': 362576945 + 67108868,
-    'dsd_bwd  p^T.do': 403227301 + 67108864, 'dds_bwd  (q^T.ds)^T': 403227301 + 67108864,
-    'softmax_fwd': 269842570 + 268435456, 'softmax_bwd': 538083047 + 268435456,
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'traffic_attention_seq4096_fp16_blk64.json')
+
+# kernel behind each launch of the step, for the per-kernel totals
+KERNEL_OF = {
+    'sdd_fwd  q.k^T': 'k_sdd64_rg', 'sdd_bwd  do.v^T': 'k_sdd64_rg',
+    'dsd_fwd  p.v': 'k_xsd64_rg<sparse operand as stored>', 'dsd_bwd  ds.k': 'k_xsd64_rg<sparse operand as stored>',
+    'dsd_bwd  p^T.do': 'k_xsd64_rg<sparse operand transposed>', 'dds_bwd  (q^T.ds)^T': 'k_xsd64_rg<sparse operand transposed>',
+    'softmax_fwd': 'k_softmax_fwd', 'softmax_bwd': 'k_softmax_bwd',
 }
+
+
+def kernel_sources_sha():
+    """Hash of the HIP sources the library is built from: ties recorded counter readings to a build of the kernels."""
+    h = hashlib.sha256()
+    for f in sorted(glob.glob(os.path.join(PKG, 'csrc', '*'))):
+        if f.endswith(('.hip', '.h')) and not f.endswith('probe.hip'):
+            h.update(os.path.basename(f).encode())
+            h.update(open(f, 'rb').read())
+    return h.hexdigest()
+
+
+def recorded_traffic():
+    """HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), or {} when the kernels' sources have
+    changed since the counters were read (the figure would describe other kernels)."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return {}
+    return rec.get('bytes_per_launch', {}) if rec.get('kernel_sources_sha256') == kernel_sources_sha() else {}
 
 
 def main():
@@ -43,50 +76,33 @@ def main():
     ap.add_argument('--steps', type=int, default=200)
     ap.add_argument('--warmup', type=int, default=30)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-other-configs', action='store_true', help='headline only: skip configurations 2, 4 and 5')
     ap.add_argument('--batch', type=int, default=8)
     ap.add_argument('--block', type=int, default=64, choices=[16, 32, 64],
                     help='config 3 only: express the same attention mask in smaller blocks (64 = the headline workload)')
     ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
                     help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
+    ap.add_argument('--calibrate', action='store_true')
+    ap.add_argument('--record-traffic', nargs=2, metavar=('FETCH_DIR', 'WRITE_DIR'))
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit('bench.py measures one GPU: the path shards over batch and heads without communication, '
                  'and no multi-GPU run is part of this build (got --gpus %d)' % args.gpus)
+    if args.record_traffic:
+        return record_traffic(*args.record_traffic)
+    if args.calibrate:
+        return calibrate(args)
     if args.config != 3:
-        return other_config(args)
+        res = other_config(args.config, min(args.steps, 50), max(1, min(args.warmup, 5)))
+        print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
+                          'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic',
+                          'config': {'workload': res['workload'], 'config': args.config}, 'launches': res['launches']}))
+        return
 
     import torch
     import torch_blocksparse as tb
-    from torch_blocksparse.matmul import _sparse_matmul
-    dev = torch.device('cuda:0')
-    torch.manual_seed(0)
-    B, H, L, dh, block = args.batch, 16, 4096, 64, args.block
-    dtype = torch.float16
-    scale = 0.125
-    lay = tb.sparse_transformer_layout(H, L // 64, 4, 16, True)
-    if block != 64:   # the same mask, every 64-block split into (64 / block)^2 blocks: same flops, same bytes
-        lay = lay.repeat_interleave(64 // block, 1).repeat_interleave(64 // block, 2)
-    nnz = int(lay.sum())
-    q, k, v, do = [torch.randn(B, H, L, dh, dtype=dtype, device=dev) for _ in range(4)]
-    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
-    g = torch.Generator().manual_seed(1)
-    kpm = torch.zeros(B, L, dtype=dtype)
-    for z in range(B):
-        pad = int(torch.randint(0, L // 4 + 1, (1,), generator=g))
-        if pad:
-            kpm[z, L - pad:] = float('-inf')
-    kpm = kpm.to(dev)
-    sdd = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=True)
-    dsd = tb.MatMul(lay, block, 'dsd')
-    sm = tb.Softmax(lay, block)
-
-    def step():
-        q.grad = k.grad = v.grad = None
-        w = sdd(q, k)
-        p = sm(w, scale=scale, key_padding_mask=kpm)
-        o = dsd(p, v)
-        o.backward(do)
-
+    w = Attention(args.batch, args.block)
+    step = w.step
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -96,60 +112,9 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    flops_mm = 2.0 * B * dh * nnz * block * block          # per product (K = N = M = head_dim in all six)
-    es = 2
-    x_bytes = B * nnz * block * block * es
-    dense_bytes = B * H * L * dh * es
-    mm_bytes = x_bytes + 2 * dense_bytes                    # one sparse tensor + two dense tensors, each touched once
-
     # Per-launch timing with HIP events on the launch stream, the eight launches of a step issued back to back in
     # step order (so each kernel sees the cache state its predecessor leaves), K steps, one synchronisation at the end.
-    luts = {m: m.make_lut(dtype, dev) for m in (sdd, dsd)}
-    sm_lut, sm_maxlut = sm.make_lut(dev)
-    t = [None]
-    fn = _sparse_matmul.fn
-    sl, dl = luts[sdd], luts[dsd]
-    spd = lay.shape
-    st = {}
-
-    def k_sdd_fwd():
-        st['w'] = fn['sdd'](q, k, False, True, False, spd, block, sl[0], sl[1], sl[2], sl[3], False, t)
-
-    def k_softmax_fwd():
-        st['p'] = tb.Softmax.sparse_softmax(st['w'], scale, None, kpm, None, 'add', 'add', spd, block, sm_lut, sm_maxlut, False, t)
-
-    def k_dsd_fwd():
-        st['o'] = fn['dsd'](st['p'], v, False, False, False, spd, block, dl[0], dl[1], dl[2], dl[3], False, t)
-
-    def k_sdd_bwd():     # dp = do . v^T restricted to the layout
-        st['dp'] = fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t)
-
-    def k_dsd_bwd_t():   # dv = p^T . do
-        st['dv'] = fn['dsd'](st['p'], do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t)
-
-    def k_softmax_bwd():
-        _bwd_softmax(tb, st['p'], st['dp'], scale, sm_lut, sm_maxlut, spd, block)
-
-    def k_dsd_bwd():     # dq = ds . k
-        st['dq'] = fn['dsd'](st['dp'], k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t)
-
-    def k_dds_bwd():     # dk = (q^T . ds)^T
-        st['dk'] = fn['dds'](q, st['dp'], True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t)
-
-    def k_copy():        # plain copy of |x| bytes: the known-size kernel the traffic counters are calibrated on
-        st['copy'] = st['dp'].clone()
-
-    launches = [
-        ('sdd_fwd  q.k^T', k_sdd_fwd, flops_mm, mm_bytes),
-        ('softmax_fwd', k_softmax_fwd, 0.0, 2 * x_bytes + kpm.numel() * es),
-        ('dsd_fwd  p.v', k_dsd_fwd, flops_mm, mm_bytes),
-        ('dsd_bwd  p^T.do', k_dsd_bwd_t, flops_mm, mm_bytes),
-        ('sdd_bwd  do.v^T', k_sdd_bwd, flops_mm, mm_bytes),
-        ('softmax_bwd', k_softmax_bwd, 0.0, 3 * x_bytes),
-        ('dds_bwd  (q^T.ds)^T', k_dds_bwd, flops_mm, mm_bytes),
-        ('dsd_bwd  ds.k', k_dsd_bwd, flops_mm, mm_bytes),
-        ('calibration_copy', k_copy, 0.0, 2 * x_bytes),
-    ]
+    launches = w.launches() + [('calibration_copy', w.k_copy, 0.0, 2 * w.x_bytes)]
     reps = max(args.steps, 10)
     events = {name: [] for name, _, _, _ in launches}
     with torch.no_grad():
@@ -162,55 +127,172 @@ def main():
                 if it >= 3:
                     events[name].append((e0, e1))
     torch.cuda.synchronize()
+    traffic = recorded_traffic() if (args.batch == 8 and args.block == 64) else {}
     kernels = {}
     for name, _, flops, nbytes in launches:
         ms = sum(a.elapsed_time(b) for a, b in events[name]) / len(events[name])
         ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
-               'bytes': nbytes, 'traffic': TRAFFIC_BYTES.get(name) if (B == 8 and block == 64) else None}
+               'bytes': nbytes, 'traffic': traffic.get(name)}
         if flops:
             ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
             ent['mfma_frac'] = round(flops / ms * 1e-9 / MFMA_PEAK_TFLOPS, 4)
         kernels[name] = ent
     calib = kernels.pop('calibration_copy')
-    dom = max(kernels, key=lambda n: kernels[n]['ms'])
-    roofline = {'kernel': dom, 'bound': 'hbm', 'achieved': kernels[dom]['GB/s'], 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-                'frac': kernels[dom]['hbm_frac'], 'traffic': kernels[dom]['traffic']}
+    # the dominant kernel = the one with the largest total time per step over all its launches
+    per_kernel = {}
+    for name, ent in kernels.items():
+        k = per_kernel.setdefault(KERNEL_OF[name], {'launches_per_step': 0, 'ms_per_step': 0.0, 'bytes': 0, 'traffic': 0, 'have_traffic': True})
+        k['launches_per_step'] += 1
+        k['ms_per_step'] += ent['ms']
+        k['bytes'] += ent['bytes']
+        k['have_traffic'] = k['have_traffic'] and ent['traffic'] is not None
+        k['traffic'] += ent['traffic'] or 0
+    dom = max(per_kernel, key=lambda n: per_kernel[n]['ms_per_step'])
+    d = per_kernel[dom]
+    n_l = d['launches_per_step']
+    avg_ms = d['ms_per_step'] / n_l
+    achieved = d['bytes'] / n_l / avg_ms * 1e-6
+    roofline = {'kernel': dom, 'launches_per_step': n_l, 'avg_launch_ms': round(avg_ms, 4), 'bound': 'hbm',
+                'achieved': round(achieved, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s', 'frac': round(achieved / HBM_PEAK_GBS, 4),
+                'traffic': (d['traffic'] // n_l) if d['have_traffic'] else None,
+                'share_of_step': round(d['ms_per_step'] / sum(k['ms_per_step'] for k in per_kernel.values()), 4)}
 
+    block, B = args.block, args.batch
     out = {
         'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk%d' % block,
-        'value': round(6 * flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
+        'value': round(6 * w.flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f16', 'data': 'synthetic',
         'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block %d, fixed '
                                'layout (local 4 blocks + 1 global per 16 at block 64, causal), scale 1/8, additive key-padding mask' % (B, block),
-                   'nnz_blocks': nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
-        'matmul_TFLOP/s_kernel_time_only': round(6 * flops_mm / sum(e['ms'] for n, e in kernels.items() if 'softmax' not in n) * 1e-9, 2),
+                   'nnz_blocks': w.nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
+        'matmul_TFLOP/s_kernel_time_only': round(6 * w.flops_mm / sum(e['ms'] for n, e in kernels.items() if 'softmax' not in n) * 1e-9, 2),
         'softmax_GB/s': {'fwd': kernels['softmax_fwd']['GB/s'], 'bwd': kernels['softmax_bwd']['GB/s']},
         'roofline': roofline, 'kernels': kernels, 'calibration_copy': calib,
+        'traffic_source': os.path.relpath(TRAFFIC_FILE, ROOT) if traffic else None,
     }
+    lay, dh, scale = w.lay, w.dh, w.scale
+    del w
+    torch.cuda.empty_cache()
+    if not args.no_other_configs:
+        out['other_configs'] = {str(c): other_config(c, 20, 3) for c in (2, 4, 5)}
     if not args.no_cpu_baseline:
-        out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, L)
+        out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, 4096)
     print(json.dumps(out))
 
 
-def other_config(args):
+class Attention:
+    """The headline workload: operands, operators, the autograd step and its eight launches one by one."""
+
+    def __init__(self, B=8, block=64):
+        import torch
+        import torch_blocksparse as tb
+        from torch_blocksparse.matmul import _sparse_matmul
+        self.tb, self.torch = tb, torch
+        dev = torch.device('cuda:0')
+        torch.manual_seed(0)
+        H, L, dh = 16, 4096, 64
+        dtype = torch.float16
+        self.scale, self.dh, self.block = 0.125, dh, block
+        lay = tb.sparse_transformer_layout(H, L // 64, 4, 16, True)
+        if block != 64:   # the same mask, every 64-block split into (64 / block)^2 blocks: same flops, same bytes
+            lay = lay.repeat_interleave(64 // block, 1).repeat_interleave(64 // block, 2)
+        self.lay, self.nnz = lay, int(lay.sum())
+        self.q, self.k, self.v, self.do = [torch.randn(B, H, L, dh, dtype=dtype, device=dev) for _ in range(4)]
+        for t in (self.q, self.k, self.v):
+            t.requires_grad_(True)
+        g = torch.Generator().manual_seed(1)
+        kpm = torch.zeros(B, L, dtype=dtype)
+        for z in range(B):
+            pad = int(torch.randint(0, L // 4 + 1, (1,), generator=g))
+            if pad:
+                kpm[z, L - pad:] = float('-inf')
+        self.kpm = kpm.to(dev)
+        self.sdd = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=True)
+        self.dsd = tb.MatMul(lay, block, 'dsd')
+        self.sm = tb.Softmax(lay, block)
+        es = 2
+        self.flops_mm = 2.0 * B * dh * self.nnz * block * block     # per product (K = N = M = head_dim in all six)
+        self.x_bytes = B * self.nnz * block * block * es
+        self.dense_bytes = B * H * L * dh * es
+        self.mm_bytes = self.x_bytes + 2 * self.dense_bytes          # one sparse tensor + two dense tensors, each touched once
+        self.kpm_bytes = self.kpm.numel() * es
+        self.sl, self.dl = self.sdd.make_lut(dtype, dev), self.dsd.make_lut(dtype, dev)
+        self.sm_lut, self.sm_maxlut = self.sm.make_lut(dev)
+        self.fn, self.spd, self.t, self.st = _sparse_matmul.fn, lay.shape, [None], {}
+
+    def step(self):
+        q, k, v = self.q, self.k, self.v
+        q.grad = k.grad = v.grad = None
+        w = self.sdd(q, k)
+        p = self.sm(w, scale=self.scale, key_padding_mask=self.kpm)
+        o = self.dsd(p, v)
+        o.backward(self.do)
+
+    # the launches of a step, callable one by one (no autograd)
+    def k_sdd_fwd(self):
+        sl = self.sl
+        self.st['w'] = self.fn['sdd'](self.q, self.k, False, True, False, self.spd, self.block, sl[0], sl[1], sl[2], sl[3], False, self.t)
+
+    def k_softmax_fwd(self):
+        self.st['p'] = self.tb.Softmax.sparse_softmax(self.st['w'], self.scale, None, self.kpm, None, 'add', 'add', self.spd, self.block,
+                                                      self.sm_lut, self.sm_maxlut, False, self.t)
+
+    def k_dsd_fwd(self):
+        dl = self.dl
+        self.st['o'] = self.fn['dsd'](self.st['p'], self.v, False, False, False, self.spd, self.block, dl[0], dl[1], dl[2], dl[3], False, self.t)
+
+    def k_sdd_bwd(self):     # dp = do . v^T restricted to the layout
+        dl = self.dl
+        self.st['dp'] = self.fn['sdd'](self.do, self.v, False, True, False, self.spd, self.block, dl[4], dl[5], dl[6], dl[7], False, self.t)
+
+    def k_dsd_bwd_t(self):   # dv = p^T . do
+        dl = self.dl
+        self.st['dv'] = self.fn['dsd'](self.st['p'], self.do, True, False, False, self.spd, self.block, dl[8], dl[9], dl[10], dl[11], False, self.t)
+
+    def k_softmax_bwd(self):
+        _bwd_softmax(self.tb, self.st['p'], self.st['dp'], self.scale, self.sm_lut, self.sm_maxlut, self.spd, self.block)
+
+    def k_dsd_bwd(self):     # dq = ds . k
+        sl = self.sl
+        self.st['dq'] = self.fn['dsd'](self.st['dp'], self.k, False, False, False, self.spd, self.block, sl[4], sl[5], sl[6], sl[7], False, self.t)
+
+    def k_dds_bwd(self):     # dk = (q^T . ds)^T
+        sl = self.sl
+        self.st['dk'] = self.fn['dds'](self.q, self.st['dp'], True, False, True, self.spd, self.block, sl[8], sl[9], sl[10], sl[11], False, self.t)
+
+    def k_copy(self):        # plain copy of |x| bytes: the known-size kernel the traffic counters are calibrated on
+        self.st['copy'] = self.st['dp'].clone()
+
+    def launches(self):
+        """(name, callable, flops, algorithmic bytes) in step order."""
+        f, b, x = self.flops_mm, self.mm_bytes, self.x_bytes
+        return [('sdd_fwd  q.k^T', self.k_sdd_fwd, f, b), ('softmax_fwd', self.k_softmax_fwd, 0.0, 2 * x + self.kpm_bytes),
+                ('dsd_fwd  p.v', self.k_dsd_fwd, f, b), ('dsd_bwd  p^T.do', self.k_dsd_bwd_t, f, b),
+                ('sdd_bwd  do.v^T', self.k_sdd_bwd, f, b), ('softmax_bwd', self.k_softmax_bwd, 0.0, 3 * x),
+                ('dds_bwd  (q^T.ds)^T', self.k_dds_bwd, f, b), ('dsd_bwd  ds.k', self.k_dsd_bwd, f, b)]
+
+
+def other_config(config, steps, warmup):
     """The configurations the headline metric is not quoted on: every launch timed on its own (HIP events, mean of
-    `--steps` back-to-back launches), effective throughput over the nonzero blocks.  One JSON line, not the headline."""
+    `steps` back-to-back launches), effective throughput over the nonzero blocks, as a fraction of the fp16 MFMA peak
+    (the MFMA-bound configurations 2 and 5; fp32 peak for configuration 1) or of the HBM peak (configuration 4).
+    Returns {'workload': ..., 'launches': [...]}."""
     import torch
     import torch_blocksparse as tb
     dev = torch.device('cuda:0')
     out = []
 
     def timeit(f):
-        for _ in range(max(args.warmup, 1)):
+        for _ in range(max(warmup, 1)):
             f()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(args.steps):
+        for _ in range(steps):
             f()
         e1.record()
         e1.synchronize()
-        return e0.elapsed_time(e1) / args.steps
+        return e0.elapsed_time(e1) / steps
 
     def bernoulli(shape, density, seed, one_per_row=False):
         g = torch.Generator().manual_seed(seed)
@@ -235,10 +317,13 @@ def other_config(args):
             ms = timeit(lambda: op(a, b))
         D = {'sdd': K, 'dsd': N, 'dds': M}[mode]
         fl = 2.0 * Z * D * nnz * block * block
-        peak = 157.3 if dtype == torch.float32 else MFMA_PEAK_TFLOPS
-        out.append({'launch': name, 'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'mfma_frac': round(fl / ms * 1e-9 / peak, 4)})
+        es = a.element_size()
+        nbytes = es * (Z * nnz * block * block + Z * H * (M * K if mode != 'dsd' else K * N) + Z * H * (M * N if mode != 'sdd' else K * N))
+        peak = FP32_PEAK_TFLOPS if dtype == torch.float32 else MFMA_PEAK_TFLOPS
+        out.append({'launch': name, 'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'mfma_frac': round(fl / ms * 1e-9 / peak, 4),
+                    'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)})
 
-    if args.config == 1:
+    if config == 1:
         torch.manual_seed(0)
         lay = torch.randint(0, 2, (2, 16, 32))
         mm('sdd trans_a fp32 blk16 Z4 H2 256x512x384', 'sdd', True, False, 16, torch.float32, 4, 2, 256, 512, 384, lay)
@@ -248,20 +333,20 @@ def other_config(args):
             ms = timeit(lambda: sm(x))
         out.append({'launch': 'softmax fwd fp32 blk16', 'ms': round(ms, 4), 'GB/s': round(2 * x.numel() * 4 / ms * 1e-6, 1)})
         workload = 'README shape: sdd trans_a fp32 block 16 + softmax'
-    elif args.config == 2:
+    elif config == 2:
         lay = bernoulli((16, 64, 64), 0.25, 2, one_per_row=True)
         for ta in (False, True):
             for tb_ in (False, True):
                 mm('dsd trans_a=%d trans_b=%d' % (ta, tb_), 'dsd', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
                 mm('dds trans_a=%d trans_b=%d' % (ta, tb_), 'dds', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
         mm('sdd (gradient of the sparse operand)', 'sdd', False, True, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay)
-        workload = 'fp16 block 32, Z 8, H 16, M=N=K=2048, Bernoulli(0.25) layout'
-    elif args.config == 5:
+        workload = 'fp16 block 32, Z 8, H 16, M=N=K=2048, Bernoulli(0.25) layout; bound: MFMA'
+    elif config == 5:
         lay = bernoulli((1, 32, 32), 0.1, 5)
         mm('dds trans_b (y = x.W^T)', 'dds', False, True, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
         mm('dds (dx = dy.W)', 'dds', False, False, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
         mm('sdd trans_a (dW = dy^T.x on the layout)', 'sdd', True, False, 128, torch.float16, 1, 1, 4096, 4096, 8192, lay, 0.1)
-        workload = 'block-sparse linear layer: 8192 tokens, 4096x4096 weight, block 128, 10 % density, fp16'
+        workload = 'block-sparse linear layer: 8192 tokens, 4096x4096 weight, block 128, 10 % density, fp16; bound: MFMA'
     else:
         lay = tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True)
         B, H, L, dh, block = 2, 12, 16384, 64, 64
@@ -277,42 +362,151 @@ def other_config(args):
         causal = torch.tril(torch.ones(L, L, dtype=torch.float16, device=dev))
         fl = 2.0 * B * dh * nnz * block * block
         xb = B * nnz * block * block * 2
+        # both masks are shared by batch and heads (the rpe through stride-0 views): the bytes of each that the layout
+        # touches are the block positions present in any head
+        touched = int(lay.sum(0).ne(0).sum()) * block * block * 2
         do = torch.randn_like(q)
         from torch_blocksparse.matmul import _sparse_matmul
         fn, spd, t = _sparse_matmul.fn, lay.shape, [None]
         sl, dl = sdd.make_lut(torch.float16, dev), dsd.make_lut(torch.float16, dev)   # (c, da, db) tables of each op
         sm_lut, sm_maxlut = sm.make_lut(dev)
+        mmb = xb + 2 * B * H * L * dh * 2
         with torch.no_grad():
             w = sdd(q, k)
             dw = torch.randn_like(w)
             for name, f, flops, nbytes in (
-                    ('sdd q.k^T', lambda: sdd(q, k), fl, xb + 2 * B * H * L * dh * 2),
+                    ('sdd q.k^T', lambda: sdd(q, k), fl, mmb),
                     ('softmax fwd, scale only', lambda: sm(w, scale=0.125), 0, 2 * xb),
-                    ('softmax fwd, rpe + causal mask', lambda: sm(w, scale=0.125, rpe=rpe, attn_mask=causal, attn_mask_mode='mul'), 0, 2 * xb),   # x only: both masks are shared by batch and heads
-                    ('dsd p.v', lambda: dsd(w, v), fl, xb + 2 * B * H * L * dh * 2),
+                    ('softmax fwd, rpe + causal mask', lambda: sm(w, scale=0.125, rpe=rpe, attn_mask=causal, attn_mask_mode='mul'), 0, 2 * xb + 2 * touched),
+                    ('dsd p.v', lambda: dsd(w, v), fl, mmb),
                     # backward, in the order autograd runs it (the products of MatMul.backward are MatMul modes of their own)
-                    ('dsd p^T.do', lambda: fn['dsd'](w, do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t), fl, xb + 2 * B * H * L * dh * 2),
-                    ('sdd do.v^T', lambda: fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t), fl, xb + 2 * B * H * L * dh * 2),
+                    ('dsd p^T.do', lambda: fn['dsd'](w, do, True, False, False, spd, block, dl[8], dl[9], dl[10], dl[11], False, t), fl, mmb),
+                    ('sdd do.v^T', lambda: fn['sdd'](do, v, False, True, False, spd, block, dl[4], dl[5], dl[6], dl[7], False, t), fl, mmb),
                     ('softmax bwd', lambda: _bwd_softmax(tb, w, dw, 0.125, sm_lut, sm_maxlut, spd, block), 0, 3 * xb),
-                    ('dds (q^T.ds)^T', lambda: fn['dds'](q, dw, True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t), fl, xb + 2 * B * H * L * dh * 2),
-                    ('dsd ds.k', lambda: fn['dsd'](dw, k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t), fl, xb + 2 * B * H * L * dh * 2)):
+                    ('dds (q^T.ds)^T', lambda: fn['dds'](q, dw, True, False, True, spd, block, sl[8], sl[9], sl[10], sl[11], False, t), fl, mmb),
+                    ('dsd ds.k', lambda: fn['dsd'](dw, k, False, False, False, spd, block, sl[4], sl[5], sl[6], sl[7], False, t), fl, mmb)):
                 ms = timeit(f)
                 ent = {'launch': name, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)}
                 if flops:
                     ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
                 out.append(ent)
-        workload = 'BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, forward and backward launches'
-    print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
-                      'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic', 'config': {'workload': workload, 'config': args.config},
-                      'launches': out}))
+        workload = ('BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, '
+                    'forward and backward launches; bound: HBM (softmax bytes: 2|x| + the mask and rpe bytes the layout touches)')
+    torch.cuda.empty_cache()
+    return {'workload': workload, 'launches': out}
 
 
 def _bwd_softmax(tb, y, dy, scale, lut, maxlut, spdims, block):
-    import ctypes
     from torch_blocksparse import _lib
     rc = _lib.load().bsp_softmax_bwd(_lib.DTYPES[y.dtype], _lib.ptr(y), _lib.ptr(dy), float(scale), _lib.ptr(lut), maxlut,
                                      y.size(0), spdims[0], spdims[1], block, y.stride(0), dy.stride(0), _lib.stream_ptr(y.device))
     _lib.check(rc, 'bsp_softmax_bwd')
+
+
+def calibrate(args):
+    """What this box streams, and the step's kernels with cold caches.  Probes (libbsp_probe.so): 16-byte accesses in
+    address order over a 4 GiB footprint (far beyond the 256 MB memory-side cache) and over the 268 MB footprint of the
+    step's sparse tensor (which fits it).  Then every launch of the headline step timed alone, once as in the step
+    (its predecessor's output still cached) and once after a 1 GiB write that flushes L2 and the memory-side cache."""
+    import torch
+    from torch_blocksparse import _lib
+    probe_path = os.path.join(PKG, 'lib', 'libbsp_probe.so')
+    if not os.path.exists(probe_path):
+        sys.exit('%s not found: build it with `python torch-blocksparse_amd/build.py`' % probe_path)
+    probe = ctypes.CDLL(probe_path)
+    probe.bsp_probe_stream.restype = ctypes.c_int
+    probe.bsp_probe_stream.argtypes = [ctypes.c_int] + [ctypes.c_void_p] * 3 + [ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    dev = torch.device('cuda:0')
+    stream = _lib.stream_ptr(dev)
+    reps = 20
+
+    def timed(f, before=None):
+        total = 0.0
+        for it in range(reps + 2):
+            if before:
+                before()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            f()
+            e1.record()
+            e1.synchronize()
+            if it >= 2:
+                total += e0.elapsed_time(e1)
+        return total / reps
+
+    res = {'probes': []}
+    moved = {0: 1, 1: 1, 2: 2, 3: 2, 4: 3}
+    names = {0: 'read only', 1: 'write only', 2: 'copy (1 read : 1 write)', 3: 'in place (read + write back)', 4: '1 read : 2 writes'}
+    for nbytes, label in ((4 << 30, '4 GiB per buffer'), (268435456, '268 MB per buffer')):
+        bufs = [torch.empty(nbytes, dtype=torch.uint8, device=dev) for _ in range(3)]
+        for b in bufs:
+            b.zero_()
+        for mode in range(5):
+            ms = timed(lambda: probe.bsp_probe_stream(mode, _lib.ptr(bufs[0]), _lib.ptr(bufs[1]), _lib.ptr(bufs[2]), nbytes, 256 * 16, stream))
+            res['probes'].append({'probe': names[mode], 'footprint': label, 'ms': round(ms, 4),
+                                  'GB/s': round(moved[mode] * nbytes / ms * 1e-6, 1)})
+        del bufs
+        torch.cuda.empty_cache()
+    w = Attention(8, 64)
+    flush_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+
+    def flush():
+        probe.bsp_probe_stream(1, _lib.ptr(flush_buf), None, None, flush_buf.numel(), 256 * 16, stream)
+
+    launches = w.launches()
+    with torch.no_grad():
+        for _ in range(3):
+            for _, f, _, _ in launches:
+                f()
+        res['launches'] = []
+        for i, (name, f, flops, nbytes) in enumerate(launches):
+            prev = launches[i - 1][1]
+            warm = timed(f, before=prev)        # the cache state of the step: the predecessor has just run
+            cold = timed(f, before=flush)
+            res['launches'].append({'launch': name, 'bytes': nbytes, 'ms_after_predecessor': round(warm, 4),
+                                    'GB/s_after_predecessor': round(nbytes / warm * 1e-6, 1), 'ms_cold': round(cold, 4),
+                                    'GB/s_cold': round(nbytes / cold * 1e-6, 1)})
+    print(json.dumps({'metric': 'streaming calibration, not the headline metric', 'n_gpus': 1, 'data': 'synthetic', **res}))
+
+
+def record_traffic(fetch_dir, write_dir):
+    """Reads the counter CSVs of two runs
+         rocprofv3 --pmc FETCH_SIZE --output-format csv -d FETCH_DIR -o f -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline --no-other-configs
+         rocprofv3 --pmc WRITE_SIZE --output-format csv -d WRITE_DIR -o w -- python3 bench.py --steps 3 --warmup 1 --no-cpu-baseline --no-other-configs
+    and writes the HBM bytes per launch of each of the step's kernels to profiles/, scaled by what the same counter reads
+    for the run's calibration copy of 268 435 456 bytes, together with the hash of the kernel sources they belong to."""
+    import csv
+    import collections
+
+    def read(d, counter):
+        per = collections.defaultdict(list)
+        for f in glob.glob(os.path.join(d, '**', '*counter_collection.csv'), recursive=True):
+            for r in csv.DictReader(open(f)):
+                if r['Counter_Name'] == counter:
+                    per[r['Kernel_Name']].append(float(r['Counter_Value']))
+        return per
+
+    fetch, write = read(fetch_dir, 'FETCH_SIZE'), read(write_dir, 'WRITE_SIZE')
+
+    def copy_scale(per):
+        vals = [v for k, vs in per.items() if 'copyBuffer' in k for v in vs if v > 100000]    # the 268 MB copies only
+        return 268435456.0 / (sum(vals) / len(vals))
+    fs, ws = copy_scale(fetch), copy_scale(write)
+
+    def kernel_bytes(sub, *more):
+        def pick(per):
+            vals = [v for k, vs in per.items() if sub in k and all(m in k for m in more) for v in vs]
+            return sum(vals) / len(vals)
+        return int(pick(fetch) * fs + pick(write) * ws)
+    per_kernel = {'k_sdd64_rg': kernel_bytes('k_sdd64_rg'), 'k_xsd64_rg<sparse operand as stored>': kernel_bytes('k_xsd64_rg', 'Lb0E'),
+                  'k_xsd64_rg<sparse operand transposed>': kernel_bytes('k_xsd64_rg', 'Lb1E'),
+                  'k_softmax_fwd': kernel_bytes('k_softmax_fwd'), 'k_softmax_bwd': kernel_bytes('k_softmax_bwd')}
+    rec = {'kernel_sources_sha256': kernel_sources_sha(), 'bytes_per_counted_KiB': {'FETCH_SIZE': round(fs, 1), 'WRITE_SIZE': round(ws, 1)},
+           'bytes_per_kernel_launch': per_kernel, 'bytes_per_launch': {name: per_kernel[k] for name, k in KERNEL_OF.items()},
+           'note': 'averages over the launches of each kernel in a 3-step run; launches of one kernel share a figure'}
+    with open(TRAFFIC_FILE, 'w') as f:
+        json.dump(rec, f, indent=1)
+    print(json.dumps(rec))
 
 
 def cpu_baseline(lay, block, dh, scale, L):

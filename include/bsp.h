@@ -97,17 +97,33 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * and gather each tile from its blocks (bsp_sdd_matmul: scatter each result tile to the blocks present).
  * order_buckets > 0 sorts the header by entries in units of 1/order_buckets of the largest group instead of exactly
  * (equal keys head by head: better L2 reuse of the dense rows when one head's share of them is small); 0 = exact.
- * *n_groups counts groups and chains.  plan_cap >= bsp_group_plan_cap(...). */
+ * split_len > 0: a chain with more than split_len entries is cut into up to BSP_CHAIN_PARTS parts of equal length, one
+ * header row each (next to each other, in part order): the count field holds the part's entries in bits 0..19, the
+ * part's index in bits 20..25 and the number of parts minus one in bits 26..30; bits 16..30 of the head field number
+ * the split chains of the plan (fewer than 2^15, and fewer than 2^16 heads).  bsp_dsd_matmul / bsp_dds_matmul give
+ * every part a workgroup of its own; the parts leave fp32 partial results in the launcher's workspace and the last
+ * one to arrive adds them in part order (no floating-point atomics: the result does not depend on the arrival
+ * order).  This is the role of the lock epilogue in the reference's kernel (matmul.py:191-203, 246-262).
+ * Pass 0 for plans given to bsp_sdd_matmul and for blocks of 32.
+ * *n_groups counts header rows (groups, chains and parts of chains), *n_split the chains that were split.
+ * plan_cap >= bsp_group_plan_cap(...). */
 #define BSP_GROUP 4
+#define BSP_CHAIN_PARTS 8
 int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows);
-int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int order_buckets,
-                         int32_t *d_plan, int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len,
-                         void *stream);
+int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int split_len,
+                         int order_buckets, int32_t *d_plan, int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups,
+                         int *n_split, int64_t *plan_len, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Matmul launchers.  Strides are in elements; the innermost stride of every operand is 1 and rows start on
  * 16-byte boundaries.  trans_x means the stored matrix is read transposed, as in the reference.
+ * flags: 0, or a combination of the bsp_launch_flags below.  Kernel selection is a pure function of the arguments:
+ * the library reads no environment variable and keeps no state between calls.
  * ------------------------------------------------------------------------------------------------- */
+typedef enum {
+  BSP_FLAG_GENERAL_ONLY = 1,  /* take the general kernels even where a specialised one would serve (for cross-checks) */
+  BSP_FLAG_NO_GROUPS = 2      /* ignore the group plan (the per-block / per-segment kernels run instead) */
+} bsp_launch_flags;
 
 /* sparse = dense x dense: replaces _sparse_matmul._sdd_matmul + the SDD branch of the kernel
  * (matmul.py:299-364, 30-54).  One call per pack level of the sdd table.  For every valid table row
@@ -121,25 +137,36 @@ int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_ro
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
                    int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                    int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
-                   const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
+                   const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups, int plan_lines, int flags,
+                   void *stream);
 
 /* dense = sparse x dense: replaces _sparse_matmul._dsd_matmul + the DSD branch (matmul.py:507-552, 56-82).
  * C[z, h] = op(A_sparse)[h] . op(B)[z, h], written transposed when trans_c.  N = free dimension of op(B).
  * a_stride_z = 0 shares one sparse operand over the batch.  d_lut / d_plan / width from bsp_dxx_lut_build
  * with trans = !trans_a; d_gplan (optional) from bsp_group_plan_build with by_rows = !trans_a; plan_lines < 0: a
- * plan over tiles (see bsp_group_plan_build). */
+ * plan over tiles (see bsp_group_plan_build).
+ * n_split / d_ws / ws_bytes: a plan with split chains (n_split of them, as bsp_group_plan_build reported) needs
+ * scratch memory of at least bsp_xsd_workspace_bytes(n_split, N, Z) bytes, 256-byte aligned: one int32 counter per
+ * (split chain, 64-wide tile of the free dimension, batch) followed by BSP_CHAIN_PARTS fp32 tiles of 64 x 64 each.
+ * The counters must be zero when the launch starts; every launch leaves them zero, so clearing the buffer once after
+ * allocating it is enough.  Launches that share a buffer must not overlap (one stream, or one buffer per stream).
+ * 0 / NULL / 0 for plans without split chains. */
+int64_t bsp_xsd_workspace_bytes(int n_split, int free_dim, int Z);
 int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                    int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
+                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
+                   int n_split, void *d_ws, int64_t ws_bytes, int flags, void *stream);
 
 /* dense = dense x sparse: replaces _sparse_matmul._dds_matmul + the DDS branch (matmul.py:460-505, 83-99).
  * C[z, h] = op(A)[z, h] . op(B_sparse)[h], written transposed when trans_c.  M = free dimension of op(A).
- * Tables from bsp_dxx_lut_build with trans = trans_b; d_gplan (optional) with by_rows = trans_b. */
+ * Tables from bsp_dxx_lut_build with trans = trans_b; d_gplan (optional) with by_rows = trans_b; workspace as for
+ * bsp_dsd_matmul, with M as the free dimension. */
 int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                    int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
-                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines, void *stream);
+                   const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
+                   int n_split, void *d_ws, int64_t ws_bytes, int flags, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Softmax launchers: replace softmax_fwd / softmax_bwd and their dispatch (softmax.py:7-138, 144-194,

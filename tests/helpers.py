@@ -41,3 +41,46 @@ def random_layout(shape, density, seed, at_least_one_per_row=False):
                 if lay[h, r].sum() == 0:
                     lay[h, r, r % C] = 1
     return lay
+
+
+DEV = 'cuda'
+
+
+def operand_shapes(mode, trans_a, trans_b, M, N, K):
+    a = (K, M) if trans_a else (M, K)
+    b = (N, K) if trans_b else (K, N)
+    sp = {'sdd': (M, N), 'dsd': a, 'dds': b}[mode]
+    return a, b, sp
+
+
+def run_matmul_case(mode, trans_a, trans_b, block, dtype, Z=3, H=2, M=256, N=512, K=384, density=0.5, seed=1, layout=None,
+             dist='rand', scale=1.0, backward=True):
+    """Same protocol as the reference's run_test_mm (tests/test_matmul.py:44-76): y, dx, dw, through MatMul on the GPU,
+    against the fp32 dense-masked oracle."""
+    import torch_blocksparse as tb
+    from oracle import dense_oracle as D
+    torch.manual_seed(seed)
+    ashape, bshape, sp = operand_shapes(mode, trans_a, trans_b, M, N, K)
+    lay = layout if layout is not None else random_layout((H, sp[0] // block, sp[1] // block), density, seed)
+    gen = torch.rand if dist == 'rand' else torch.randn
+    a = (gen((Z, H) + ashape) * scale).to(dtype)
+    b = (gen((Z, H) + bshape) * scale).to(dtype)
+    dc = gen((Z, H, M, N)).to(dtype)
+    if mode == 'dsd':
+        a = D.dense_to_sparse(a, lay, block)
+    if mode == 'dds':
+        b = D.dense_to_sparse(b, lay, block)
+    if mode == 'sdd':
+        dc = D.dense_to_sparse(dc, lay, block)
+    rc, rda, rdb = D.matmul(a, b, mode, trans_a, trans_b, lay, block, dc=dc)
+    op = tb.MatMul(lay, block, mode, trans_a=trans_a, trans_b=trans_b)
+    ag = a.to(DEV).requires_grad_(True)
+    bg = b.to(DEV).requires_grad_(True)
+    c = op(ag, bg)
+    tag = '%s ta=%d tb=%d block=%d %s' % (mode, trans_a, trans_b, block, dtype)
+    assert_close(c, rc, dtype, tag + ' c')
+    if not backward:
+        return
+    c.backward(dc.to(DEV))
+    assert_close(ag.grad, rda, dtype, tag + ' da')
+    assert_close(bg.grad, rdb, dtype, tag + ' db')

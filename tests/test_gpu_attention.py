@@ -163,9 +163,10 @@ def test_specialised_and_general_kernels_agree(monkeypatch):
         o.backward(do)
         return o, qg.grad, kg.grad, vg.grad
     grouped = run()                                   # row-group kernels (default for block 64)
-    monkeypatch.setenv('BSP_NO_GROUPS', '1')
+    from torch_blocksparse import _lib, matmul
+    monkeypatch.setattr(matmul, 'KERNEL_FLAGS', _lib.FLAG_NO_GROUPS)
     fast = run()                                      # per-block / per-segment specialised kernels
-    monkeypatch.setenv('BSP_GENERIC_ONLY', '1')
+    monkeypatch.setattr(matmul, 'KERNEL_FLAGS', _lib.FLAG_NO_GROUPS | _lib.FLAG_GENERAL_ONLY)
     general = run()                                   # general LDS-tiled kernels
     for a, b, c, name in zip(grouped, fast, general, ('out', 'dq', 'dk', 'dv')):
         assert_close(a, c.float(), torch.float16, name + ' grouped vs general')
@@ -192,3 +193,61 @@ def test_full_size_properties():
     perm = torch.randperm(B, device=DEV)
     p2 = sm(sdd(q[perm].contiguous(), k[perm].contiguous()), scale=0.125)
     assert torch.equal(dsd(p2, v[perm].contiguous()), o1[perm])
+
+
+@pytest.mark.parametrize('batch_first', [False, True])
+def test_replace_mha_in_a_transformer_encoder_layer(batch_first):
+    # replace_mha on a small nn.TransformerEncoderLayer (all-ones layout: the replaced model must reproduce the original),
+    # in training mode without dropout so that the layer calls the attention module's forward; with a 0/1 key padding
+    # mask ('mul' mode: 0 = padded) and an additive causal mask, forward and backward.  Both models run in fp32 (two
+    # fp16 pipelines would differ from each other by their own rounding, amplified by the layer norms); the bound is
+    # 1e-4 of the largest reference value, the two models share nothing but the weights.
+    import copy
+    torch.manual_seed(21)
+    E, heads, L, B, block = 128, 2, 128, 3, 32
+    dense = torch.nn.TransformerEncoderLayer(E, heads, dim_feedforward=256, dropout=0.0, batch_first=batch_first).to(DEV)
+    sparse = copy.deepcopy(dense)
+    tb.replace_mha(sparse, torch.ones(heads, L // block, L // block, dtype=torch.int64), block)
+    assert isinstance(sparse.self_attn, tb.MultiheadAttention) and sparse.self_attn.batch_first == batch_first
+    x = torch.randn((B, L, E) if batch_first else (L, B, E), device=DEV)
+    causal = torch.full((L, L), float('-inf'), device=DEV).triu(1)
+    pad = torch.zeros(B, L, dtype=torch.bool, device=DEV)
+    pad[1, 100:] = True                                   # nn.MultiheadAttention: True = ignore this key
+    keep = (~pad).float()                                 # 'mul' mode of the sparse softmax: 0 = ignore
+    xd, xs = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    yd = dense(xd, src_mask=causal, src_key_padding_mask=pad)
+    ys = sparse(xs, src_mask=causal, src_key_padding_mask=keep)
+    g = torch.randn_like(yd)
+    yd.backward(g)
+    ys.backward(g)
+    for name, got, ref in (('output', ys, yd), ('input gradient', xs.grad, xd.grad),
+                           ('in_proj gradient', sparse.self_attn.in_proj_weight.grad, dense.self_attn.in_proj_weight.grad),
+                           ('out_proj gradient', sparse.self_attn.out_proj.weight.grad, dense.self_attn.out_proj.weight.grad)):
+        err = float((got.detach() - ref.detach()).abs().max())
+        assert err <= 1e-4 * float(ref.detach().abs().max()), 'encoder layer %s: max err %g' % (name, err)
+
+
+def test_separate_projection_weights_and_no_bias():
+    # multi_head_attention_forward with use_separate_proj_weight (q / k / v weights given one by one) and without
+    # projection biases, against torch's own functional form on an all-ones layout
+    import torch.nn.functional as F
+    torch.manual_seed(22)
+    E, heads, L, B, block = 64, 2, 64, 2, 16
+    lay = torch.ones(heads, L // block, L // block, dtype=torch.int64)
+    x = torch.randn(L, B, E, device=DEV, dtype=torch.float16)
+    wq, wk, wv, wo = [(0.1 * torch.randn(E, E, device=DEV)).half() for _ in range(4)]
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.MatMul(lay, block, 'dsd'), tb.Softmax(lay, block))
+    from torch_blocksparse.attention import multi_head_attention_forward
+    got, _ = multi_head_attention_forward(x, x, x, E, heads, None, None, None, None, False, 0.0, wo, None, *ops,
+                                          use_separate_proj_weight=True, q_proj_weight=wq, k_proj_weight=wk, v_proj_weight=wv)
+    ref, _ = F.multi_head_attention_forward(x, x, x, E, heads, None, None, None, None, False, 0.0, wo, None,
+                                            use_separate_proj_weight=True, q_proj_weight=wq, k_proj_weight=wk, v_proj_weight=wv,
+                                            need_weights=False)
+    assert_close(got, ref.float(), torch.float16, 'separate projection weights')
+
+
+def test_extra_key_position_is_refused():
+    lay = torch.ones(2, 4, 4, dtype=torch.int64)
+    for kw in (dict(add_bias_kv=True), dict(add_zero_attn=True)):
+        with pytest.raises(NotImplementedError):
+            tb.MultiheadAttention(64, 2, lay, 16, **kw)

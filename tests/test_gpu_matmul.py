@@ -4,47 +4,10 @@ import torch
 
 import torch_blocksparse as tb
 from oracle import dense_oracle as D
-from helpers import assert_close, random_layout
+from helpers import assert_close, operand_shapes, random_layout, run_matmul_case as run_case
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
-
-
-def operand_shapes(mode, trans_a, trans_b, M, N, K):
-    a = (K, M) if trans_a else (M, K)
-    b = (N, K) if trans_b else (K, N)
-    sp = {'sdd': (M, N), 'dsd': a, 'dds': b}[mode]
-    return a, b, sp
-
-
-def run_case(mode, trans_a, trans_b, block, dtype, Z=3, H=2, M=256, N=512, K=384, density=0.5, seed=1, layout=None,
-             dist='rand', scale=1.0, backward=True):
-    """Same protocol as the reference's run_test_mm (tests/test_matmul.py:44-76): y, dx, dw."""
-    torch.manual_seed(seed)
-    ashape, bshape, sp = operand_shapes(mode, trans_a, trans_b, M, N, K)
-    lay = layout if layout is not None else random_layout((H, sp[0] // block, sp[1] // block), density, seed)
-    gen = torch.rand if dist == 'rand' else torch.randn
-    a = (gen((Z, H) + ashape) * scale).to(dtype)
-    b = (gen((Z, H) + bshape) * scale).to(dtype)
-    dc = gen((Z, H, M, N)).to(dtype)
-    if mode == 'dsd':
-        a = D.dense_to_sparse(a, lay, block)
-    if mode == 'dds':
-        b = D.dense_to_sparse(b, lay, block)
-    if mode == 'sdd':
-        dc = D.dense_to_sparse(dc, lay, block)
-    rc, rda, rdb = D.matmul(a, b, mode, trans_a, trans_b, lay, block, dc=dc)
-    op = tb.MatMul(lay, block, mode, trans_a=trans_a, trans_b=trans_b)
-    ag = a.to(DEV).requires_grad_(True)
-    bg = b.to(DEV).requires_grad_(True)
-    c = op(ag, bg)
-    tag = '%s ta=%d tb=%d block=%d %s' % (mode, trans_a, trans_b, block, dtype)
-    assert_close(c, rc, dtype, tag + ' c')
-    if not backward:
-        return
-    c.backward(dc.to(DEV))
-    assert_close(ag.grad, rda, dtype, tag + ' da')
-    assert_close(bg.grad, rdb, dtype, tag + ' db')
 
 
 # the reference's 21 cases (tests/test_matmul.py:87-103): fp16, Z=3 H=2 M=256 N=512 K=384, half of the blocks kept
@@ -235,24 +198,61 @@ def test_sparse_linear_layer_config_reduced():
     run_case('dds', False, True, 128, torch.float16, Z=1, H=1, M=1024, N=4096, K=4096, layout=lay, dist='randn', scale=0.14)
 
 
-def test_linear_module():
+@pytest.mark.parametrize('tokens', [(5, 7), (3, 16)])
+def test_linear_module(tokens):
+    # y, dx and the weight gradient against dense fp32; 35 tokens are padded to a multiple of 16 inside the module (the
+    # weight gradient is an sdd product over the tokens), 48 are not
     torch.manual_seed(3)
     lay = random_layout((1, 4, 6), 0.5, 3)
     lin = tb.Linear(256, 384, 64, lay).to(DEV).half()
-    x = torch.randn(5, 7, 256, device=DEV, dtype=torch.float16, requires_grad=True)
+    x = torch.randn(*tokens, 256, device=DEV, dtype=torch.float16, requires_grad=True)
+    dy = torch.randn(*tokens, 384, device=DEV, dtype=torch.float16)
     y = lin(x)
     wd = D.sparse_to_dense(lin.weight.detach().cpu().float()[None], lay, 64)[0, 0]
     ref = x.detach().cpu().float() @ wd
     assert_close(y, ref, torch.float16, 'linear y')
-    y.sum().backward()
-    assert lin.weight.grad.shape == lin.weight.shape and x.grad.shape == x.shape
-    assert_close(x.grad, torch.ones(5, 7, 384) @ wd.t(), torch.float16, 'linear dx')
+    y.backward(dy)
+    assert_close(x.grad, dy.cpu().float() @ wd.t(), torch.float16, 'linear dx')
+    dw = x.detach().cpu().float().reshape(-1, 256).t() @ dy.cpu().float().reshape(-1, 384)
+    assert_close(lin.weight.grad, D.dense_to_sparse(dw[None, None], lay, 64)[0], torch.float16, 'linear dw')
+
+
+@pytest.mark.parametrize('mode,trans_a,trans_b', [('dsd', False, False), ('dsd', True, False), ('dds', False, False), ('dds', False, True)])
+@pytest.mark.parametrize('block', [32, 64])
+def test_sparse_operand_shared_by_the_batch(mode, trans_a, trans_b, block):
+    # a 3-D sparse operand [nnz, block, block] with a dense batch of 3: every batch multiplies the same blocks and the
+    # gradient of the sparse operand is the sum over the batch
+    torch.manual_seed(17)
+    Z, H, M, N, K = 3, 2, 128, 192, 256
+    ashape, bshape, sp = operand_shapes(mode, trans_a, trans_b, M, N, K)
+    lay = random_layout((H, sp[0] // block, sp[1] // block), 0.5, 17)
+    a = (0.25 * torch.randn((Z, H) + ashape)).half()
+    b = (0.25 * torch.randn((Z, H) + bshape)).half()
+    dc = torch.randn(Z, H, M, N).half()
+    if mode == 'dsd':
+        a = D.dense_to_sparse(a[:1], lay, block)[0]                       # [nnz, block, block]
+        full = (a[None].expand(Z, -1, -1, -1).contiguous(), b)
+    else:
+        b = D.dense_to_sparse(b[:1], lay, block)[0]
+        full = (a, b[None].expand(Z, -1, -1, -1).contiguous())
+    rc, rda, rdb = D.matmul(full[0], full[1], mode, trans_a, trans_b, lay, block, dc=dc)
+    ag, bg = a.to(DEV).requires_grad_(True), b.to(DEV).requires_grad_(True)
+    c = tb.MatMul(lay, block, mode, trans_a=trans_a, trans_b=trans_b)(ag, bg)
+    c.backward(dc.to(DEV))
+    assert_close(c, rc, torch.float16, 'c')
+    if mode == 'dsd':
+        assert_close(ag.grad, rda.sum(0), torch.float16, 'da summed over the batch')
+        assert_close(bg.grad, rdb, torch.float16, 'db')
+    else:
+        assert_close(ag.grad, rda, torch.float16, 'da')
+        assert_close(bg.grad, rdb.sum(0), torch.float16, 'db summed over the batch')
 
 
 def test_random_attention_shapes_specialised_against_general(monkeypatch):
     # 60 random layouts / block sizes / head dimensions / dtypes: the row-group kernels (blocks 16, 32, 64) must agree
     # with the general kernels on the same inputs; covers ragged groups, empty and full lines, chains, one to three batches
     import random
+    from torch_blocksparse import _lib, matmul
     rnd = random.Random(7)
     for it in range(60):
         block = rnd.choice([16, 32, 64])
@@ -285,10 +285,10 @@ def test_random_attention_shapes_specialised_against_general(monkeypatch):
                     return c
                 c.backward(ops[2])
                 return torch.cat([a.grad.flatten(), b.grad.flatten()])
-        monkeypatch.delenv('BSP_GENERIC_ONLY', raising=False)
+        monkeypatch.setattr(matmul, 'KERNEL_FLAGS', 0)
         x = f(*ops[:2]).float()
-        monkeypatch.setenv('BSP_GENERIC_ONLY', '1')
+        monkeypatch.setattr(matmul, 'KERNEL_FLAGS', _lib.FLAG_GENERAL_ONLY)
         y = f(*ops[:2]).float()
-        monkeypatch.delenv('BSP_GENERIC_ONLY', raising=False)
+        monkeypatch.setattr(matmul, 'KERNEL_FLAGS', 0)
         tol = (2e-2 if dtype == torch.bfloat16 else 4e-3) * (float(y.abs().max()) + 1e-6)
         assert torch.isfinite(x).all() and float((x - y).abs().max()) <= tol, (it, mode, block, H, R, C, Z, free, dtype)

@@ -104,3 +104,55 @@ def test_dense_oracle_softmax_properties():
     assert torch.allclose(rows, torch.ones_like(rows), atol=1e-6)
     # the gradient of a softmax row sums to zero
     assert D.sparse_to_dense(dx, lay, block).sum(-1).abs().max() < 1e-5
+
+
+def test_operand_shapes_are_checked_against_the_layout_before_any_launch():
+    # The kernels take every address from the tables, so a wrong extent must be a Python error, never a launch.  The
+    # checks run before the library is touched: CPU tensors and a stand-in table are enough to reach them.
+    from torch_blocksparse.matmul import _sparse_matmul, _check_dense, _check_sparse
+    from torch_blocksparse.softmax import _sparse_softmax
+
+    class Table:
+        nnz = 5
+    fn, spd, block = _sparse_matmul.fn, (2, 3, 4), 16      # layout [2 heads, 3 block-rows, 4 block-cols]
+    ok_sparse = torch.zeros(2, 5, 16, 16)
+    t = [None]
+    # dsd: a sparse [M=48, K=64], b dense [Z, 2, 64, N]
+    for bad_b in (torch.zeros(2, 3, 64, 32), torch.zeros(2, 2, 48, 32), torch.zeros(2, 64, 32)):
+        with pytest.raises(ValueError):
+            fn['dsd'](ok_sparse, bad_b, False, False, False, spd, block, Table(), 1, 7, None, False, t)
+    with pytest.raises(ValueError):                        # read transposed, the reduction runs over the 48 rows
+        fn['dsd'](ok_sparse, torch.zeros(2, 2, 64, 32), True, False, False, spd, block, Table(), 1, 7, None, False, t)
+    for bad_a in (torch.zeros(2, 4, 16, 16), torch.zeros(2, 5, 16, 32), torch.zeros(3, 5, 16, 16), torch.zeros(5, 16)):
+        with pytest.raises(ValueError):
+            fn['dsd'](bad_a, torch.zeros(2, 2, 64, 32), False, False, False, spd, block, Table(), 1, 7, None, False, t)
+    # dds: a dense [Z, 2, M, K=48], b sparse [48, 64]
+    with pytest.raises(ValueError):
+        fn['dds'](torch.zeros(2, 2, 32, 64), ok_sparse, False, False, False, spd, block, Table(), 1, 7, None, False, t)
+    with pytest.raises(ValueError):
+        fn['dds'](torch.zeros(2, 1, 32, 48), ok_sparse, False, False, False, spd, block, Table(), 1, 7, None, False, t)
+    # sdd: op(a) [48, K], op(b) [K, 64]
+    with pytest.raises(ValueError):
+        fn['sdd'](torch.zeros(1, 2, 32, 16), torch.zeros(1, 2, 16, 64), False, False, False, spd, block, [], None, [], [], False, t)
+    with pytest.raises(ValueError):
+        fn['sdd'](torch.zeros(1, 2, 48, 16), torch.zeros(1, 2, 16, 48), False, False, False, spd, block, [], None, [], [], False, t)
+    with pytest.raises(ValueError):
+        fn['sdd'](torch.zeros(1, 3, 48, 16), torch.zeros(1, 3, 16, 64), False, False, False, spd, block, [], None, [], [], False, t)
+    _check_dense('a', torch.zeros(1, 2, 16, 48), 2, 48, None, True)      # the accepted forms raise nothing
+    _check_sparse('b', torch.zeros(5, 16, 16), 5, 16, 3)
+    # softmax: x [Z, nnz, block, block], key_padding_mask [Z or 1, >= 64], attn_mask >= [48, 64], rpe broadcastable
+    x = torch.zeros(2, 5, 16, 16, dtype=torch.float16)
+    chk = _sparse_softmax._check_shapes
+    chk(x, torch.zeros(2, 48, 64), torch.zeros(1, 64), torch.zeros(48, 64), spd, block, 5)
+    for kw in (dict(x=torch.zeros(2, 4, 16, 16)), dict(x=torch.zeros(2, 5, 16, 8)), dict(kpm=torch.zeros(2, 48)),
+               dict(kpm=torch.zeros(3, 64)), dict(attn=torch.zeros(32, 64)), dict(attn=torch.zeros(48, 63)),
+               dict(rpe=torch.zeros(2, 2, 48, 32)), dict(rpe=torch.zeros(3, 2, 48, 64)), dict(rpe=torch.zeros(2, 3, 48, 64))):
+        with pytest.raises(ValueError):
+            chk(kw.get('x', x), kw.get('rpe'), kw.get('kpm'), kw.get('attn'), spd, block, 5)
+
+
+def test_workspace_size_of_split_chains():
+    lib = _lib.load()
+    assert lib.bsp_xsd_workspace_bytes(0, 64, 8) == 0
+    # 3 split chains x 2 tiles x 2 batches = 12 counters (rounded up to 64 ints) + 12 x 8 fp32 tiles of 64 x 64
+    assert lib.bsp_xsd_workspace_bytes(3, 128, 2) == 64 * 4 + 12 * 8 * 64 * 64 * 4

@@ -13,6 +13,7 @@ CSRC = os.path.join(HERE, 'csrc')
 LIBDIR = os.path.join(HERE, 'lib')
 OBJDIR = os.path.join(HERE, 'build')
 LIBNAME = 'libbsp_hip.so'
+PROBE_LIBNAME = 'libbsp_probe.so'
 SOURCES = ['lut.hip', 'softmax.hip', 'matmul_f16.hip', 'matmul_bf16.hip', 'matmul_f32.hip', 'matmul_fast64.hip', 'elementwise.hip', 'capi.hip']
 FLAGS = ['--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-fno-gpu-rdc', '-Wall', '-Wno-unused-function',
          # packed-fp32 instruction selection is switched off on purpose
@@ -45,7 +46,18 @@ def build(verbose=False, jobs=None, sources=None):
                 print(err)
     objs = [os.path.join(OBJDIR, os.path.splitext(s)[0] + '.o') for s in SOURCES]
     subprocess.check_call(['hipcc', '--offload-arch=gfx950', '-shared', '-fPIC', '-o', lib_path()] + objs)
+    if sources is None:
+        build_probe()
     return lib_path()
+
+
+def build_probe():
+    """The streaming probes of `bench.py --calibrate`: a separate small library, not part of the operator ABI."""
+    out = os.path.join(LIBDIR, PROBE_LIBNAME)
+    r = subprocess.run(['hipcc'] + FLAGS + ['-shared', os.path.join(CSRC, 'probe.hip'), '-o', out], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError('hipcc failed on probe.hip:\n%s' % r.stderr)
+    return out
 
 
 if __name__ == '__main__':

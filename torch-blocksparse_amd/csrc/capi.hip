@@ -1,21 +1,12 @@
 // C-ABI entry points of the matmul launchers: argument validation and dispatch.  (The table builders and
 // the softmax entry points live next to their kernels in lut.hip / softmax.hip.)
 #include "matmul_generic.h"
-#include <cstdlib>
 
 using namespace bsp;
 
 namespace {
-// BSP_GENERIC_ONLY=1 in the environment routes every launch to the general kernels (used to test both paths).
-// BSP_NO_GROUPS=1 ignores group plans (the per-block / per-segment specialised kernels run instead).
-bool no_groups() {
-  const char *e = std::getenv("BSP_NO_GROUPS");
-  return e && e[0] == '1';
-}
-bool generic_only() {
-  const char *e = std::getenv("BSP_GENERIC_ONLY");
-  return e && e[0] == '1';
-}
+bool no_groups(int flags) { return (flags & BSP_FLAG_NO_GROUPS) != 0; }
+bool general_only(int flags) { return (flags & BSP_FLAG_GENERAL_ONLY) != 0; }
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool block_ok(int block) { return block == 16 || block == 32 || block == 64 || block == 128; }
 int elems16(int dtype) { return dtype == BSP_F32 ? 4 : 8; }   // elements per 16 bytes
@@ -42,7 +33,7 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
                               int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                               int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
                               const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups,
-                              int plan_lines, void *stream) {
+                              int plan_lines, int flags, void *stream) {
   if (!a || !b || !c || !d_lut || Z <= 0 || K <= 0 || n_groups < 0) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   if (K % 16) return BSP_ERR_K_MULTIPLE;   // reference matmul.py:318-319
@@ -54,12 +45,12 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.a_sz = a_stride_z; g.a_sh = a_stride_h; g.lda = lda;
   g.b_sz = b_stride_z; g.b_sh = b_stride_h; g.ldb = ldb; g.c_sz = c_stride_z;
   g.lut = d_lut; g.valid = d_valid; g.n_groups = n_groups;
-  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  g.gplan = no_groups(flags) ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
   if (g.gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);
-  int rc = generic_only() ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
+  int rc = general_only(flags) ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
   if (rc < 0) return rc;
   if (rc >= 1) { BSP_LAUNCH_CHECK(); return rc == 2 ? BSP_OK_WHOLE_LAYOUT : BSP_OK; }
   switch (dtype) {
@@ -73,9 +64,33 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   return BSP_OK;
 }
 
-static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, void *stream) {
+// Workspace of a plan with split chains: counters (one per (split chain, free tile, batch), rounded up to a multiple of
+// 64) followed by BSP_CHAIN_PARTS fp32 tiles per counter.
+static int64_t xsd_ws_slots(int n_split, int free_dim, int Z) { return (int64_t)n_split * ((free_dim + 63) / 64) * Z; }
+static int64_t xsd_ws_counter_ints(int64_t slots) { return (slots + 63) & ~(int64_t)63; }
+
+extern "C" int64_t bsp_xsd_workspace_bytes(int n_split, int free_dim, int Z) {
+  if (n_split <= 0 || free_dim <= 0 || Z <= 0) return 0;
+  const int64_t slots = xsd_ws_slots(n_split, free_dim, Z);
+  return 4 * xsd_ws_counter_ints(slots) + slots * BSP_CHAIN_PARTS * (int64_t)(64 * 64 * sizeof(float));
+}
+
+// Fills in the workspace fields of the arguments; the plan is dropped when it has split chains and no workspace came.
+static int xsd_workspace(XsdArgs &g, int n_split, int free_dim, void *d_ws, int64_t ws_bytes) {
+  g.n_split = 0; g.counters = nullptr; g.partials = nullptr;
+  if (n_split < 0) return BSP_ERR_ARG;
+  if (!g.gplan || n_split == 0) return BSP_OK;
+  if (!d_ws || (reinterpret_cast<uintptr_t>(d_ws) & 255)) return BSP_ERR_ARG;
+  if (ws_bytes < bsp_xsd_workspace_bytes(n_split, free_dim, g.Z)) return BSP_ERR_CAPACITY;
+  g.n_split = n_split;
+  g.counters = reinterpret_cast<int32_t *>(d_ws);
+  g.partials = reinterpret_cast<float *>(g.counters + xsd_ws_counter_ints(xsd_ws_slots(n_split, free_dim, g.Z)));
+  return BSP_OK;
+}
+
+static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, int flags, void *stream) {
   hipStream_t st = as_stream(stream);
-  int rc = generic_only() ? 0 : xsd_fast64(dtype, g, block, sp_trans, dn_kc, out_nc, st);
+  int rc = general_only(flags) ? 0 : xsd_fast64(dtype, g, block, sp_trans, dn_kc, out_nc, st);
   if (rc < 0) return rc;
   if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
   switch (dtype) {
@@ -93,7 +108,7 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
                               int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
                               int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
                               const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
-                              void *stream) {
+                              int n_split, void *d_ws, int64_t ws_bytes, int flags, void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || N <= 0 || width < 0) return BSP_ERR_ARG;
   if (d_gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
@@ -107,17 +122,18 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
   g.lut = d_lut; g.order = d_plan; g.plan = d_plan + bsp_dxx_plan_pairs_offset(width); g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));   // step of the table: 8 for fp32, 16 otherwise (matmul.py:617)
   g.n_tiles = (N + 63) / 64;
-  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  g.gplan = (no_groups(flags) || general_only(flags)) ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  if (int rc = xsd_workspace(g, n_split, N, d_ws, ws_bytes)) return rc;
   // rows of the kernel = rows of op(A); op(A)(m,k) is stored [k][m] when trans_a.  Dense (n,k) = op(B)[k][n]:
   // reduction contiguous when B is read transposed.  C[m][n] has n contiguous unless written transposed.
-  return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, stream);
+  return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, flags, stream);
 }
 
 extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
                               int M, int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z,
                               int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
                               const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
-                              void *stream) {
+                              int n_split, void *d_ws, int64_t ws_bytes, int flags, void *stream) {
   if (!a || !b || !c || !d_lut || !d_plan || Z <= 0 || M <= 0 || width < 0) return BSP_ERR_ARG;
   if (d_gplan && (n_plan_groups <= 0 || plan_lines == 0)) return BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
@@ -131,9 +147,10 @@ extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, 
   g.lut = d_lut; g.order = d_plan; g.plan = d_plan + bsp_dxx_plan_pairs_offset(width); g.width = width;
   g.div2 = 2 * (block / (dtype == BSP_F32 ? 8 : 16));
   g.n_tiles = (M + 63) / 64;
-  g.gplan = no_groups() ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  g.gplan = (no_groups(flags) || general_only(flags)) ? nullptr : d_gplan; g.n_pgroups = n_plan_groups; g.lines = plan_lines;
+  if (int rc = xsd_workspace(g, n_split, M, d_ws, ws_bytes)) return rc;
   // dds is dsd on the transposed problem: kernel rows = columns of op(B) (stored [k][col] unless trans_b), dense
   // rows = rows of op(A) (reduction contiguous unless trans_a), and C[row][col] has the kernel's m index contiguous
   // unless written transposed.
-  return xsd_dispatch(dtype, g, block, !trans_b, !trans_a, trans_c != 0, stream);
+  return xsd_dispatch(dtype, g, block, !trans_b, !trans_a, trans_c != 0, flags, stream);
 }

@@ -16,7 +16,7 @@ namespace {
 // ---------------------------------------------------------------------------------------------------------
 struct Ws {
   int64_t rowcnt, rowstart, colcnt, colstart, linepacks, segstart, headmax, rank, lay, tmp, top, counts, offsets, scal;
-  int64_t gcnt, gstart, galive, gapos, end;   // group plan: per slot entries, their prefix sums, alive flag, its prefix sums
+  int64_t gcnt, gstart, galive, gapos, gsplit, gseq, end;   // group plan: per slot entries, their prefix sums, header rows, their prefix sums, split flag, its prefix sums
   __host__ Ws(int H, int R, int C) {
     int64_t hr = (int64_t)H * R, hc = (int64_t)H * C, cells = (int64_t)H * R * C, hl = hr > hc ? hr : hc;
     int64_t o = 0;
@@ -29,6 +29,7 @@ struct Ws {
     scal = take(16);
     const int64_t slots = 2 * hl + H + 8;   // groups of BSP_GROUP lines + one potential chain per line
     gcnt = take(slots); gstart = take(slots + 1); galive = take(slots); gapos = take(slots + 1);
+    gsplit = take(slots); gseq = take(slots + 1);
     end = o;
   }
 };
@@ -373,8 +374,20 @@ __device__ __forceinline__ int64_t cell(int R, int C, int h, int line, int b, in
 __device__ __forceinline__ bool thin_line(const int32_t *linecnt, int64_t j, int thin_min) {
   return thin_min > 0 && linecnt[j] >= thin_min;
 }
+// parts of a chain of n entries: 1, or (split_len > 0 and n > split_len) ceil(n / split_len), at most BSP_CHAIN_PARTS
+__device__ __forceinline__ int chain_parts(int n, int split_len) {
+  if (split_len <= 0 || n <= split_len) return 1;
+  int s = (n + split_len - 1) / split_len;
+  s = s > BSP_CHAIN_PARTS ? BSP_CHAIN_PARTS : s;
+  const int per = (n + s - 1) / s;
+  return (n + per - 1) / per;                      // no part without entries where that can be helped
+}
+// sort key of a slot's header rows: their number of entries (a split chain: the entries of one part)
+__device__ __forceinline__ int slot_key(int cnt, int rows) { return rows > 1 ? (cnt + rows - 1) / rows : cnt; }
+
+// alive[i] = number of header rows of slot i (0: none, 1: a group or a whole chain, > 1: the parts of a split chain)
 __global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H, int R, int C, int by_rows, int thin_min,
-                              int32_t *cnt, int32_t *alive) {
+                              int split_len, int32_t *cnt, int32_t *alive, int32_t *split) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
   const int64_t ng = (int64_t)H * NG;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
@@ -382,7 +395,8 @@ __global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H,
   if (i >= ng) {
     const bool thin = thin_line(linecnt, i - ng, thin_min);
     cnt[i] = thin ? linecnt[i - ng] : 0;
-    alive[i] = thin;
+    alive[i] = thin ? chain_parts(linecnt[i - ng], split_len) : 0;
+    split[i] = alive[i] > 1;
     return;
   }
   const int h = (int)(i / NG), lg = (int)(i % NG);
@@ -400,10 +414,11 @@ __global__ void k_gplan_count(const int32_t *lay, const int32_t *linecnt, int H,
   }
   cnt[i] = n;
   alive[i] = 1;   // a group without entries still zero-fills the output of its (non-thin) lines
+  split[i] = 0;
 }
 __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int32_t *linecnt, const int32_t *cnt,
-                             const int32_t *start, const int32_t *alive, int H, int R, int C, int by_rows, int thin_min,
-                             int64_t n_alive, int stream_hint, int order_buckets, int32_t *plan) {
+                             const int32_t *start, const int32_t *alive, const int32_t *seq, int H, int R, int C, int by_rows,
+                             int thin_min, int64_t n_alive, int stream_hint, int order_buckets, int32_t *plan) {
   const int L = by_rows ? R : C, B = by_rows ? C : R, NG = (L + BSP_GROUP - 1) / BSP_GROUP;
   const int64_t ng = (int64_t)H * NG, slots = ng + (int64_t)H * L;
   int64_t i = blockIdx.x * (int64_t)blockDim.x + threadIdx.x;
@@ -412,18 +427,22 @@ __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int3
   // key is the number of entries in units of 1/order_buckets of the largest group (chains not counted for the scale):
   // the long groups still start first, but the many short ones behind them run head by head, so that the workgroups
   // on the chip at one time want the dense rows of a few heads only and find them in L2.
-  const int mine = cnt[i];
+  // The parts of a split chain sort by the entries of one part and stay next to each other, in part order.
+  const int mine = cnt[i], parts = alive[i], key = slot_key(mine, parts);
   int64_t pos = 0;
   if (order_buckets > 0) {
     int mx = 0;
     for (int64_t j = 0; j < ng; j++) mx = alive[j] && cnt[j] > mx ? cnt[j] : mx;
-    const int64_t km = (int64_t)mine * order_buckets / (mx + 1);
+    const int64_t km = (int64_t)key * order_buckets / (mx + 1);
     for (int64_t j = 0; j < slots; j++) {
-      const int64_t kj = (int64_t)cnt[j] * order_buckets / (mx + 1);
-      pos += alive[j] && ((kj > km) || (kj == km && j < i));
+      const int64_t kj = (int64_t)slot_key(cnt[j], alive[j]) * order_buckets / (mx + 1);
+      pos += ((kj > km) || (kj == km && j < i)) ? alive[j] : 0;
     }
   } else {
-    for (int64_t j = 0; j < slots; j++) pos += alive[j] && ((cnt[j] > mine) || (cnt[j] == mine && j < i));
+    for (int64_t j = 0; j < slots; j++) {
+      const int kj = slot_key(cnt[j], alive[j]);
+      pos += ((kj > key) || (kj == key && j < i)) ? alive[j] : 0;
+    }
   }
   int32_t *hd = plan + 4 * pos;
   int32_t *e = plan + 4 * n_alive + (int64_t)(BSP_GROUP + 1) * start[i];
@@ -438,7 +457,17 @@ __global__ void k_gplan_fill(const int32_t *lay, const int32_t *rank, const int3
     use[g] = chain ? g == 0 : (line < L && !thin);
     skip |= thin ? 1 << g : 0;
   }
-  hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = chain ? -(first + 1) : (first / BSP_GROUP) | (skip << 24) | (stream_hint << 28);
+  if (parts > 1) {
+    // part p of a split chain: entries [p * key, min((p + 1) * key, mine)), its index and the number of parts in bits
+    // 20.. and 26.. of the count field, the chain's number among the split chains of the plan in bits 16.. of the head field
+    for (int p = 0; p < parts; p++) {
+      const int lo = p * key, hi = lo + key < mine ? lo + key : mine;
+      int32_t *hp = hd + 4 * p;
+      hp[0] = start[i] + lo; hp[1] = (hi > lo ? hi - lo : 0) | (p << 20) | ((parts - 1) << 26); hp[2] = h | (seq[i] << 16); hp[3] = -(first + 1);
+    }
+  } else {
+    hd[0] = start[i]; hd[1] = mine; hd[2] = h; hd[3] = chain ? -(first + 1) : (first / BSP_GROUP) | (skip << 24) | (stream_hint << 28);
+  }
   for (int bb = 0; bb < B; bb++) {
     // Column groups list their positions from the last one down: the long lines of a causal layout (global
     // columns) then walk the dense operand's rows in step with each other and share them in L2 (measured: 12 % fewer
@@ -643,16 +672,16 @@ extern "C" int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, i
 
 extern "C" int64_t bsp_group_plan_cap(int H, int R, int C, int64_t nnz, int by_rows) {
   const int64_t L = by_rows ? R : C;
-  return 4 * ((int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (int64_t)H * L) + (BSP_GROUP + 1) * nnz;
+  return 4 * ((int64_t)H * ((L + BSP_GROUP - 1) / BSP_GROUP) + (int64_t)BSP_CHAIN_PARTS * H * L) + (BSP_GROUP + 1) * nnz;
 }
 
-extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int order_buckets,
-                                    int32_t *d_plan,
-                                    int64_t plan_cap, void *d_ws, int64_t ws_bytes, int *n_groups, int64_t *plan_len,
-                                    void *stream) {
+extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_rows, int thin_min, int split_len,
+                                    int order_buckets, int32_t *d_plan, int64_t plan_cap, void *d_ws, int64_t ws_bytes,
+                                    int *n_groups, int *n_split, int64_t *plan_len, void *stream) {
   int rc = check_args(d_layout, H, R, C, d_ws, ws_bytes);
   if (rc != BSP_OK) return rc;
-  if (!d_plan || !n_groups || !plan_len || thin_min < 0 || order_buckets < 0) return BSP_ERR_ARG;
+  if (!d_plan || !n_groups || !n_split || !plan_len || thin_min < 0 || split_len < 0 || order_buckets < 0) return BSP_ERR_ARG;
+  if (H >= (1 << 16)) return BSP_ERR_UNSUPPORTED;   // the head shares its header field with a split chain's number
   hipStream_t st = as_stream(stream);
   Ws o(H, R, C);
   int32_t *ws = (int32_t *)d_ws;
@@ -665,16 +694,20 @@ extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C
   const int32_t *linecnt = ws + (by_rows ? o.rowcnt : o.colcnt);
   hipLaunchKernelGGL(k_rank, dim3(cdiv((int64_t)H * R, T)), dim3(T), 0, st, d_layout, H, R, C, ws + o.rowstart, ws + o.rank);
   hipLaunchKernelGGL(k_gplan_count, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, linecnt, H, R, C, by_rows, thin_min,
-                     ws + o.gcnt, ws + o.galive);
+                     split_len, ws + o.gcnt, ws + o.galive, ws + o.gsplit);
   hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.gcnt, ws + o.gstart, slots, (int32_t *)nullptr);
   hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.galive, ws + o.gapos, slots, (int32_t *)nullptr);
+  hipLaunchKernelGGL(k_exclusive_scan, dim3(1), dim3(1024), 0, st, ws + o.gsplit, ws + o.gseq, slots, (int32_t *)nullptr);
   BSP_LAUNCH_CHECK();
-  int32_t total = 0, n_alive = 0, in_groups = 0;
+  int32_t total = 0, n_alive = 0, in_groups = 0, splits = 0;
+  BSP_HIP_CHECK(hipMemcpyAsync(&splits, ws + o.gseq + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipMemcpyAsync(&total, ws + o.gstart + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipMemcpyAsync(&in_groups, ws + o.gstart + ng, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipMemcpyAsync(&n_alive, ws + o.gapos + slots, sizeof(int32_t), hipMemcpyDeviceToHost, st));
   BSP_HIP_CHECK(hipStreamSynchronize(st));
+  if (splits >= (1 << 15)) return BSP_ERR_UNSUPPORTED;
   *n_groups = (int)n_alive;
+  *n_split = (int)splits;
   *plan_len = 4 * (int64_t)n_alive + (int64_t)(BSP_GROUP + 1) * total;
   if (*plan_len > plan_cap) return BSP_ERR_CAPACITY;
   // Streaming hint (bit 28 of every group's index field): set when a dense tile is wanted by few groups (at most
@@ -683,7 +716,7 @@ extern "C" int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C
   // per tile), 20-30 % slower on the long-context layout with random blocks (3.9-4.5), whose tiles come back later.
   const int stream_hint = 2 * (int64_t)in_groups <= 5 * (int64_t)H * (by_rows ? C : R);
   hipLaunchKernelGGL(k_gplan_fill, dim3(cdiv(slots, T)), dim3(T), 0, st, d_layout, ws + o.rank, linecnt, ws + o.gcnt, ws + o.gstart,
-                     ws + o.galive, H, R, C, by_rows, thin_min, (int64_t)n_alive, stream_hint, order_buckets, d_plan);
+                     ws + o.galive, ws + o.gseq, H, R, C, by_rows, thin_min, (int64_t)n_alive, stream_hint, order_buckets, d_plan);
   BSP_LAUNCH_CHECK();
   BSP_HIP_CHECK(hipStreamSynchronize(st));
   return BSP_OK;

@@ -426,7 +426,8 @@ __global__ void __launch_bounds__(256) k_sdd64_rg(SddArgs g) {
 // the reduction instead: wavefront w takes entries w, w+4, ... and computes all 64 rows of the line for them, in its
 // own piece of LDS and without workgroup barriers; the four partial results are added through LDS at the end.
 template <typename T, bool SP_TRANS, int SUBS = 1>
-__device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int n0, int depth, int line, table_ptr ent, int ne) {
+__device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int n0, int depth, int line, table_ptr ent, int ne,
+                                          int part, int parts, int seq) {
   constexpr int ENT = plan_entry_ints<SUBS>(), BLKF = 64 / SUBS;
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
@@ -537,6 +538,37 @@ __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int 
     }
   }
   __syncthreads();
+  if (parts > 1) {
+    // One part of a split chain.  Its sums go to the workspace as fp32; the part that arrives last (a counter per
+    // chain, tile and batch, stepped with an integer atomic after a release fence) reads all parts back and adds them
+    // in part order, so the result does not depend on which part was last.  The counter returns to zero.
+    const int64_t slot = ((int64_t)seq * g.n_tiles + n0 / 64) * g.Z + z;
+    f32x4 *ws = reinterpret_cast<f32x4 *>(g.partials) + (slot * BSP_CHAIN_PARTS) * 1024;   // 1024 f32x4 = one 64 x 64 tile
+#pragma unroll
+    for (int j = 0; j < 4; j++) ws[((int64_t)part * 4 + wave) * 256 + j * 64 + lane] = fin[j];
+    __threadfence();                                 // the tile is visible device-wide before the counter moves
+    __syncthreads();
+    int *flag = reinterpret_cast<int *>(smem);
+    if (threadIdx.x == 0) {
+      const int seen = atomicAdd(g.counters + slot, 1);
+      if (seen == parts - 1) g.counters[slot] = 0;   // nobody else touches this counter until the next launch
+      *flag = seen;
+    }
+    __syncthreads();
+    const bool last = *flag == parts - 1;
+    __syncthreads();                                 // the flag's LDS word is staging space again below
+    if (!last) return;
+    __threadfence();                                 // read the other parts' tiles only after seeing their counter steps
+#pragma unroll
+    for (int j = 0; j < 4; j++) fin[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int p = 0; p < parts; p++) {
+#pragma unroll
+      for (int j = 0; j < 4; j++) {
+        const f32x4 v = ws[((int64_t)p * 4 + wave) * 256 + j * 64 + lane];
+        fin[j] += v;
+      }
+    }
+  }
   T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
   store_slice<T, true>(smem + (wave * 16) * kLdsRow, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, fin, lane);
 }
@@ -559,8 +591,9 @@ __device__ __forceinline__ void xsd64_rg_body(const XsdArgs &g, T *smem) {
   const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
   const int e0 = hd[0], ne = hd[1], depth = hd[2], code = hd[3];
   const table_ptr ent = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)ENT * e0;
-  if (code < 0) {   // a chain: the line -(code + 1) on its own
-    xsd_chain<T, SP_TRANS, SUBS>(g, smem, z, n0, depth, -(code + 1), ent, ne);
+  if (code < 0) {   // a chain: the line -(code + 1) on its own, or one part of it (see bsp_group_plan_build)
+    xsd_chain<T, SP_TRANS, SUBS>(g, smem, z, n0, depth & 0xffff, -(code + 1), ent, ne & 0xfffff, (ne >> 20) & 63, ((ne >> 26) & 31) + 1,
+                                 depth >> 16);
     return;
   }
   const int lg = code & 0xffffff, skip = (code >> 24) & 0xf;   // members whose line is a chain are left to that chain
@@ -1118,7 +1151,7 @@ bool fast_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
 // The member-per-wavefront kernel pays while the free dimension is short; with many 64-wide tiles the general kernel's
 // 256-wide tile reuses each sparse block four times.
 bool small_ok_xsd(const XsdArgs &g, int block, bool dn_kc, bool out_nc) {
-  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && !dn_kc && out_nc && g.NF % 64 == 0 && g.NF <= 128;
+  return (block == 16 || block == 32) && g.gplan && g.n_pgroups > 0 && g.n_split == 0 && !dn_kc && out_nc && g.NF % 64 == 0 && g.NF <= 128;
 }
 template <typename T> int xsd_small_t(const XsdArgs &g, int block, bool sp_trans, hipStream_t st) {
   const int64_t n = (int64_t)g.n_pgroups * g.n_tiles * g.Z;

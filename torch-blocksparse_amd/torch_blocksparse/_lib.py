@@ -15,6 +15,8 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), 'lib', 'libbsp_hip.so')
 F16, BF16, F32 = 0, 1, 2
 DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 
+FLAG_GENERAL_ONLY, FLAG_NO_GROUPS = 1, 2   # bsp_launch_flags
+
 OK = 0
 OK_WHOLE_LAYOUT = 1   # bsp_sdd_matmul: the group plan was used, every block of the layout is written
 ERR_CAPACITY = -3
@@ -39,13 +41,14 @@ SIGNATURES = {
     'bsp_dxx_lut_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _vp, _i64, _pi64, _pi, _pi, _vp]),
     'bsp_sdd_lut_build': (_i, [_vp, _i, _i, _i, _i, _vp, _vp, _i64, _vp, _i64, _pi, _pi, _pi64, _pi64, _pi, _vp]),
     'bsp_group_plan_cap': (_i64, [_i, _i, _i, _i64, _i]),
-    'bsp_group_plan_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _i64, _pi, _pi64, _vp]),
+    'bsp_group_plan_build': (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp, _i64, _vp, _i64, _pi, _pi, _pi64, _vp]),
+    'bsp_xsd_workspace_bytes': (_i64, [_i, _i, _i]),
     'bsp_sdd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _i, _vp, _vp,
-                            _i64, _vp, _i, _i, _vp]),
+                            _i64, _vp, _i, _i, _i, _vp]),
     'bsp_dsd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
-                            _i, _vp, _i, _i, _vp]),
+                            _i, _vp, _i, _i, _i, _vp, _i64, _i, _vp]),
     'bsp_dds_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
-                            _i, _vp, _i, _i, _vp]),
+                            _i, _vp, _i, _i, _i, _vp, _i64, _i, _vp]),
     'bsp_softmax_fwd': (_i, [_i, _vp, _f, _vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _i, _vp, _i64, _i, _i, _i, _i, _i,
                              _i64, _vp]),
     'bsp_softmax_bwd': (_i, [_i, _vp, _vp, _f, _vp, _i, _i, _i, _i, _i, _i64, _i64, _vp]),

@@ -112,6 +112,10 @@ class MultiheadAttention(nn.modules.activation.MultiheadAttention):
                  kdim=None, vdim=None, key_padding_mask_mode='add', attn_mask_mode='mul'):
         if dropout != 0:
             raise NotImplementedError('dropout is not supported for now')
+        if add_bias_kv or add_zero_attn:
+            # one more key position than the sequence has: L + 1 is not a whole number of blocks, so no [L/block, L/block]
+            # layout can describe the scores (the reference accepts the flags and then fails inside its kernels)
+            raise NotImplementedError('add_bias_kv / add_zero_attn append a key position, which a square block layout cannot hold')
         super(MultiheadAttention, self).__init__(embed_dim, num_heads, dropout, bias, add_bias_kv, add_zero_attn, kdim, vdim)
         self.layout = layout
         self.block = block
@@ -119,32 +123,47 @@ class MultiheadAttention(nn.modules.activation.MultiheadAttention):
         self.attn_mask_mode = attn_mask_mode
         self._ops = dict()
 
-    def forward(self, query, key, value, key_padding_mask=None, need_weights=True, attn_mask=None):
+    def forward(self, query, key, value, key_padding_mask=None, need_weights=True, attn_mask=None,
+                average_attn_weights=True, is_causal=False):
+        """query / key / value: [L, batch, embed] ([batch, L, embed] if the module was made batch_first by replace_mha).
+        The last two arguments exist because current torch.nn layers pass them; attention weights are never returned
+        (the second result is None, as in the reference) and is_causal without a mask is refused."""
         if query.shape != key.shape or key.shape != value.shape:
             raise NotImplementedError('only self-attention is supported for now')
+        if is_causal and attn_mask is None:
+            raise NotImplementedError('is_causal needs the causal mask passed as attn_mask (or a causal layout)')
+        if self.batch_first:
+            query, key, value = [t.transpose(0, 1) for t in (query, key, value)]
         sdd_nt, dsd_nn, softmax = self.get_ops(query.shape[0])
         extra = dict()
         if not self._qkv_same_embed_dim:
             extra = dict(use_separate_proj_weight=True, q_proj_weight=self.q_proj_weight,
                          k_proj_weight=self.k_proj_weight, v_proj_weight=self.v_proj_weight)
-        return multi_head_attention_forward(
+        out, _ = multi_head_attention_forward(
             query, key, value, self.embed_dim, self.num_heads, self.in_proj_weight, self.in_proj_bias,
             self.bias_k, self.bias_v, self.add_zero_attn, self.dropout, self.out_proj.weight, self.out_proj.bias,
             sdd_nt, dsd_nn, softmax, training=self.training, key_padding_mask=key_padding_mask,
             need_weights=need_weights, attn_mask=attn_mask, key_padding_mask_mode=self.key_padding_mask_mode,
             attn_mask_mode=self.attn_mask_mode, **extra)
+        return (out.transpose(0, 1) if self.batch_first else out), None
 
 
 def replace_mha(model, layout, block):
-    """Swap every nn.MultiheadAttention inside `model` for the block-sparse one, keeping its parameters."""
+    """Swap every nn.MultiheadAttention inside `model` for the block-sparse one, keeping its parameters, dtype, device
+    and batch_first setting.  The reference's replace_mha(model, info) hands `info` to a constructor that needs layout
+    AND block (attention.py:267-281) and cannot run; this one takes both.  Like the reference it builds the replacement
+    with key_padding_mask_mode='mul' and attn_mask_mode='add', the conventions of nn.MultiheadAttention's masks
+    (boolean / 0-1 padding mask, additive float attention mask); masks must have the dtype of the activations."""
     for child_name, child in model.named_children():
         if isinstance(child, nn.modules.activation.MultiheadAttention) and not isinstance(child, MultiheadAttention):
-            device = child.in_proj_weight.device if child.in_proj_weight is not None else child.q_proj_weight.device
+            ref = child.in_proj_weight if child.in_proj_weight is not None else child.q_proj_weight
             mha = MultiheadAttention(child.embed_dim, child.num_heads, layout, block, dropout=child.dropout,
-                                     add_bias_kv=child.bias_k is not None, add_zero_attn=child.add_zero_attn,
-                                     kdim=child.kdim, vdim=child.vdim, key_padding_mask_mode='mul',
-                                     attn_mask_mode='add').to(device)
+                                     bias=child.in_proj_bias is not None, add_bias_kv=child.bias_k is not None,
+                                     add_zero_attn=child.add_zero_attn, kdim=child.kdim, vdim=child.vdim,
+                                     key_padding_mask_mode='mul', attn_mask_mode='add').to(device=ref.device, dtype=ref.dtype)
+            mha.batch_first = child.batch_first
             mha.load_state_dict(child.state_dict())
+            mha.train(child.training)
             setattr(model, child_name, mha)
         else:
             replace_mha(child, layout, block)

@@ -13,8 +13,28 @@ import torch
 from . import _lib
 
 
+# Flags handed to every matmul launch (bsp_launch_flags of the C ABI).  0 in normal use; the tests that compare the kernel
+# families with each other set _lib.FLAG_GENERAL_ONLY / _lib.FLAG_NO_GROUPS here.
+KERNEL_FLAGS = 0
+
+
 def _vec(dtype):
     return 4 if dtype == torch.float32 else 8
+
+
+class _LayoutOnDevice:
+    """The int32 copy of a layout on the device, its number of blocks and the builders' workspace: made once per
+    `MatMul.make_lut` and shared by the tables it builds."""
+
+    def __init__(self, layout, device):
+        self.device = torch.device(device)
+        self.lay = _lib.layout_to_device(layout, self.device)
+        self.ws, self.ws_bytes = _lib.workspace(self.lay, self.device)
+        self.nnz = int((layout != 0).sum())
+
+    @staticmethod
+    def of(layout, device, ctx):
+        return ctx if ctx is not None else _LayoutOnDevice(layout, device)
 
 
 def _prep(x):
@@ -44,10 +64,13 @@ class _Timer:
 
 
 class GroupPlan:
-    """Work list of the row-group kernels (see bsp_group_plan_build): device table, number of groups, lines per head."""
+    """Work list of the row-group kernels (see bsp_group_plan_build): device table, number of header rows, lines per
+    head, number of split chains (their fp32 partial tiles live in `workspace`)."""
 
-    def __init__(self, table, n_groups, lines):
-        self.table, self.n_groups, self.lines = table, n_groups, lines
+    def __init__(self, table, n_groups, lines, n_split=0):
+        self.table, self.n_groups, self.lines, self.n_split = table, n_groups, lines, n_split
+        self.coarse = False
+        self._ws = None
 
     @staticmethod
     def thin_min(layout, by_rows, block=64):
@@ -59,6 +82,9 @@ class GroupPlan:
         mean = float((layout != 0).sum()) / max(1, H * (R if by_rows else C))
         return max(16 if block >= 64 else 128, int(2 * mean + 0.5))
 
+    # A chain with more entries than this is cut into parts that run as workgroups of their own (block-64 kernels).
+    SPLIT_LEN = 64
+
     @staticmethod
     def order_buckets(layout, by_rows, block):
         """Coarse (8 steps) rather than exact longest-first order of the groups when the dense rows one head reads are
@@ -69,24 +95,23 @@ class GroupPlan:
         return 8 if (C if by_rows else R) * block <= 8192 else 0
 
     @staticmethod
-    def build(layout, by_rows, device, thin_min=None, order_buckets=0):
+    def build(layout, by_rows, device, thin_min=None, order_buckets=0, split_len=0, ctx=None):
         """thin_min: lines at least this long become chains; None = GroupPlan.thin_min(...), 0 = no chains.
-        order_buckets: see GroupPlan.order_buckets; 0 = exact longest-first order."""
+        order_buckets: see GroupPlan.order_buckets; 0 = exact longest-first order.  split_len: chains longer than this
+        are cut into parts (0 = never; only the block-64 dsd/dds kernels know how to add the parts up)."""
         lib = _lib.load()
-        dev = torch.device(device)
-        lay = _lib.layout_to_device(layout, dev)
+        ctx = _LayoutOnDevice.of(layout, device, ctx)
+        dev, lay = ctx.device, ctx.lay
         H, R, C = lay.shape
-        ws, ws_bytes = _lib.workspace(lay, dev)
-        nnz = int((layout != 0).sum())
-        cap = lib.bsp_group_plan_cap(H, R, C, nnz, int(bool(by_rows)))
+        cap = lib.bsp_group_plan_cap(H, R, C, ctx.nnz, int(bool(by_rows)))
         table = torch.empty((cap,), dtype=torch.int32, device=dev)
-        n_groups, n = ctypes.c_int(0), ctypes.c_int64(0)
+        n_groups, n_split, n = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int64(0)
         thin = GroupPlan.thin_min(layout, by_rows) if thin_min is None else int(thin_min)
-        rc = lib.bsp_group_plan_build(_lib.ptr(lay), H, R, C, int(bool(by_rows)), thin, int(order_buckets), _lib.ptr(table), cap,
-                                      _lib.ptr(ws), ws_bytes,
-                                      ctypes.byref(n_groups), ctypes.byref(n), _lib.stream_ptr(dev))
+        rc = lib.bsp_group_plan_build(_lib.ptr(lay), H, R, C, int(bool(by_rows)), thin, int(split_len), int(order_buckets),
+                                      _lib.ptr(table), cap, _lib.ptr(ctx.ws), ctx.ws_bytes, ctypes.byref(n_groups),
+                                      ctypes.byref(n_split), ctypes.byref(n), _lib.stream_ptr(dev))
         _lib.check(rc, 'bsp_group_plan_build')
-        return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C)
+        return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C, n_split.value)
 
     @staticmethod
     def build_coarse(layout, block, by_rows, device, for_sdd=False):
@@ -105,7 +130,8 @@ class GroupPlan:
         lay = (layout != 0)
         coarse = lay.reshape(H, R // S, S, C // S, S).any(4).any(2).to(torch.int64)
         plan = GroupPlan.build(coarse, by_rows, dev, thin_min=0 if for_sdd else GroupPlan.thin_min(coarse, by_rows, 64),
-                               order_buckets=2 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64))
+                               order_buckets=2 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64),
+                               split_len=0 if for_sdd else GroupPlan.SPLIT_LEN)
         ng, G = plan.n_groups, 4
         table = plan.table
         header, entries = table[:4 * ng], table[4 * ng:].view(-1, G + 1)
@@ -117,15 +143,62 @@ class GroupPlan:
         ids = entries[:, 1:].to(torch.int64)                                    # [entries, G] tile ids or -1
         sub = torch.where((ids >= 0).unsqueeze(2), tiles[ids.clamp(min=0)], torch.full((), -1, dtype=torch.int32, device=dev))
         wide = torch.cat([entries, sub.reshape(entries.shape[0], G * S * S)], 1).to(torch.int32)
-        out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines)
+        out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines, plan.n_split)
         out.coarse = True
         return out
+
+    def workspace(self, free_dim, Z):
+        """(pointer, bytes) of the scratch buffer the split chains of this plan need for a launch with this free dimension
+        and batch: counters + fp32 partial tiles, zeroed when allocated (every launch leaves the counters zero) and
+        kept for the next call; (NULL, 0) for a plan without split chains.  One buffer per plan: launches of one
+        operator are assumed to be ordered on one stream."""
+        if self.n_split == 0:
+            return ctypes.c_void_p(0), 0
+        need = _lib.load().bsp_xsd_workspace_bytes(self.n_split, int(free_dim), int(Z))
+        if self._ws is None or self._ws.numel() < need:
+            self._ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+        return _lib.ptr(self._ws), self._ws.numel()
 
     @staticmethod
     def args(plan):
         if plan is None:
             return ctypes.c_void_p(0), 0, 0
-        return _lib.ptr(plan.table), plan.n_groups, (-plan.lines if getattr(plan, 'coarse', False) else plan.lines)
+        return _lib.ptr(plan.table), plan.n_groups, (-plan.lines if plan.coarse else plan.lines)
+
+    @staticmethod
+    def xsd_args(plan, free_dim, Z):
+        """The plan, its split chains and their workspace, as bsp_dsd_matmul / bsp_dds_matmul take them."""
+        if plan is None:
+            return ctypes.c_void_p(0), 0, 0, 0, ctypes.c_void_p(0), 0
+        ws, ws_bytes = plan.workspace(free_dim, Z)
+        return GroupPlan.args(plan) + (plan.n_split, ws, ws_bytes)
+
+
+def _check_dense(name, x, heads, rows, cols, trans):
+    """A dense operand against the layout: [Z, heads, rows, cols] as stored when not read transposed, [Z, heads, cols,
+    rows] otherwise; None = the free dimension, any size.  The kernels take every address from the tables (head,
+    block-row, block id), so a wrong extent would be an out-of-bounds access on the device, not an error."""
+    if x.dim() != 4:
+        raise ValueError('matmul operand %s must have 4 dimensions [batch, heads, rows, cols], got %s' % (name, tuple(x.shape)))
+    if x.size(1) != heads:
+        raise ValueError('matmul operand %s has %d heads, the layout has %d' % (name, x.size(1), heads))
+    r, c = (x.size(3), x.size(2)) if trans else (x.size(2), x.size(3))
+    if rows is not None and r != rows:
+        raise ValueError('matmul operand %s: op(%s) has %d rows, the layout needs %d' % (name, name, r, rows))
+    if cols is not None and c != cols:
+        raise ValueError('matmul operand %s: op(%s) has %d columns, the layout needs %d' % (name, name, c, cols))
+
+
+def _check_sparse(name, x, nnz, block, Z):
+    """A sparse operand: [nnz, block, block] (shared by the batch) or [Z or 1, nnz, block, block]."""
+    if x.dim() not in (3, 4):
+        raise ValueError('sparse matmul operand %s must be [nnz, block, block] or [batch, nnz, block, block], got %s' % (name, tuple(x.shape)))
+    if tuple(x.shape[-2:]) != (block, block):
+        raise ValueError('sparse matmul operand %s has blocks of %s, expected (%d, %d)' % (name, tuple(x.shape[-2:]), block, block))
+    if nnz is not None and x.size(-3) != nnz:
+        raise ValueError('sparse matmul operand %s has %d blocks, the layout has %d' % (name, x.size(-3), nnz))
+    if x.dim() == 4 and x.size(0) not in (1, Z):
+        raise ValueError('sparse matmul operand %s has batch %d, the dense operand has %d' % (name, x.size(0), Z))
 
 
 class SddTables(list):
@@ -141,7 +214,7 @@ class _sparse_matmul(torch.autograd.Function):
     # SPARSE = DENSE x DENSE #
     ##########################
     @staticmethod
-    def make_sdd_lut(layout, block, dtype, device):
+    def make_sdd_lut(layout, block, dtype, device, ctx=None):
         """-> (luts, None, widths, packs) as the reference (matmul.py:281-297); built on `device`.
 
         start_width is 64 // block in the reference, which is 0 for block 128 and leaves the table empty
@@ -149,12 +222,10 @@ class _sparse_matmul(torch.autograd.Function):
         Each table tensor carries `.valid` (None, or a uint8 tensor marking the rows that really are blocks).
         """
         lib = _lib.load()
-        dev = torch.device(device)
-        lay = _lib.layout_to_device(layout, dev)
+        ctx = _LayoutOnDevice.of(layout, device, ctx)
+        dev, lay, nnz = ctx.device, ctx.lay, ctx.nnz
         H, R, C = lay.shape
-        ws, ws_bytes = _lib.workspace(lay, dev)
         start_width = max(1, 64 // block)
-        nnz = int((layout != 0).sum())
         cap = nnz + nnz // 8 + 64
         n_levels = ctypes.c_int(0)
         packs = (ctypes.c_int * 8)()
@@ -164,8 +235,8 @@ class _sparse_matmul(torch.autograd.Function):
         for attempt in range(2):
             lut = torch.empty((cap, 4), dtype=torch.int32, device=dev)
             valid = torch.empty((cap,), dtype=torch.uint8, device=dev)
-            rc = lib.bsp_sdd_lut_build(_lib.ptr(lay), H, R, C, start_width, _lib.ptr(lut), _lib.ptr(valid), cap, _lib.ptr(ws),
-                                       ws_bytes, ctypes.byref(n_levels), packs, rows, ctypes.byref(total),
+            rc = lib.bsp_sdd_lut_build(_lib.ptr(lay), H, R, C, start_width, _lib.ptr(lut), _lib.ptr(valid), cap, _lib.ptr(ctx.ws),
+                                       ctx.ws_bytes, ctypes.byref(n_levels), packs, rows, ctypes.byref(total),
                                        ctypes.byref(all_valid), _lib.stream_ptr(dev))
             if rc == _lib.ERR_CAPACITY and attempt == 0:
                 cap = int(total.value)
@@ -174,10 +245,11 @@ class _sparse_matmul(torch.autograd.Function):
             break
         luts, widths, out_packs = SddTables(), [], []
         luts.nnz = nnz
+        luts.spdims = tuple(layout.shape)
         if block in (16, 32, 64):
             luts.gplan = GroupPlan.build_coarse(layout, block, True, dev, for_sdd=True) if block == 16 else None
             if luts.gplan is None:
-                luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0)
+                luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0, ctx=ctx)
         done = 0
         for k in range(n_levels.value):
             p, r = int(packs[k]), int(rows[k])
@@ -201,6 +273,8 @@ class _sparse_matmul(torch.autograd.Function):
             raise ValueError('Reduction size for SDD must be a multiple of 16')
         if b.size(0) != AS0 or b.size(1) != a.size(1) or b.size(3 if trans_b else 2) != AS3:
             raise ValueError('incompatible operand shapes for sdd: %s and %s' % (tuple(a.shape), tuple(b.shape)))
+        _check_dense('a', a, spdims[0], block * spdims[1], None, trans_a)
+        _check_dense('b', b, spdims[0], None, block * spdims[2], trans_b)
         lib = _lib.load()
         total_width = luts.nnz if isinstance(luts, SddTables) else sum(w * p * p for w, p in zip(widths, packs))
         c = torch.empty((AS0, total_width, block, block), dtype=a.dtype, device=a.device)
@@ -212,7 +286,7 @@ class _sparse_matmul(torch.autograd.Function):
             rc = lib.bsp_sdd_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                     AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
                                     c.stride(0), block, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
-                                    gplan[0], gplan[1], gplan[2], _lib.stream_ptr(a.device))
+                                    gplan[0], gplan[1], gplan[2], KERNEL_FLAGS, _lib.stream_ptr(a.device))
             if rc == _lib.OK_WHOLE_LAYOUT:
                 break
             _lib.check(rc, 'bsp_sdd_matmul')
@@ -224,7 +298,7 @@ class _sparse_matmul(torch.autograd.Function):
     # DENSE = DENSE x SPARSE #
     ##########################
     @staticmethod
-    def make_dxx_lut(layout, block, step, trans, device, transform=lambda idx: idx):
+    def make_dxx_lut(layout, block, step, trans, device, transform=lambda idx: idx, ctx=None):
         """-> (lut, num_locks, width, None) as the reference (matmul.py:372-458); built on `device`.
 
         The table tensor carries `.plan`: per block, in table order, (position in the dense operand's reduction
@@ -232,11 +306,9 @@ class _sparse_matmul(torch.autograd.Function):
         `.planbuf`, the buffer the launchers take: the order in which they dispatch the segments, then `.plan`.
         """
         lib = _lib.load()
-        dev = torch.device(device)
-        lay = _lib.layout_to_device(layout, dev)
+        ctx = _LayoutOnDevice.of(layout, device, ctx)
+        dev, lay, nnz = ctx.device, ctx.lay, ctx.nnz
         H, R, C = lay.shape
-        ws, ws_bytes = _lib.workspace(lay, dev)
-        nnz = int((layout != 0).sum())
         cap = lib.bsp_dxx_lut_cap(H, R, C, nnz, block, step, int(bool(trans)))
         lut = torch.empty((cap,), dtype=torch.int32, device=dev)
         planbuf = torch.empty((lib.bsp_dxx_plan_cap(H, R, C, max(nnz, 1), int(bool(trans))),), dtype=torch.int32, device=dev)
@@ -244,7 +316,7 @@ class _sparse_matmul(torch.autograd.Function):
         width = ctypes.c_int(0)
         num_locks = ctypes.c_int(0)
         rc = lib.bsp_dxx_lut_build(_lib.ptr(lay), H, R, C, block, step, int(bool(trans)), _lib.ptr(lut), cap, _lib.ptr(planbuf),
-                                   _lib.ptr(ws), ws_bytes, ctypes.byref(n), ctypes.byref(width), ctypes.byref(num_locks),
+                                   _lib.ptr(ctx.ws), ctx.ws_bytes, ctypes.byref(n), ctypes.byref(width), ctypes.byref(num_locks),
                                    _lib.stream_ptr(dev))
         if rc == _lib.ERR_EMPTY_HEAD:
             raise RuntimeError('block-sparse layout has a head without any nonzero block')
@@ -253,10 +325,13 @@ class _sparse_matmul(torch.autograd.Function):
         first = lib.bsp_dxx_plan_pairs_offset(width.value)
         lut.planbuf = planbuf
         lut.plan = planbuf[first:first + 2 * nnz].view(nnz, 2)
+        lut.nnz = nnz
+        lut.spdims = tuple(layout.shape)
         lut.gplan = GroupPlan.build_coarse(layout, block, trans, dev) if block == 16 else None
         if lut.gplan is None and block in (16, 32, 64):
             lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block),
-                                        order_buckets=GroupPlan.order_buckets(layout, trans, block))
+                                        order_buckets=GroupPlan.order_buckets(layout, trans, block),
+                                        split_len=GroupPlan.SPLIT_LEN if block == 64 else 0, ctx=ctx)
         return lut, num_locks.value, width.value, None
 
     @staticmethod
@@ -271,6 +346,8 @@ class _sparse_matmul(torch.autograd.Function):
     @staticmethod
     def _dds_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, lut, num_locks, width, packs, bench, time):
         v = _vec(a.dtype)
+        _check_sparse('b', b, getattr(lut, 'nnz', None), block, a.size(0))
+        _check_dense('a', a, spdims[0], None, block * spdims[2 if trans_b else 1], trans_a)
         AS2 = a.size(3 if trans_a else 2)                     # free dimension M (matmul.py:467)
         a = _prep(_sparse_matmul._pad_free_dim(a, 3 if trans_a else 2, v))
         M = a.size(3 if trans_a else 2)
@@ -283,7 +360,8 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dds_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), a.size(0), M, a.stride(0), a.stride(1), a.stride(2), b_sz, c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
-                                        *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(a.device))
+                                        *GroupPlan.xsd_args(getattr(lut, 'gplan', None), M, a.size(0)), KERNEL_FLAGS,
+                                        _lib.stream_ptr(a.device))
         _lib.check(rc, 'bsp_dds_matmul')
         time[0] = timer.done()
         if M != AS2:
@@ -293,6 +371,8 @@ class _sparse_matmul(torch.autograd.Function):
     @staticmethod
     def _dsd_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, lut, num_locks, width, packs, bench, time):
         v = _vec(b.dtype)
+        _check_sparse('a', a, getattr(lut, 'nnz', None), block, b.size(0))
+        _check_dense('b', b, spdims[0], block * spdims[1 if trans_a else 2], None, trans_b)
         BS3 = b.size(2 if trans_b else 3)                     # free dimension N (matmul.py:518)
         b = _prep(_sparse_matmul._pad_free_dim(b, 2 if trans_b else 3, v))
         N = b.size(2 if trans_b else 3)
@@ -305,7 +385,8 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dsd_matmul(_lib.DTYPES[b.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), b.size(0), N, a_sz, b.stride(0), b.stride(1), b.stride(2), c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
-                                        *GroupPlan.args(getattr(lut, 'gplan', None)), _lib.stream_ptr(b.device))
+                                        *GroupPlan.xsd_args(getattr(lut, 'gplan', None), N, b.size(0)), KERNEL_FLAGS,
+                                        _lib.stream_ptr(b.device))
         _lib.check(rc, 'bsp_dsd_matmul')
         time[0] = timer.done()
         if N != BS3:
@@ -367,8 +448,9 @@ class MatMul:
             return self.lut_cache[key]
         layout, block = self.layout, self.block
         step = 8 if dtype == torch.float32 else 16             # matmul.py:617
-        sdd = lambda: _sparse_matmul.make_sdd_lut(layout, block, dtype, device)
-        dxx = lambda trans: _sparse_matmul.make_dxx_lut(layout, block, step, trans, device)
+        ctx = _LayoutOnDevice(layout, device)                  # one upload of the layout and one workspace for all tables
+        sdd = lambda: _sparse_matmul.make_sdd_lut(layout, block, dtype, device, ctx=ctx)
+        dxx = lambda trans: _sparse_matmul.make_dxx_lut(layout, block, step, trans, device, ctx=ctx)
         if self.mode == 'sdd':                                 # matmul.py:618-637
             c, da, db = sdd(), dxx(True), dxx(False)
         elif self.mode == 'dsd':

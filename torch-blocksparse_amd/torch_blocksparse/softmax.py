@@ -37,6 +37,25 @@ class _sparse_softmax(torch.autograd.Function):
             raise NotImplementedError('Reductions larger than 32768 elements are not yet implemented')
 
     @staticmethod
+    def _check_shapes(x, rpe, key_padding_mask, attn_mask, spdims, block, nnz):
+        """Operand extents against the layout.  The kernels take every address from the table (block id, block-row,
+        block-column, head), so a tensor that is too small would be read or written out of bounds on the device."""
+        H, R, C = spdims
+        if x.dim() != 4 or x.size(1) != nnz or tuple(x.shape[2:]) != (block, block):
+            raise ValueError('softmax input must be [batch, %d, %d, %d] for this layout, got %s' % (nnz, block, block, tuple(x.shape)))
+        Z = x.size(0)
+        if key_padding_mask is not None:
+            if key_padding_mask.dim() != 2 or key_padding_mask.size(0) not in (1, Z) or key_padding_mask.size(1) < C * block:
+                raise ValueError('key_padding_mask must be [%d or 1, >= %d], got %s' % (Z, C * block, tuple(key_padding_mask.shape)))
+        if attn_mask is not None:
+            if attn_mask.dim() != 2 or attn_mask.size(0) < R * block or attn_mask.size(1) < C * block:
+                raise ValueError('attn_mask must be at least [%d, %d], got %s' % (R * block, C * block, tuple(attn_mask.shape)))
+        if rpe is not None:
+            shape = (1,) * (4 - rpe.dim()) + tuple(rpe.shape)
+            if len(shape) != 4 or shape[0] not in (1, Z) or shape[1] not in (1, H) or shape[2] < R * block or shape[3] < C * block:
+                raise ValueError('rpe must broadcast to [%d, %d, >= %d, >= %d], got %s' % (Z, H, R * block, C * block, tuple(rpe.shape)))
+
+    @staticmethod
     def _strided16(t, what):
         """Masks are read with vector loads: unit inner stride, 16-byte aligned rows."""
         v = 4 if t.dtype == torch.float32 else 8
@@ -57,6 +76,7 @@ class _sparse_softmax(torch.autograd.Function):
         if not x.is_contiguous():
             raise ValueError('softmax works in place on a contiguous [Z, nnz, block, block] tensor')
         _sparse_softmax._check_rows(maxlut, block)
+        _sparse_softmax._check_shapes(x, rpe, key_padding_mask, attn_mask, spdims, block, (lut.numel() - 2 * spdims[0] * spdims[1]) // 4)
         null = ctypes.c_void_p(0)
         rpe_args = (null, 0, 0, 0)
         if rpe is not None:                                # element (z, h, r, c), softmax.py:50-55, 265
@@ -88,6 +108,8 @@ class _sparse_softmax(torch.autograd.Function):
     @staticmethod
     def backward(ctx, dx):
         x, lut = ctx.saved_tensors
+        if dx.shape != x.shape:
+            raise ValueError('softmax gradient has shape %s, the output has %s' % (tuple(dx.shape), tuple(x.shape)))
         dx = dx.contiguous()
         if dx.data_ptr() % 16 != 0:
             dx = dx.clone()
