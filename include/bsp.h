@@ -101,9 +101,9 @@ int bsp_sdd_lut_build(const int32_t *d_layout, int H, int R, int C, int start_wi
  * header row each (next to each other, in part order): the count field holds the part's entries in bits 0..19, the
  * part's index in bits 20..25 and the number of parts minus one in bits 26..30; bits 16..30 of the head field number
  * the split chains of the plan (fewer than 2^15, and fewer than 2^16 heads).  bsp_dsd_matmul / bsp_dds_matmul give
- * every part a workgroup of its own; the parts leave fp32 partial results in the launcher's workspace and the last
- * one to arrive adds them in part order (no floating-point atomics: the result does not depend on the arrival
- * order).  This is the role of the lock epilogue in the reference's kernel (matmul.py:191-203, 246-262).
+ * every part a workgroup of its own; the parts leave fp32 partial results in the launcher's workspace and a second
+ * pass adds them in part order (no atomics, no locks: the result does not depend on the order in which the parts
+ * ran).  This is the role of the lock epilogue in the reference's kernel (matmul.py:191-203, 246-262).
  * Pass 0 for plans given to bsp_sdd_matmul and for blocks of 32.
  * *n_groups counts header rows (groups, chains and parts of chains), *n_split the chains that were split.
  * plan_cap >= bsp_group_plan_cap(...). */
@@ -146,10 +146,10 @@ int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a
  * with trans = !trans_a; d_gplan (optional) from bsp_group_plan_build with by_rows = !trans_a; plan_lines < 0: a
  * plan over tiles (see bsp_group_plan_build).
  * n_split / d_ws / ws_bytes: a plan with split chains (n_split of them, as bsp_group_plan_build reported) needs
- * scratch memory of at least bsp_xsd_workspace_bytes(n_split, N, Z) bytes, 256-byte aligned: one int32 counter per
- * (split chain, 64-wide tile of the free dimension, batch) followed by BSP_CHAIN_PARTS fp32 tiles of 64 x 64 each.
- * The counters must be zero when the launch starts; every launch leaves them zero, so clearing the buffer once after
- * allocating it is enough.  Launches that share a buffer must not overlap (one stream, or one buffer per stream).
+ * scratch memory of at least bsp_xsd_workspace_bytes(n_split, N, Z) bytes, 256-byte aligned: BSP_CHAIN_PARTS fp32
+ * tiles of 64 x 64 per (split chain, 64-wide tile of the free dimension, batch).  Its contents need no
+ * initialisation and mean nothing after the call; a second small kernel launched behind the product adds the parts
+ * up.  Launches that share a buffer must not overlap (one stream, or one buffer per stream).
  * 0 / NULL / 0 for plans without split chains. */
 int64_t bsp_xsd_workspace_bytes(int n_split, int free_dim, int Z);
 int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,

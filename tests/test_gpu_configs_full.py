@@ -119,9 +119,9 @@ def test_config5_sparse_linear_layer_full_size():
 @pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
 def test_block64_chains_of_hundreds_of_blocks_split_over_workgroups(dtype):
     # Lines of 264 and 600 blocks of 64: chains cut into 5 and 8 parts, each part a workgroup of its own that leaves an
-    # fp32 partial tile in the operator's workspace; the last part to arrive adds them up.  Tall layouts give the chains
+    # fp32 partial tile in the operator's workspace; a second pass adds them up in part order.  Tall layouts give the chains
     # to the transposed product (block-columns are the lines), their transposes to the plain one; free dimension of one
-    # and of two 64-wide tiles; Z = 3; every product runs twice (the counters must return to zero).
+    # and of two 64-wide tiles; Z = 3; every product runs twice.
     from torch_blocksparse.matmul import GroupPlan
     for n, others in ((264, 7), (600, 3)):
         tall = random_layout((2, n, 1 + others), 0.15, n)
@@ -138,9 +138,8 @@ def test_block64_chains_of_hundreds_of_blocks_split_over_workgroups(dtype):
                          dist='randn', scale=0.1)
         run_case('dds', False, False, 64, dtype, Z=2, H=2, M=64, K=n * 64, N=(1 + others) * 64, layout=tall, seed=n + 2, dist='randn',
                  scale=0.1)
-        # one operator called again and again: its workspace is reused, so the counters must be back at zero after
-        # every launch, also when a launch with fewer tiles follows one with more; the parts are added in a fixed order,
-        # so repeated launches agree bit for bit
+        # one operator called again and again: its workspace is reused, also by a launch with fewer tiles after one with
+        # more; the parts are added in a fixed order, so repeated launches agree bit for bit
         op = tb.MatMul(tall, 64, 'dsd', trans_a=True)
         g = torch.Generator().manual_seed(n)
         a = (0.1 * torch.randn(3, int(tall.sum()), 64, 64, generator=g)).to(dtype).to(DEV)

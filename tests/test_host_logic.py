@@ -154,5 +154,5 @@ def test_operand_shapes_are_checked_against_the_layout_before_any_launch():
 def test_workspace_size_of_split_chains():
     lib = _lib.load()
     assert lib.bsp_xsd_workspace_bytes(0, 64, 8) == 0
-    # 3 split chains x 2 tiles x 2 batches = 12 counters (rounded up to 64 ints) + 12 x 8 fp32 tiles of 64 x 64
-    assert lib.bsp_xsd_workspace_bytes(3, 128, 2) == 64 * 4 + 12 * 8 * 64 * 64 * 4
+    # 3 split chains x 2 tiles x 2 batches = 12 slots of 8 fp32 tiles of 64 x 64
+    assert lib.bsp_xsd_workspace_bytes(3, 128, 2) == 12 * 8 * 64 * 64 * 4

@@ -64,27 +64,23 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   return BSP_OK;
 }
 
-// Workspace of a plan with split chains: counters (one per (split chain, free tile, batch), rounded up to a multiple of
-// 64) followed by BSP_CHAIN_PARTS fp32 tiles per counter.
+// Workspace of a plan with split chains: BSP_CHAIN_PARTS fp32 tiles of 64 x 64 per (split chain, free tile, batch).
 static int64_t xsd_ws_slots(int n_split, int free_dim, int Z) { return (int64_t)n_split * ((free_dim + 63) / 64) * Z; }
-static int64_t xsd_ws_counter_ints(int64_t slots) { return (slots + 63) & ~(int64_t)63; }
 
 extern "C" int64_t bsp_xsd_workspace_bytes(int n_split, int free_dim, int Z) {
   if (n_split <= 0 || free_dim <= 0 || Z <= 0) return 0;
-  const int64_t slots = xsd_ws_slots(n_split, free_dim, Z);
-  return 4 * xsd_ws_counter_ints(slots) + slots * BSP_CHAIN_PARTS * (int64_t)(64 * 64 * sizeof(float));
+  return xsd_ws_slots(n_split, free_dim, Z) * BSP_CHAIN_PARTS * (int64_t)(64 * 64 * sizeof(float));
 }
 
-// Fills in the workspace fields of the arguments; the plan is dropped when it has split chains and no workspace came.
+// Fills in the workspace fields of the arguments.
 static int xsd_workspace(XsdArgs &g, int n_split, int free_dim, void *d_ws, int64_t ws_bytes) {
-  g.n_split = 0; g.counters = nullptr; g.partials = nullptr;
+  g.n_split = 0; g.partials = nullptr;
   if (n_split < 0) return BSP_ERR_ARG;
   if (!g.gplan || n_split == 0) return BSP_OK;
   if (!d_ws || (reinterpret_cast<uintptr_t>(d_ws) & 255)) return BSP_ERR_ARG;
   if (ws_bytes < bsp_xsd_workspace_bytes(n_split, free_dim, g.Z)) return BSP_ERR_CAPACITY;
   g.n_split = n_split;
-  g.counters = reinterpret_cast<int32_t *>(d_ws);
-  g.partials = reinterpret_cast<float *>(g.counters + xsd_ws_counter_ints(xsd_ws_slots(n_split, free_dim, g.Z)));
+  g.partials = reinterpret_cast<float *>(d_ws);
   return BSP_OK;
 }
 

@@ -539,38 +539,46 @@ __device__ __forceinline__ void xsd_chain(const XsdArgs &g, T *smem, int z, int 
   }
   __syncthreads();
   if (parts > 1) {
-    // One part of a split chain.  Its sums go to the workspace as fp32; the part that arrives last (a counter per
-    // chain, tile and batch, stepped with an integer atomic after a release fence) reads all parts back and adds them
-    // in part order, so the result does not depend on which part was last.  The counter returns to zero.
+    // One part of a split chain: its sums go to the workspace as fp32, 16 bytes per lane in address order;
+    // k_xsd_chain_sum, launched behind this kernel, adds the parts in part order and writes the line.
     const int64_t slot = ((int64_t)seq * g.n_tiles + n0 / 64) * g.Z + z;
-    f32x4 *ws = reinterpret_cast<f32x4 *>(g.partials) + (slot * BSP_CHAIN_PARTS) * 1024;   // 1024 f32x4 = one 64 x 64 tile
+    f32x4 *ws = reinterpret_cast<f32x4 *>(g.partials) + (slot * BSP_CHAIN_PARTS + part) * 1024;   // 1024 f32x4 = one 64 x 64 tile
 #pragma unroll
-    for (int j = 0; j < 4; j++) ws[((int64_t)part * 4 + wave) * 256 + j * 64 + lane] = fin[j];
-    __threadfence();                                 // the tile is visible device-wide before the counter moves
-    __syncthreads();
-    int *flag = reinterpret_cast<int *>(smem);
-    if (threadIdx.x == 0) {
-      const int seen = atomicAdd(g.counters + slot, 1);
-      if (seen == parts - 1) g.counters[slot] = 0;   // nobody else touches this counter until the next launch
-      *flag = seen;
-    }
-    __syncthreads();
-    const bool last = *flag == parts - 1;
-    __syncthreads();                                 // the flag's LDS word is staging space again below
-    if (!last) return;
-    __threadfence();                                 // read the other parts' tiles only after seeing their counter steps
-#pragma unroll
-    for (int j = 0; j < 4; j++) fin[j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int p = 0; p < parts; p++) {
-#pragma unroll
-      for (int j = 0; j < 4; j++) {
-        const f32x4 v = ws[((int64_t)p * 4 + wave) * 256 + j * 64 + lane];
-        fin[j] += v;
-      }
-    }
+    for (int j = 0; j < 4; j++) ws[(wave * 4 + j) * 64 + lane] = fin[j];
+    return;
   }
   T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + n0;
   store_slice<T, true>(smem + (wave * 16) * kLdsRow, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, fin, lane);
+}
+
+// Second pass over the split chains of a plan: one workgroup per (header row, tile of the free dimension, batch); the
+// rows that are part 0 of a split chain add the chain's partial tiles in part order and write the output line, all
+// others leave at once.  A kernel of its own rather than a last-arriver epilogue: the kernel boundary orders the
+// partial sums before their use without device-wide fences inside the product kernel (which cost more than this
+// launch: a release fence writes the whole L2 of its XCD back), and the sum has one fixed order.
+template <typename T>
+__global__ void __launch_bounds__(256) k_xsd_chain_sum(XsdArgs g) {
+  __shared__ __attribute__((aligned(16))) T stage[4 * 16 * kLdsRow];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int z = blockIdx.x % g.Z;
+  const int64_t rest = blockIdx.x / g.Z;
+  const int tile = (int)(rest % g.n_tiles);
+  const table_ptr hd = as_table(g.gplan) + 4 * (rest / g.n_tiles);
+  const int cnt = hd[1], code = hd[3];
+  const int part = (cnt >> 20) & 63, parts = ((cnt >> 26) & 31) + 1;
+  if (code >= 0 || parts == 1 || part != 0) return;
+  const int depth = hd[2] & 0xffff, seq = hd[2] >> 16, line = -(code + 1);
+  const int64_t slot = ((int64_t)seq * g.n_tiles + tile) * g.Z + z;
+  const f32x4 *ws = reinterpret_cast<const f32x4 *>(g.partials) + (slot * BSP_CHAIN_PARTS) * 1024;
+  f32x4 fin[4];
+#pragma unroll
+  for (int j = 0; j < 4; j++) fin[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < parts; p++) {
+#pragma unroll
+    for (int j = 0; j < 4; j++) fin[j] += __builtin_nontemporal_load(ws + (int64_t)p * 1024 + (wave * 4 + j) * 64 + lane);
+  }
+  T *po = reinterpret_cast<T *>(g.out) + z * g.out_sz + depth * g.out_sh + tile * 64;
+  store_slice<T, true>(stage + (wave * 16) * kLdsRow, po + ((int64_t)line * 64 + wave * 16) * g.ldo, g.ldo, fin, lane);
 }
 
 // dsd / dds: members = output lines (block-rows of the result), entries = positions of the reduction
@@ -1201,6 +1209,7 @@ template <typename T> int xsd_fast_t(const XsdArgs &g, bool sp_trans, hipStream_
     if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
     if (sp_trans) hipLaunchKernelGGL((k_xsd64_rg<T, true>), dim3((unsigned)n), dim3(256), 0, st, g);
     else hipLaunchKernelGGL((k_xsd64_rg<T, false>), dim3((unsigned)n), dim3(256), 0, st, g);
+    if (g.n_split > 0) hipLaunchKernelGGL((k_xsd_chain_sum<T>), dim3((unsigned)n), dim3(256), 0, st, g);
     return BSP_OK;
   }
   const int64_t n_wg = (int64_t)g.width * g.n_tiles * g.Z;
@@ -1250,6 +1259,7 @@ template <typename T, int SUBS> int xsd_coarse_t(const XsdArgs &g, bool sp_trans
   if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   if (sp_trans) hipLaunchKernelGGL((k_xsd64_rg<T, true, SUBS>), dim3((unsigned)n), dim3(256), 0, st, g);
   else hipLaunchKernelGGL((k_xsd64_rg<T, false, SUBS>), dim3((unsigned)n), dim3(256), 0, st, g);
+  if (g.n_split > 0) hipLaunchKernelGGL((k_xsd_chain_sum<T>), dim3((unsigned)n), dim3(256), 0, st, g);
   return BSP_OK;
 }
 int xsd_fast64(int dtype, const XsdArgs &g0, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {

@@ -461,8 +461,8 @@ struct XsdArgs {
   const int32_t *order;                 // order[p] = segment dispatched p-th (head by head, longest first inside a head), or null
   int n_tiles;                          // 64-wide tiles of the free dimension (specialised kernels)
   const int32_t *gplan; int n_pgroups; int lines;   // optional group plan, its groups, lines (block-rows or -columns) per head
-  int n_split = 0;                      // split chains of the plan; their counters and fp32 partial tiles (caller's workspace)
-  int32_t *counters = nullptr; float *partials = nullptr;
+  int n_split = 0;                      // split chains of the plan; their fp32 partial tiles (caller's workspace)
+  float *partials = nullptr;
 };
 
 // A reduction step of TK elements lies inside one block (BLOCK >= TK) or covers TK / BLOCK whole blocks.

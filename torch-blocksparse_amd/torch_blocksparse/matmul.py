@@ -149,14 +149,13 @@ class GroupPlan:
 
     def workspace(self, free_dim, Z):
         """(pointer, bytes) of the scratch buffer the split chains of this plan need for a launch with this free dimension
-        and batch: counters + fp32 partial tiles, zeroed when allocated (every launch leaves the counters zero) and
-        kept for the next call; (NULL, 0) for a plan without split chains.  One buffer per plan: launches of one
-        operator are assumed to be ordered on one stream."""
+        and batch (fp32 partial tiles; kept for the next call, contents never matter); (NULL, 0) for a plan without
+        split chains.  One buffer per plan: launches of one operator are assumed to be ordered on one stream."""
         if self.n_split == 0:
             return ctypes.c_void_p(0), 0
         need = _lib.load().bsp_xsd_workspace_bytes(self.n_split, int(free_dim), int(Z))
         if self._ws is None or self._ws.numel() < need:
-            self._ws = torch.zeros(need, dtype=torch.uint8, device=self.table.device)
+            self._ws = torch.empty(need, dtype=torch.uint8, device=self.table.device)
         return _lib.ptr(self._ws), self._ws.numel()
 
     @staticmethod
