@@ -31,7 +31,8 @@ typedef enum {
   BSP_ERR_EMPTY_HEAD = -4,   /* a head of the layout has no nonzero block (the reference raises here) */
   BSP_ERR_HIP = -5,          /* a HIP runtime call failed */
   BSP_ERR_ROW_TOO_LONG = -6, /* softmax row of >= 32768 elements (reference softmax.py:225-227) */
-  BSP_ERR_K_MULTIPLE = -7    /* sdd reduction size not a multiple of 16 (reference matmul.py:318-319) */
+  BSP_ERR_K_MULTIPLE = -7,   /* sdd reduction size not a multiple of 16 (reference matmul.py:318-319) */
+  BSP_ERR_SCRATCH_LIMIT = -8 /* bsp_dsd_matmul_noalloc: the launch needs more scratch than the library's static buffer holds */
 } bsp_status;
 
 int bsp_version(void);
@@ -157,6 +158,24 @@ int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a
                    int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
                    const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
                    int n_split, void *d_ws, int64_t ws_bytes, int flags, void *stream);
+
+/* bsp_dsd_matmul for callers that cannot allocate.  No counterpart in the reference: it is for code under HIP graph
+ * capture, tight serving loops and harnesses that forbid hipMalloc, which have nowhere to take the workspace of a plan
+ * with split chains from.  Same arguments and results as bsp_dsd_matmul without d_ws / ws_bytes: the fp32 partial
+ * tiles live in a buffer inside the library (static device memory, BSP_NOALLOC_SCRATCH_BYTES per GPU the library
+ * runs on, held until the process ends).  It serves launches with at most BSP_NOALLOC_MAX_SLOTS =
+ * n_split * ceil(N / 64) * Z (split chain, tile, batch) combinations and returns BSP_ERR_SCRATCH_LIMIT beyond that,
+ * before anything is launched.  The call allocates and frees nothing (the first call on a device looks the buffer's address up
+ * once; make that call outside a capture).  Every call on a GPU uses that GPU's one buffer: calls that overlap on one
+ * GPU (two streams, two threads) race; calls ordered on one stream do not.  Nothing in the buffer has to start at
+ * zero: every tile a call reads it has written before. */
+#define BSP_NOALLOC_MAX_SLOTS 64
+#define BSP_NOALLOC_SCRATCH_BYTES (BSP_NOALLOC_MAX_SLOTS * BSP_CHAIN_PARTS * 64 * 64 * 4)
+int bsp_dsd_matmul_noalloc(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                           int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
+                           int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                           const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups, int plan_lines,
+                           int n_split, int flags, void *stream);
 
 /* dense = dense x sparse: replaces _sparse_matmul._dds_matmul + the DDS branch (matmul.py:460-505, 83-99).
  * C[z, h] = op(A)[z, h] . op(B_sparse)[h], written transposed when trans_c.  M = free dimension of op(A).

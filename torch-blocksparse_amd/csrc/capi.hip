@@ -1,6 +1,7 @@
 // C-ABI entry points of the matmul launchers: argument validation and dispatch.  (The table builders and
 // the softmax entry points live next to their kernels in lut.hip / softmax.hip.)
 #include "matmul_generic.h"
+#include <mutex>
 
 using namespace bsp;
 
@@ -25,6 +26,7 @@ extern "C" const char *bsp_strerror(int status) {
     case BSP_ERR_HIP: return "HIP runtime error";
     case BSP_ERR_ROW_TOO_LONG: return "Reductions larger than 32768 elements are not yet implemented";
     case BSP_ERR_K_MULTIPLE: return "Reduction size for SDD must be a multiple of 16";
+    case BSP_ERR_SCRATCH_LIMIT: return "the launch needs more (split chain, tile, batch) slots than the library's static scratch buffer holds; use bsp_dsd_matmul with a workspace";
     default: return "unknown status";
   }
 }
@@ -123,6 +125,54 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
   // rows of the kernel = rows of op(A); op(A)(m,k) is stored [k][m] when trans_a.  Dense (n,k) = op(B)[k][n]:
   // reduction contiguous when B is read transposed.  C[m][n] has n contiguous unless written transposed.
   return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, flags, stream);
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// The allocation-free variant of bsp_dsd_matmul: the workspace of the split chains is a static device array.
+// In host code the array's name only stands for the symbol; its device address differs from GPU to GPU and is looked
+// up once per device with hipGetSymbolAddress, with that device current, and kept.  Everything below uses that
+// address, never the name.
+// ---------------------------------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[BSP_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[kMaxDevices] = {};   // per device: the address of its copy of `scratch`
+
+// the device address of `scratch` on the current device (nullptr on failure)
+void *scratch_address() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return nullptr;
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int bsp_dsd_matmul_noalloc(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,
+                                      int N, int64_t a_stride_z, int64_t b_stride_z, int64_t b_stride_h, int64_t ldb,
+                                      int64_t c_stride_z, int64_t c_stride_h, int64_t ldc, int block, const int32_t *d_lut,
+                                      const int32_t *d_plan, int width, const int32_t *d_gplan, int n_plan_groups,
+                                      int plan_lines, int n_split, int flags, void *stream) {
+  if (n_split < 0 || Z <= 0 || N <= 0) return BSP_ERR_ARG;
+  void *ws = nullptr;
+  int64_t ws_bytes = 0;
+  if (d_gplan && n_split > 0) {
+    if (xsd_ws_slots(n_split, N, Z) > BSP_NOALLOC_MAX_SLOTS) return BSP_ERR_SCRATCH_LIMIT;
+    ws = scratch_address();
+    if (!ws) return BSP_ERR_HIP;
+    ws_bytes = BSP_NOALLOC_SCRATCH_BYTES;
+    // (the buffer keeps what the last call left, which is harmless: every tile that is read was written by this call)
+  }
+  return bsp_dsd_matmul(dtype, a, b, c, trans_a, trans_b, trans_c, Z, N, a_stride_z, b_stride_z, b_stride_h, ldb, c_stride_z,
+                        c_stride_h, ldc, block, d_lut, d_plan, width, d_gplan, n_plan_groups, plan_lines, n_split, ws, ws_bytes,
+                        flags, stream);
 }
 
 extern "C" int bsp_dds_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int trans_c, int Z,

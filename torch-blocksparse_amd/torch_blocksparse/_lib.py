@@ -23,6 +23,7 @@ ERR_CAPACITY = -3
 ERR_EMPTY_HEAD = -4
 ERR_ROW_TOO_LONG = -6
 ERR_K_MULTIPLE = -7
+ERR_SCRATCH_LIMIT = -8
 
 _c = ctypes
 _vp, _i, _i64, _f = _c.c_void_p, _c.c_int, _c.c_int64, _c.c_float
@@ -47,6 +48,8 @@ SIGNATURES = {
                             _i64, _vp, _i, _i, _i, _vp]),
     'bsp_dsd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
                             _i, _vp, _i, _i, _i, _vp, _i64, _i, _vp]),
+    'bsp_dsd_matmul_noalloc': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
+                                    _i, _vp, _i, _i, _i, _i, _vp]),
     'bsp_dds_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
                             _i, _vp, _i, _i, _i, _vp, _i64, _i, _vp]),
     'bsp_softmax_fwd': (_i, [_i, _vp, _f, _vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _i, _vp, _i64, _i, _i, _i, _i, _i,
