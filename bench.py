@@ -442,9 +442,10 @@ def calibrate(args):
         for b in bufs:
             b.zero_()
         for mode in range(5):
-            ms = timed(lambda: probe.bsp_probe_stream(mode, _lib.ptr(bufs[0]), _lib.ptr(bufs[1]), _lib.ptr(bufs[2]), nbytes, 256 * 16, stream))
-            res['probes'].append({'probe': names[mode], 'footprint': label, 'ms': round(ms, 4),
-                                  'GB/s': round(moved[mode] * nbytes / ms * 1e-6, 1)})
+            for groups in (256 * 8, 256 * 32):
+                ms = timed(lambda: probe.bsp_probe_stream(mode, _lib.ptr(bufs[0]), _lib.ptr(bufs[1]), _lib.ptr(bufs[2]), nbytes, groups, stream))
+                res['probes'].append({'probe': names[mode], 'footprint': label, 'workgroups': groups, 'ms': round(ms, 4),
+                                      'GB/s': round(moved[mode] * nbytes / ms * 1e-6, 1)})
         del bufs
         torch.cuda.empty_cache()
     w = Attention(8, 64)

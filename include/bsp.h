@@ -204,6 +204,24 @@ int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int m
 int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
                     int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream);
 
+/* Softmax with dropout on its result.  No counterpart in the reference, whose attention module refuses dropout
+ * (attention.py:223-224); this is what nn.MultiheadAttention's dropout on the attention weights needs.
+ * Forward: x receives softmax(...) as bsp_softmax_fwd would leave it (the backward pass needs it), y_drop (same shape,
+ * own batch stride) receives softmax(...) * mask / (1 - p).  The mask is not stored: element i (its linear offset in
+ * x: z * x_stride_z + blockid * block^2 + row * block + col) is kept iff (w >> 8) * 2^-24 >= p, where w is word
+ * i % 4 of Philox4x32-10 with counter (i / 4 as two 32-bit words, offset as two 32-bit words) and key seed.
+ * Backward: dy holds the gradient of y_drop and is overwritten with the gradient of the softmax input,
+ * y * (dy * mask / (1 - p) - sum(...)) * scale, the mask re-created from the same (seed, offset); y is x as the forward
+ * call left it and y_stride_z the x_stride_z of that call.  0 <= p < 1. */
+int bsp_softmax_dropout_fwd(int dtype, void *x, void *y_drop, float scale, const int32_t *d_lut, int maxlut, const void *rpe,
+                            int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm,
+                            int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r, int attn_mul, int Z,
+                            int H, int R, int block, int64_t x_stride_z, int64_t y_drop_stride_z, float drop_p, uint64_t seed,
+                            uint64_t offset, void *stream);
+int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
+                            int R, int block, int64_t y_stride_z, int64_t dy_stride_z, float drop_p, uint64_t seed,
+                            uint64_t offset, void *stream);
+
 /* ---------------------------------------------------------------------------------------------------
  * Dense utility ops of the reference package.
  * ReLU: replaces the relu_y / relu_dxdsdbdres kernels and their launches (relu.py:8-91).  All tensors hold n

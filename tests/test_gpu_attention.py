@@ -251,3 +251,31 @@ def test_extra_key_position_is_refused():
     for kw in (dict(add_bias_kv=True), dict(add_zero_attn=True)):
         with pytest.raises(NotImplementedError):
             tb.MultiheadAttention(64, 2, lay, 16, **kw)
+
+
+def test_multihead_attention_with_dropout():
+    # dropout on the attention weights: active in training mode only, scaled so that the expectation is unchanged
+    torch.manual_seed(31)
+    E, heads, L, B, block = 64, 2, 128, 4, 32
+    lay = torch.ones(heads, L // block, L // block, dtype=torch.int64)
+    mha = tb.MultiheadAttention(E, heads, lay, block, dropout=0.5).to(DEV).half()
+    x = torch.randn(L, B, E, device=DEV, dtype=torch.float16)
+    mha.eval()
+    ref, _ = mha(x, x, x)
+    assert torch.equal(ref, mha(x, x, x)[0])
+    mha.train()
+    torch.manual_seed(1)
+    a, _ = mha(x, x, x)
+    torch.manual_seed(1)
+    b, _ = mha(x, x, x)
+    c, _ = mha(x, x, x)
+    assert torch.equal(a, b) and not torch.equal(a, c) and not torch.equal(a, ref)
+    # the mean over many masks approaches the result without dropout
+    acc = torch.zeros_like(ref, dtype=torch.float32)
+    n = 200
+    for _ in range(n):
+        acc += mha(x, x, x)[0].float()
+    err = (acc / n - ref.float()).abs().mean() / ref.float().abs().mean()
+    assert err < 0.15, err
+    a.sum().backward()
+    assert torch.isfinite(mha.in_proj_weight.grad).all()

@@ -124,3 +124,66 @@ def test_in_place_and_row_too_long():
     big = torch.ones(1, 1, 512, dtype=torch.int64)
     with pytest.raises(NotImplementedError):
         tb.Softmax(big, 64)(torch.zeros(1, 512, 64, 64, dtype=torch.float16, device=DEV))
+
+
+def run_dropout_case(Z, H, R, C, block, dtype, density, seed, p, masks=False, layout=None):
+    # forward and backward with dropout against the oracle with the mask re-created from the same counter
+    from oracle.philox_oracle import keep_mask
+    torch.manual_seed(seed)
+    lay = layout if layout is not None else random_layout((H, R, C), density, seed, at_least_one_per_row=True)
+    nnz = int(lay.sum())
+    x = torch.rand((Z, nnz, block, block)).to(dtype)
+    dy = torch.rand((Z, nnz, block, block)).to(dtype)
+    kw = {}
+    if masks:
+        kw['rpe'] = (0.5 * torch.randn(Z, H, R * block, C * block)).to(dtype)
+        kw['attn_mask'] = torch.randn(R * block, C * block).to(dtype)
+    drop_seed, drop_off = 0x1234567 + seed, 3 * seed
+    keep = torch.from_numpy(keep_mask(x.numel(), p, drop_seed, drop_off)).reshape(x.shape)
+    m = keep.float() / (1.0 - p)
+    ry, rdx = D.softmax(x, lay, block, scale=0.4, dy=dy.float() * m, **kw)
+    xg = x.to(DEV).requires_grad_(True)
+    xin = xg * 1.0
+    y = tb.Softmax(lay, block)(xin, scale=0.4, dropout_p=p, dropout_seed=drop_seed, dropout_offset=drop_off,
+                               **{k: v.to(DEV) for k, v in kw.items()})
+    assert y.data_ptr() != xin.data_ptr()
+    assert_close(xin, ry, dtype, 'softmax kept for the backward pass')
+    assert_close(y, ry * m, dtype, 'dropped softmax')
+    assert torch.equal(y.cpu() == 0, ~keep | (ry == 0)), 'mask differs from the oracle\'s'
+    y.backward(dy.to(DEV))
+    assert_close(xg.grad, rdx, dtype, 'softmax + dropout dx')
+
+
+@pytest.mark.parametrize('block', [16, 32, 64, 128])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+def test_dropout_matches_the_counter_based_oracle(block, dtype):
+    run_dropout_case(2, 2, 5, 6, block, dtype, 0.5, block, 0.3)
+    run_dropout_case(1, 2, 3, 4, block, dtype, 0.7, block + 1, 0.1, masks=True)
+
+
+def test_dropout_in_every_kernel_variant():
+    # long rows: the 32-block bucket (block 16), the streaming variant (more blocks than registers hold), 16-block bucket
+    for block, cols, dtype in ((16, 28, torch.float16), (64, 20, torch.float16), (32, 14, torch.bfloat16), (16, 70, torch.float32)):
+        run_dropout_case(2, 1, 2, cols, block, dtype, 0.95, cols, 0.25)
+        run_dropout_case(1, 1, 2, cols, block, dtype, 0.95, cols + 1, 0.5, masks=True)
+
+
+def test_dropout_rate_and_repeatability():
+    lay = tb.sparse_transformer_layout(2, 16, 4, 8, True)
+    nnz = int(lay.sum())
+    x = torch.randn(4, nnz, 64, 64, dtype=torch.float16, device=DEV)
+    sm = tb.Softmax(lay, 64)
+    for p in (0.1, 0.5):
+        y = sm(x.clone(), dropout_p=p, dropout_seed=99)
+        kept = (y != 0).float().mean().item()
+        n = y.numel()
+        assert abs(kept - (1 - p)) < 5 * (p * (1 - p) / n) ** 0.5 + 1e-4      # (softmax values that round to 0 in fp16 are rare)
+        assert torch.equal(y, sm(x.clone(), dropout_p=p, dropout_seed=99))
+        assert not torch.equal(y, sm(x.clone(), dropout_p=p, dropout_seed=100))
+        assert not torch.equal(y, sm(x.clone(), dropout_p=p, dropout_seed=99, dropout_offset=1))
+    torch.manual_seed(5)
+    a = sm(x.clone(), dropout_p=0.2)
+    torch.manual_seed(5)
+    b = sm(x.clone(), dropout_p=0.2)
+    assert torch.equal(a, b)                               # the seed comes from torch's generator when not given
+    assert torch.equal(sm(x.clone(), dropout_p=0.0), sm(x.clone()))

@@ -44,9 +44,11 @@ def test_constructor_errors():
     with pytest.raises(NotImplementedError):
         tb.SparsityConfig(attention='causal')
     with pytest.raises(NotImplementedError):
-        tb.MultiheadAttention(32, 2, lay, 16, dropout=0.1)
+        tb.MultiheadAttention(32, 2, lay, 16, add_zero_attn=True)
     with pytest.raises(ValueError):
         tb.Softmax(lay, 16)(torch.zeros(1, 4, 16, 16, dtype=torch.float16), attn_mask=torch.zeros(32, 32))
+    with pytest.raises(ValueError):
+        tb.Softmax(lay, 16)(torch.zeros(1, 4, 16, 16, dtype=torch.float16), dropout_p=1.0)
     with pytest.raises(ValueError):
         tb.fixed_layout(2, 16, 'fixed', 4, 'unidirectional', 1, 3)
     with pytest.raises(ValueError):

@@ -175,3 +175,22 @@ def test_against_compiled_reference(seed):
     nb = 4 * int(torch.randint(1, 6, (1,), generator=g))
     for uni in (True, False):
         assert (O.make_layout_cpp(3, nb, 'fixed', 4, uni, 2, 1) == ref.make_layout(3, nb, 'fixed', 4, uni, 2, 1).numpy()).all()
+
+
+def test_philox_known_answers():
+    # Random123's published known-answer vectors for philox4x32-10 (counter, key -> output); they pin the generator
+    # behind the dropout mask of the softmax
+    from oracle.philox_oracle import philox4x32_10, keep_mask
+    kats = [((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+            ((0xffffffff,) * 4, (0xffffffff, 0xffffffff), (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+            ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0), (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1))]
+    for ctr, key, want in kats:
+        got = philox4x32_10(*[np.array([c], dtype=np.uint64) for c in ctr], *key)
+        assert tuple(int(g[0]) for g in got) == want
+    # vectorised evaluation = one counter at a time; the mask takes word i % 4 of counter i / 4
+    m = keep_mask(1000, 0.25, seed=0x299f31d0a4093822, offset=7)
+    w = philox4x32_10(np.array([3], dtype=np.uint64), np.array([0]), 7, 0, 0xa4093822, 0x299f31d0)
+    assert [bool(x) for x in m[12:16]] == [((int(v[0]) >> 8) * 2.0 ** -24) >= 0.25 for v in w]
+    big = keep_mask(1 << 20, 0.25, seed=12345)
+    assert abs(big.mean() - 0.75) < 4 * (0.25 * 0.75 / (1 << 20)) ** 0.5
+    assert keep_mask(64, 0.0, seed=1).all()

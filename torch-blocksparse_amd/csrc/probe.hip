@@ -10,33 +10,64 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 namespace {
 constexpr int kThreads = 256;
 
+// Every lane keeps U independent 16-byte accesses in flight per round (a workgroup walks U * 4 KiB of consecutive
+// addresses per round), as the operator kernels do with their prefetch rings.
+constexpr int U = 8;
+
 // mode 0: read only (the xor of everything read is written by one lane that can never exist, so that the loads stay)
 __global__ void __launch_bounds__(kThreads) k_probe_read(const u32x4 *src, u32x4 *sink, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
+  const int64_t stride = (int64_t)gridDim.x * kThreads * U;
   u32x4 acc = {0u, 0u, 0u, 0u};
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) acc ^= src[i];
+  for (int64_t i = (int64_t)blockIdx.x * kThreads * U + threadIdx.x; i < n; i += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = src[i + u * kThreads < n ? i + u * kThreads : i];
+#pragma unroll
+    for (int u = 0; u < U; u++) acc ^= v[u];
+  }
   if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && n < 0) sink[0] = acc;
 }
 // mode 1: write only
 __global__ void __launch_bounds__(kThreads) k_probe_write(u32x4 *dst, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) dst[i] = u32x4{(uint32_t)i, 1u, 2u, 3u};
+  const int64_t stride = (int64_t)gridDim.x * kThreads * U;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads * U + threadIdx.x; i < n; i += stride) {
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (i + u * kThreads < n) dst[i + u * kThreads] = u32x4{(uint32_t)i, 1u, 2u, 3u};
+  }
 }
 // mode 2: copy (1 read : 1 write); mode 3: in place (read, modify, write back); mode 4: 1 read : 2 writes
 __global__ void __launch_bounds__(kThreads) k_probe_copy(const u32x4 *src, u32x4 *dst, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) dst[i] = src[i];
+  const int64_t stride = (int64_t)gridDim.x * kThreads * U;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads * U + threadIdx.x; i < n; i += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = src[i + u * kThreads < n ? i + u * kThreads : i];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (i + u * kThreads < n) dst[i + u * kThreads] = v[u];
+  }
 }
 __global__ void __launch_bounds__(kThreads) k_probe_inplace(u32x4 *buf, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) buf[i] = buf[i] + 1u;
+  const int64_t stride = (int64_t)gridDim.x * kThreads * U;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads * U + threadIdx.x; i < n; i += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = buf[i + u * kThreads < n ? i + u * kThreads : i];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (i + u * kThreads < n) buf[i + u * kThreads] = v[u] + 1u;
+  }
 }
 __global__ void __launch_bounds__(kThreads) k_probe_r1w2(const u32x4 *src, u32x4 *dst0, u32x4 *dst1, int64_t n) {
-  const int64_t stride = (int64_t)gridDim.x * kThreads;
-  for (int64_t i = (int64_t)blockIdx.x * kThreads + threadIdx.x; i < n; i += stride) {
-    const u32x4 v = src[i];
-    dst0[i] = v;
-    dst1[i] = v;
+  const int64_t stride = (int64_t)gridDim.x * kThreads * U;
+  for (int64_t i = (int64_t)blockIdx.x * kThreads * U + threadIdx.x; i < n; i += stride) {
+    u32x4 v[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) v[u] = src[i + u * kThreads < n ? i + u * kThreads : i];
+#pragma unroll
+    for (int u = 0; u < U; u++)
+      if (i + u * kThreads < n) { dst0[i + u * kThreads] = v[u]; dst1[i + u * kThreads] = v[u]; }
   }
 }
 }  // namespace

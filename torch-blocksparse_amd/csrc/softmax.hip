@@ -73,12 +73,47 @@ template <typename T> __device__ __forceinline__ float exp_sub(float x, float mx
   else return __builtin_amdgcn_exp2f(x - mx);
 }
 
+// Dropout on the softmax result (no counterpart in the reference, which refuses dropout: attention.py:223-224).
+// Element i of the [Z, nnz, block, block] tensor (i = its linear offset, z * stride_z + ...) is kept iff
+// u(i) >= p, where u(i) = (w >> 8) * 2^-24 and w is word i % 4 of Philox4x32-10(counter = (i / 4, offset), key = seed);
+// kept elements are scaled by 1 / (1 - p).  The mask is a pure function of (seed, offset, i): the backward pass
+// re-creates it instead of reading it from memory.
+struct DropArgs {
+  float p = 0.f, inv_keep = 1.f;
+  uint32_t seed_lo = 0, seed_hi = 0, off_lo = 0, off_hi = 0;
+  void *yd = nullptr; int64_t yd_sz = 0;   // forward: where the dropped result goes (x keeps the softmax itself)
+};
+
+__device__ __forceinline__ u32x4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; r++) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  return u32x4{c0, c1, c2, c3};
+}
+
+// m[e] = 1 / (1 - p) if element idx + e is kept, else 0; idx is a multiple of 4, EV is 4 or 8
+template <int EV> __device__ __forceinline__ void keep_scale(const DropArgs &d, int64_t idx, float (&m)[EV]) {
+#pragma unroll
+  for (int e4 = 0; e4 < EV; e4 += 4) {
+    const uint64_t q = (uint64_t)(idx + e4) >> 2;
+    const u32x4 w = philox4x32_10((uint32_t)q, (uint32_t)(q >> 32), d.off_lo, d.off_hi, d.seed_lo, d.seed_hi);
+#pragma unroll
+    for (int e = 0; e < 4; e++) m[e4 + e] = (float)(w[e] >> 8) * 5.9604644775390625e-08f >= d.p ? d.inv_keep : 0.f;
+  }
+}
+
 struct FwdArgs {
   void *x; float scale; const int32_t *lut;
   const void *rpe; int64_t rpe_sz, rpe_sh, rpe_sr;
   const void *kpm; int64_t kpm_sz; int kpm_mul;
   const void *attn; int64_t attn_sr; int attn_mul;
   int Z, H, R; int64_t x_sz; int64_t n_units;
+  DropArgs drop;
 };
 
 // where does this wavefront work?  unit = ((z * H*R) + block-row) * G + row group
@@ -115,20 +150,29 @@ template <typename T, int BLOCK> struct Unit {
   }
 };
 
-template <typename T, int BLOCK>
+template <typename T, int BLOCK, bool DROP>
 __device__ __forceinline__ void fwd_store(const FwdArgs &a, const Unit<T, BLOCK> &u, int64_t blockid, const float (&y)[Geo<T, BLOCK>::EV]) {
   constexpr int EV = Geo<T, BLOCK>::EV;
-  T *x = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
+  const int64_t in_z = blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col;
+  T *x = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + in_z;
   Pack<T, EV> p;
 #pragma unroll
   for (int e = 0; e < EV; e++) p.e[e] = from_float<T>(y[e]);
   p.store(x);
+  if constexpr (DROP) {   // the dropped copy goes to its own tensor: the backward pass needs the softmax itself
+    float m[EV];
+    keep_scale<EV>(a.drop, (int64_t)u.z * a.x_sz + in_z, m);
+    Pack<T, EV> q;
+#pragma unroll
+    for (int e = 0; e < EV; e++) q.e[e] = from_float<T>(y[e] * m[e]);
+    q.store(reinterpret_cast<T *>(a.drop.yd) + (int64_t)u.z * a.drop.yd_sz + in_z);
+  }
 }
 
 // NB = number of blocks of a row kept in registers; NB == 0 selects the streaming variant.  EXTRA = a relative
 // position embedding or an attention mask is present (their values are kept beside x until the logits are built; the
 // plain variant does not pay registers for them).
-template <typename T, int BLOCK, int NB, bool EXTRA>
+template <typename T, int BLOCK, int NB, bool EXTRA, bool DROP>
 __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(FwdArgs a) {
   typedef Geo<T, BLOCK> GE;
   constexpr int WPG = waves_per_group_fwd<NB>();
@@ -287,7 +331,7 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
         if (b < size) {
 #pragma unroll
           for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
-          fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
+          fwd_store<T, BLOCK, DROP>(a, u, bid[b], fx[b]);
         }
     } else {
       typedef Pack<T, GE::EV> P;
@@ -401,7 +445,7 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
         if (b < size) {
 #pragma unroll
           for (int e = 0; e < GE::EV; e++) fx[b][e] *= inv;                                            // :137
-          fwd_store<T, BLOCK>(a, u, bid[b], fx[b]);
+          fwd_store<T, BLOCK, DROP>(a, u, bid[b], fx[b]);
         }
     }
   } else {
@@ -413,7 +457,6 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
     const float unit = logit_unit<T>();
     const float sc = a.scale * unit;
     const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
-    T *yb = reinterpret_cast<T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
     const int64_t grow = (int64_t)brow * BLOCK + u.rxm;
     const T *kz = reinterpret_cast<const T *>(a.kpm) + u.z * a.kpm_sz + u.col;
     const T *rz = reinterpret_cast<const T *>(a.rpe) + u.z * a.rpe_sz + head * a.rpe_sh + grow * a.rpe_sr + u.col;
@@ -493,10 +536,10 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
         if (b0 + j < size) {
           float l[GE::EV];
           logits(j, l);
-          P out;
+          float yv[GE::EV];
 #pragma unroll
-          for (int e = 0; e < GE::EV; e++) out.e[e] = from_float<T>(exp_sub<T>(l[e], shift) * inv);   // :131-137
-          out.store(yb + (int64_t)bid[j] * (BLOCK * BLOCK));
+          for (int e = 0; e < GE::EV; e++) yv[e] = exp_sub<T>(l[e], shift) * inv;                     // :131-137
+          fwd_store<T, BLOCK, DROP>(a, u, bid[j], yv);
         }
     }
   }
@@ -505,9 +548,21 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
 struct BwdArgs {
   const void *y; void *dy; float scale; const int32_t *lut;
   int Z, H, R; int64_t y_sz, dy_sz; int64_t n_units;
+  DropArgs drop;
 };
 
-template <typename T, int BLOCK, int NB>
+// dy <- dy * mask / (1 - p) for the chunk of block `blockid` this lane holds: the gradient of the dropped result turned
+// into the gradient of the softmax itself (the mask is re-created from the counter, see DropArgs)
+template <typename T, int BLOCK>
+__device__ __forceinline__ void drop_grad(const BwdArgs &a, const Unit<T, BLOCK> &u, int64_t blockid, Pack<T, Geo<T, BLOCK>::EV> &pd) {
+  constexpr int EV = Geo<T, BLOCK>::EV;
+  float m[EV];
+  keep_scale<EV>(a.drop, (int64_t)u.z * a.y_sz + blockid * (BLOCK * BLOCK) + u.rxm * BLOCK + u.col, m);
+#pragma unroll
+  for (int e = 0; e < EV; e++) pd.e[e] = from_float<T>(to_float(pd.e[e]) * m[e]);
+}
+
+template <typename T, int BLOCK, int NB, bool DROP>
 __global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(BwdArgs a) {
   typedef Geo<T, BLOCK> GE;
   typedef Pack<T, GE::EV> P;
@@ -543,6 +598,14 @@ __global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(
             pd[b].load(db + o);
           }
         }
+      if constexpr (DROP) {
+#pragma unroll
+        for (int g = 0; g < NB; g += 4)
+          if (g < size) {
+#pragma unroll
+            for (int b = g; b < g + 4; b++) drop_grad<T, BLOCK>(a, u, bid[b], pd[b]);
+          }
+      }
 #pragma unroll
       for (int g = 0; g < NB; g += 4)
         if (g < size) {
@@ -581,6 +644,7 @@ __global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(
 #pragma unroll
       for (int b = 0; b < NB; b++)
         if (b < size) {
+          if constexpr (DROP) drop_grad<T, BLOCK>(a, u, bid[b], pd[b]);
 #pragma unroll
           for (int e = 0; e < GE::EV; e++) dot += to_float(py[b].e[e]) * to_float(pd[b].e[e]);   // softmax.py:187-188
         }
@@ -609,6 +673,11 @@ __global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(
           py[j].load_stream(yb + off[j]);
           pd[j].load(db + off[j]);
         }
+      if constexpr (DROP) {
+#pragma unroll
+        for (int j = 0; j < CH; j++)
+          if (b0 + j < size) drop_grad<T, BLOCK>(a, u, off[j] / (BLOCK * BLOCK), pd[j]);
+      }
     };
     float dot = 0.f;
     for (int b0 = 0; b0 < size; b0 += CH) {
@@ -644,13 +713,17 @@ template <typename T, int BLOCK> constexpr int max_nb_bwd() { return Geo<T, BLOC
 template <typename T, int BLOCK, int NB> void launch_fwd_nb(const FwdArgs &a, hipStream_t st) {
   constexpr int WPG = waves_per_group_fwd<NB>();
   const int64_t n_wg = (a.n_units + WPG - 1) / WPG;
-  if (a.rpe || a.attn) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
-  else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  const bool extra = a.rpe || a.attn, drop = a.drop.yd != nullptr;
+  if (extra && drop) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true, true>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  else if (extra) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, true, false>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  else if (drop) hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false, true>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  else hipLaunchKernelGGL((k_softmax_fwd<T, BLOCK, NB, false, false>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
 }
 template <typename T, int BLOCK, int NB> void launch_bwd_nb(const BwdArgs &a, hipStream_t st) {
   constexpr int WPG = waves_per_group_bwd<NB>();
   const int64_t n_wg = (a.n_units + WPG - 1) / WPG;
-  hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  if (a.drop.p > 0.f) hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB, true>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
+  else hipLaunchKernelGGL((k_softmax_bwd<T, BLOCK, NB, false>), dim3((unsigned)n_wg), dim3(64 * WPG), 0, st, a);
 }
 
 template <typename T, int BLOCK> void launch_fwd(const FwdArgs &a, int maxlut, hipStream_t st) {
@@ -718,18 +791,27 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 
 using namespace bsp;
 
-extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int maxlut, const void *rpe,
-                               int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm,
-                               int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r, int attn_mul, int Z,
-                               int H, int R, int block, int64_t x_stride_z, void *stream) {
+namespace {
+bool drop_args(DropArgs &d, float p, uint64_t seed, uint64_t offset) {
+  if (!(p >= 0.f) || !(p < 1.f)) return false;
+  d.p = p; d.inv_keep = 1.f / (1.f - p);
+  d.seed_lo = (uint32_t)seed; d.seed_hi = (uint32_t)(seed >> 32);
+  d.off_lo = (uint32_t)offset; d.off_hi = (uint32_t)(offset >> 32);
+  return true;
+}
+
+int softmax_fwd_impl(int dtype, void *x, float scale, const int32_t *d_lut, int maxlut, const void *rpe, int64_t rpe_stride_z,
+                     int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm, int64_t kpm_stride_z, int kpm_mul,
+                     const void *attn, int64_t attn_stride_r, int attn_mul, int Z, int H, int R, int block, int64_t x_stride_z,
+                     const DropArgs &drop, void *stream) {
   if (!x || !d_lut || Z <= 0 || H <= 0 || R <= 0 || maxlut < 0) return BSP_ERR_ARG;
   if ((int64_t)maxlut * block >= 32768) return BSP_ERR_ROW_TOO_LONG;   // softmax.py:225-227
   const int64_t es = dtype == BSP_F32 ? 4 : 2;
   // vector accesses: every row segment a lane touches must start on a 16-byte boundary
   const int64_t unit = 16 / es;
-  if (!aligned16(x) || !aligned16(rpe) || !aligned16(kpm) || !aligned16(attn)) return BSP_ERR_ARG;
+  if (!aligned16(x) || !aligned16(rpe) || !aligned16(kpm) || !aligned16(attn) || !aligned16(drop.yd)) return BSP_ERR_ARG;
   if (x_stride_z % unit || rpe_stride_z % unit || rpe_stride_h % unit || rpe_stride_r % unit || kpm_stride_z % unit ||
-      attn_stride_r % unit)
+      attn_stride_r % unit || drop.yd_sz % unit)
     return BSP_ERR_ARG;
   FwdArgs a;
   a.x = x; a.scale = scale; a.lut = d_lut;
@@ -737,6 +819,7 @@ extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d
   a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
   a.Z = Z; a.H = H; a.R = R; a.x_sz = x_stride_z;
+  a.drop = drop;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
   if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 26)) return BSP_ERR_UNSUPPORTED;   // one wavefront per unit: 2^32 threads per launch at most
   int rc;
@@ -751,8 +834,8 @@ extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d
   return BSP_OK;
 }
 
-extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
-                               int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream) {
+int softmax_bwd_impl(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H, int R,
+                     int block, int64_t y_stride_z, int64_t dy_stride_z, const DropArgs &drop, void *stream) {
   if (!y || !dy || !d_lut || Z <= 0 || H <= 0 || R <= 0 || maxlut < 0) return BSP_ERR_ARG;
   if ((int64_t)maxlut * block >= 32768) return BSP_ERR_ROW_TOO_LONG;
   const int64_t unit = dtype == BSP_F32 ? 4 : 8;
@@ -760,6 +843,7 @@ extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, 
   BwdArgs a;
   a.y = y; a.dy = dy; a.scale = scale; a.lut = d_lut;
   a.Z = Z; a.H = H; a.R = R; a.y_sz = y_stride_z; a.dy_sz = dy_stride_z;
+  a.drop = drop;
   a.n_units = n_units(dtype, block, (int64_t)Z * H * R);
   if (a.n_units <= 0 || a.n_units >= ((int64_t)1 << 26)) return BSP_ERR_UNSUPPORTED;   // one wavefront per unit: 2^32 threads per launch at most
   int rc;
@@ -772,4 +856,38 @@ extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, 
   if (rc != BSP_OK) return rc;
   BSP_LAUNCH_CHECK();
   return BSP_OK;
+}
+}  // namespace
+
+extern "C" int bsp_softmax_fwd(int dtype, void *x, float scale, const int32_t *d_lut, int maxlut, const void *rpe,
+                               int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r, const void *kpm,
+                               int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r, int attn_mul, int Z,
+                               int H, int R, int block, int64_t x_stride_z, void *stream) {
+  return softmax_fwd_impl(dtype, x, scale, d_lut, maxlut, rpe, rpe_stride_z, rpe_stride_h, rpe_stride_r, kpm, kpm_stride_z, kpm_mul,
+                          attn, attn_stride_r, attn_mul, Z, H, R, block, x_stride_z, DropArgs(), stream);
+}
+
+extern "C" int bsp_softmax_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z, int H,
+                               int R, int block, int64_t y_stride_z, int64_t dy_stride_z, void *stream) {
+  return softmax_bwd_impl(dtype, y, dy, scale, d_lut, maxlut, Z, H, R, block, y_stride_z, dy_stride_z, DropArgs(), stream);
+}
+
+extern "C" int bsp_softmax_dropout_fwd(int dtype, void *x, void *y_drop, float scale, const int32_t *d_lut, int maxlut,
+                                       const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
+                                       const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r,
+                                       int attn_mul, int Z, int H, int R, int block, int64_t x_stride_z, int64_t y_drop_stride_z,
+                                       float drop_p, uint64_t seed, uint64_t offset, void *stream) {
+  DropArgs d;
+  if (!y_drop || !drop_args(d, drop_p, seed, offset)) return BSP_ERR_ARG;
+  d.yd = y_drop; d.yd_sz = y_drop_stride_z;
+  return softmax_fwd_impl(dtype, x, scale, d_lut, maxlut, rpe, rpe_stride_z, rpe_stride_h, rpe_stride_r, kpm, kpm_stride_z, kpm_mul,
+                          attn, attn_stride_r, attn_mul, Z, H, R, block, x_stride_z, d, stream);
+}
+
+extern "C" int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, const int32_t *d_lut, int maxlut, int Z,
+                                       int H, int R, int block, int64_t y_stride_z, int64_t dy_stride_z, float drop_p, uint64_t seed,
+                                       uint64_t offset, void *stream) {
+  DropArgs d;
+  if (!drop_args(d, drop_p, seed, offset)) return BSP_ERR_ARG;
+  return softmax_bwd_impl(dtype, y, dy, scale, d_lut, maxlut, Z, H, R, block, y_stride_z, dy_stride_z, d, stream);
 }

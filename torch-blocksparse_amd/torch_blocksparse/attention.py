@@ -90,8 +90,11 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
     k = k.reshape(bsz, num_heads, k.shape[1], k.shape[2]).contiguous()
     v = v.reshape(bsz, num_heads, v.shape[1], v.shape[2]).contiguous()
     w = sparse_dot_sdd_nt(q, k)
+    # dropout on the attention weights (nn.functional.multi_head_attention_forward applies it after the softmax; the
+    # reference raises NotImplementedError for dropout != 0): fused into the softmax kernel
     w = sparse_softmax(w, key_padding_mask=key_padding_mask, attn_mask=attn_mask,
-                       key_padding_mask_mode=key_padding_mask_mode, attn_mask_mode=attn_mask_mode)
+                       key_padding_mask_mode=key_padding_mask_mode, attn_mask_mode=attn_mask_mode,
+                       dropout_p=float(dropout_p) if training else 0.)
     out = sparse_dot_dsd_nn(w, v)
     out = out.reshape(bsz * num_heads, out.shape[2], out.shape[3])
     out = out.transpose(0, 1).contiguous().view(tgt_len, bsz, embed_dim)
@@ -110,8 +113,6 @@ class MultiheadAttention(nn.modules.activation.MultiheadAttention):
 
     def __init__(self, embed_dim, num_heads, layout, block, dropout=0., bias=True, add_bias_kv=False, add_zero_attn=False,
                  kdim=None, vdim=None, key_padding_mask_mode='add', attn_mask_mode='mul'):
-        if dropout != 0:
-            raise NotImplementedError('dropout is not supported for now')
         if add_bias_kv or add_zero_attn:
             # one more key position than the sequence has: L + 1 is not a whole number of blocks, so no [L/block, L/block]
             # layout can describe the scores (the reference accepts the flags and then fails inside its kernels)

@@ -83,7 +83,7 @@ class GroupPlan:
         return max(16 if block >= 64 else 128, int(2 * mean + 0.5))
 
     # A chain with more entries than this is cut into parts that run as workgroups of their own (block-64 kernels).
-    SPLIT_LEN = 64
+    SPLIT_LEN = 128
 
     @staticmethod
     def order_buckets(layout, by_rows, block):

@@ -69,7 +69,7 @@ class _sparse_softmax(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode,
-                spdims, block, lut, maxlut, bench, time):
+                spdims, block, lut, maxlut, bench, time, dropout=None):
         _lib.require_gpu_tensor(x, 'softmax input')
         if x.dtype not in _lib.DTYPES:
             raise ValueError('softmax input must be float16, bfloat16 or float32')
@@ -93,17 +93,29 @@ class _sparse_softmax(torch.autograd.Function):
             attn_mask = _sparse_softmax._strided16(attn_mask, 'attn_mask')
             attn_args = (_lib.ptr(attn_mask), attn_mask.stride(0))
         timer = _Timer(bench, x.device)
-        rc = _lib.load().bsp_softmax_fwd(_lib.DTYPES[x.dtype], _lib.ptr(x), float(scale), _lib.ptr(lut), maxlut,
-                                         rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3],
-                                         kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
-                                         attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'),
-                                         x.size(0), spdims[0], spdims[1], block, x.stride(0), _lib.stream_ptr(x.device))
-        _lib.check(rc, 'bsp_softmax_fwd')
+        common = (rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3],
+                  kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
+                  attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'),
+                  x.size(0), spdims[0], spdims[1], block, x.stride(0))
+        ctx.dropout = dropout
+        if dropout is None:
+            rc = _lib.load().bsp_softmax_fwd(_lib.DTYPES[x.dtype], _lib.ptr(x), float(scale), _lib.ptr(lut), maxlut, *common,
+                                             _lib.stream_ptr(x.device))
+            _lib.check(rc, 'bsp_softmax_fwd')
+            out = x
+            ctx.mark_dirty(x)
+        else:
+            # x keeps the softmax itself (the backward pass needs it), the dropped copy is a tensor of its own; the mask is
+            # a function of (seed, offset, element), re-created in the backward pass
+            p, seed, offset = dropout
+            out = torch.empty_like(x)
+            rc = _lib.load().bsp_softmax_dropout_fwd(_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(out), float(scale), _lib.ptr(lut), maxlut,
+                                                     *common, out.stride(0), float(p), int(seed), int(offset), _lib.stream_ptr(x.device))
+            _lib.check(rc, 'bsp_softmax_dropout_fwd')
         time[0] = timer.done()
-        ctx.mark_dirty(x)
         ctx.save_for_backward(x, lut)
         ctx.spdims, ctx.block, ctx.maxlut, ctx.scale = spdims, block, maxlut, scale
-        return x
+        return out
 
     @staticmethod
     def backward(ctx, dx):
@@ -113,11 +125,15 @@ class _sparse_softmax(torch.autograd.Function):
         dx = dx.contiguous()
         if dx.data_ptr() % 16 != 0:
             dx = dx.clone()
-        rc = _lib.load().bsp_softmax_bwd(_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(dx), float(ctx.scale), _lib.ptr(lut),
-                                         ctx.maxlut, x.size(0), ctx.spdims[0], ctx.spdims[1], ctx.block, x.stride(0),
-                                         dx.stride(0), _lib.stream_ptr(x.device))
+        args = (_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(dx), float(ctx.scale), _lib.ptr(lut), ctx.maxlut, x.size(0),
+                ctx.spdims[0], ctx.spdims[1], ctx.block, x.stride(0), dx.stride(0))
+        if ctx.dropout is None:
+            rc = _lib.load().bsp_softmax_bwd(*args, _lib.stream_ptr(x.device))
+        else:
+            p, seed, offset = ctx.dropout
+            rc = _lib.load().bsp_softmax_dropout_bwd(*args, float(p), int(seed), int(offset), _lib.stream_ptr(x.device))
         _lib.check(rc, 'bsp_softmax_bwd')
-        return (dx,) + (None,) * 12
+        return (dx,) + (None,) * 13
 
 
 class Softmax:
@@ -142,7 +158,11 @@ class Softmax:
         self.time_y = None
 
     def __call__(self, x, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
-                 key_padding_mask_mode='add', attn_mask_mode='add'):
+                 key_padding_mask_mode='add', attn_mask_mode='add', dropout_p=0., dropout_seed=None, dropout_offset=0):
+        """The reference's arguments (softmax.py:345-361), plus dropout on the result (not in the reference): with
+        dropout_p > 0 the result is softmax(...) * mask / (1 - p) in a new tensor (x itself still receives the softmax).
+        The mask is a counter-based function of (dropout_seed, dropout_offset, element); the seed is drawn from
+        torch's default generator when not given, so torch.manual_seed makes a run repeatable."""
         time_y = [None]
         if rpe is not None and rpe.dtype != x.dtype:
             raise ValueError('relative position embedding must be %s' % x.dtype)
@@ -150,9 +170,15 @@ class Softmax:
             raise ValueError('Attention mask must be %s' % x.dtype)
         if key_padding_mask is not None and key_padding_mask.dtype != x.dtype:
             raise ValueError('Key padding mask must be %s' % x.dtype)
+        if not 0. <= dropout_p < 1.:
+            raise ValueError('dropout probability must be in [0, 1), got %r' % (dropout_p,))
         _lib.require_gpu_tensor(x, 'softmax input')
         lut, maxlut = self.make_lut(x.device)
+        dropout = None
+        if dropout_p > 0.:
+            seed = int(torch.randint(0, 2 ** 62, (1,)).item()) if dropout_seed is None else int(dropout_seed)
+            dropout = (float(dropout_p), seed, int(dropout_offset))
         x = Softmax.sparse_softmax(x, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode,
-                                   self.spdims, self.block, lut, maxlut, self.bench, time_y)
+                                   self.spdims, self.block, lut, maxlut, self.bench, time_y, dropout)
         self.time_y = time_y[0]
         return x
