@@ -39,6 +39,24 @@ int bsp_version(void);
 const char *bsp_strerror(int status);
 
 /* ---------------------------------------------------------------------------------------------------
+ * Layout generators on the device: d_layout receives a [H, NB, NB] int32 layout of 0/1 values, ready for the
+ * table builders below; nothing crosses to the host.
+ * bsp_layout_fixed: the Sparse-Transformer "fixed" pattern (dense != 0: all ones).  whole_stripes = 0 replaces
+ *   torch_blocksparse_cpp_utils.make_layout (csrc/utils.cpp:123-148), which marks only the first column of a vertical
+ *   stripe; whole_stripes = 1 replaces DeepSpeedSparseSelfAttention._make_layout
+ *   (deepspeedsparseselfattention.py:31-65), which marks all `vertsize` of them.  NB must be a multiple of block_stride.
+ * bsp_layout_sparse_transformer: local windows of local_blocks blocks + the last column of every global_stride blocks
+ *   as a global column (the benchmark's attention layout; no counterpart in the reference).
+ * bsp_layout_bigbird: sliding window + num_global leading global columns (and rows unless causal) + the random columns
+ *   d_random_cols [H, NB, num_random] (int32, drawn by the caller); no counterpart in the reference.
+ * ------------------------------------------------------------------------------------------------- */
+int bsp_layout_fixed(int32_t *d_layout, int H, int NB, int dense, int block_stride, int unidirectional, int numverts,
+                     int vertsize, int whole_stripes, void *stream);
+int bsp_layout_sparse_transformer(int32_t *d_layout, int H, int NB, int local_blocks, int global_stride, int causal, void *stream);
+int bsp_layout_bigbird(int32_t *d_layout, int H, int NB, int window, int num_global, int causal, const int32_t *d_random_cols,
+                       int num_random, void *stream);
+
+/* ---------------------------------------------------------------------------------------------------
  * Look-up-table builders.  d_layout is the layout as int32 [H, R, C] in device memory (0/1 values).
  * d_ws is scratch of at least bsp_lut_workspace_bytes(H, R, C) bytes.
  * ------------------------------------------------------------------------------------------------- */

@@ -11,7 +11,7 @@
  *   orc_sdd_segment        : against the reference's own C++ (csrc/utils.cpp compiled into oracle/_ref)
  *                            on random layouts + committed golden fixtures + closed form at width 1.
  *   orc_make_layout_cpp    : against oracle/_ref make_layout + committed golden fixtures.
- *   orc_make_layout_py     : brute-force definition on small sizes + golden fixtures.
+ *   orc_make_layout_py     : golden layouts written by the reference's own _make_layout (vertical stripes of 1-4 blocks).
  *   orc_softmax_lut        : closed form from nonzero()/cumsum + hand-derived known answer.
  *   orc_load_balance,
  *   orc_dxx_lut            : committed golden fixtures generated from the reference's Python

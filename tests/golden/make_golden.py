@@ -2,8 +2,9 @@
 
 Two sources, both only available where the reference checkout is mounted:
   * oracle/_ref : the reference's csrc/utils.cpp compiled as is (oracle/Makefile) -> sdd_segment, make_layout
-  * the reference's Python `_sparse_matmul.load_balance` / `make_dxx_lut` (matmul.py:221-267, 372-458),
-    imported from the checkout.  No other reference function is run: every other table has a closed form.
+  * the reference's Python `_sparse_matmul.load_balance` / `make_dxx_lut` (matmul.py:221-267, 372-458) and
+    `DeepSpeedSparseSelfAttention._make_layout` (deepspeedsparseselfattention.py:31-65), imported from the
+    checkout.  No other reference function is run: every other table has a closed form.
 The vectors are plain JSON (inputs + expected outputs); the reference itself is not stored anywhere.
 
 usage: python tests/golden/make_golden.py [/root/reference]
@@ -63,11 +64,21 @@ def load_reference_matmul(ref_cpp):
     return mod._sparse_matmul
 
 
+def load_reference_make_layout(ref_cpp):
+    """DeepSpeedSparseSelfAttention._make_layout of the reference, through the reference's own package."""
+    sys.modules['torch_blocksparse_cpp_utils'] = ref_cpp
+    sys.path.insert(0, REF)
+    import torch_blocksparse                                  # the reference checkout (this script never adds the repository's package)
+    assert os.path.dirname(torch_blocksparse.__file__).startswith(REF)
+    from torch_blocksparse.deepspeedsparseselfattention import DeepSpeedSparseSelfAttention
+    return DeepSpeedSparseSelfAttention._make_layout
+
+
 def main():
     lays, ref_cpp = layouts()
     sm = load_reference_matmul(ref_cpp)
     gold = {'layouts': {k: v.tolist() for k, v in lays.items()}, 'sdd_segment': [], 'dxx_lut': [], 'load_balance': [],
-            'make_layout_cpp': []}
+            'make_layout_cpp': []}   # 'make_layout_py' is added below
     for name, lay in lays.items():
         for start_width in (4, 2, 1):
             seg = ref_cpp.sdd_segment(lay.to(torch.int32).clone(), start_width)
@@ -93,6 +104,13 @@ def main():
     for args in [(2, 8, 'fixed', 4, True, 1, 1), (3, 16, 'fixed', 4, False, 2, 1), (4, 16, 'fixed', 8, True, 4, 2),
                  (2, 16, 'fixed', 4, False, 2, 2), (1, 4, 'dense', 4, True, 1, 1), (4, 64, 'fixed', 16, True, 1, 1)]:
         gold['make_layout_cpp'].append({'args': list(args), 'layout': ref_cpp.make_layout(*args).tolist()})
+    make_layout_py = load_reference_make_layout(ref_cpp)
+    gold['make_layout_py'] = []
+    for args in [(2, 8, 'fixed', 4, 'unidirectional', 1, 1), (4, 16, 'fixed', 4, 'bidirectional', 2, 2),
+                 (4, 16, 'fixed', 8, 'unidirectional', 4, 2), (3, 32, 'fixed', 8, 'bidirectional', 8, 1),
+                 (3, 24, 'fixed', 6, 'unidirectional', 2, 3), (5, 16, 'fixed', 8, 'unidirectional', 2, 4),
+                 (2, 12, 'fixed', 4, 'bidirectional', 1, 4), (2, 8, 'dense', 4, 'unidirectional', 1, 1)]:
+        gold['make_layout_py'].append({'args': list(args), 'layout': make_layout_py(*args).tolist()})
     path = os.path.join(HERE, 'lut_golden.json')
     with open(path, 'w') as f:
         json.dump(gold, f, separators=(',', ':'))

@@ -175,3 +175,49 @@ def test_group_plan_over_tiles(by_rows):
                 h, tr, tc = tiles[tid].tolist()
                 assert got.tolist() == fine[h, tr * S:(tr + 1) * S, tc * S:(tc + 1) * S].tolist()
     assert GroupPlan.build_coarse(random_layout((1, 6, 9), 0.5, 1), 16, by_rows, DEV) is None   # sides must divide by 4
+
+
+def test_layouts_built_on_the_device_equal_the_host_generators(golden):
+    # every generator with device='cuda' against its host form and against the vectors written by the reference's own
+    # generators (C++ make_layout and Python _make_layout)
+    for c in golden['make_layout_cpp']:
+        assert tb.make_layout(*c['args'], device=DEV).cpu().tolist() == c['layout']
+    for c in golden['make_layout_py']:
+        assert tb.fixed_layout(*c['args'], device=DEV).cpu().tolist() == c['layout']
+    for args in [(3, 48, 'fixed', 12, 'unidirectional', 3, 4), (5, 64, 'fixed', 16, 'bidirectional', 4, 2), (2, 7, 'dense', 7, 'unidirectional', 1, 1),
+                 (16, 256, 'fixed', 4, 'unidirectional', 1, 1)]:
+        dev = tb.fixed_layout(*args, device=DEV)
+        assert dev.dtype == torch.int32 and dev.is_cuda
+        assert torch.equal(dev.cpu().long(), tb.fixed_layout(*args))
+        uni = args[4] == 'unidirectional'
+        assert torch.equal(tb.make_layout(*args[:4], uni, *args[5:], device=DEV).cpu().long(), tb.make_layout(*args[:4], uni, *args[5:]))
+    for args in [(16, 64, 4, 16, True), (3, 30, 5, 6, False), (2, 8, 2, 3, True), (3, 18, 4, 8, True)]:
+        assert torch.equal(tb.sparse_transformer_layout(*args, device=DEV).cpu().long(), tb.sparse_transformer_layout(*args))
+    for kw in [dict(seed=0, causal=True), dict(seed=3, causal=False), dict(window=5, num_global=1, num_random=0, seed=1, causal=True)]:
+        assert torch.equal(tb.bigbird_layout(4, 64, device=DEV, **kw).cpu().long(), tb.bigbird_layout(4, 64, **kw))
+    big = tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True, device=DEV)
+    assert torch.equal(big.cpu().long(), tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True))
+
+
+def test_operators_take_a_layout_that_lives_on_the_device():
+    # tables built from a device layout are the tables built from its host copy, and the operators give the same results
+    from torch_blocksparse.softmax import _sparse_softmax
+    from torch_blocksparse.matmul import _sparse_matmul
+    lay_d = tb.sparse_transformer_layout(2, 16, 4, 8, True, device=DEV)
+    lay_h = lay_d.cpu().long()
+    a, _ = _sparse_softmax.make_lut(lay_d, 64, DEV)
+    b, _ = _sparse_softmax.make_lut(lay_h, 64, DEV)
+    assert torch.equal(a, b)
+    for trans in (False, True):
+        assert torch.equal(_sparse_matmul.make_dxx_lut(lay_d, 64, 16, trans, DEV)[0], _sparse_matmul.make_dxx_lut(lay_h, 64, 16, trans, DEV)[0])
+    q, k, v = [torch.randn(2, 2, 1024, 64, device=DEV, dtype=torch.float16) for _ in range(3)]
+    outs = []
+    for lay in (lay_d, lay_h):
+        sdd, dsd, sm = tb.MatMul(lay, 64, 'sdd', trans_b=True), tb.MatMul(lay, 64, 'dsd'), tb.Softmax(lay, 64)
+        outs.append(dsd(sm(sdd(q, k), scale=0.125), v))
+    assert torch.equal(outs[0], outs[1])
+    # block 16: the plan over 64 x 64 tiles is assembled from the device layout as well
+    lay16 = tb.fixed_layout(2, 64, 'fixed', 16, 'unidirectional', 1, 1, device=DEV)
+    x = torch.randn(1, int(lay16.sum()), 16, 16, device=DEV, dtype=torch.float16)
+    y = torch.randn(1, 2, 1024, 64, device=DEV, dtype=torch.float16)
+    assert torch.equal(tb.MatMul(lay16, 16, 'dsd')(x, y), tb.MatMul(lay16.cpu().long(), 16, 'dsd')(x, y))

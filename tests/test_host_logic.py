@@ -58,6 +58,11 @@ def test_constructor_errors():
 def test_layout_generators_match_oracle(golden):
     for c in golden['make_layout_cpp']:
         assert tb.make_layout(*c['args']).tolist() == c['layout']
+    # vectors written by the reference's own DeepSpeedSparseSelfAttention._make_layout (vertical stripes wider than one
+    # block included): they pin the oracle's restatement and the package's generator alike
+    for c in golden['make_layout_py']:
+        assert O.make_layout_py(*c['args']).tolist() == c['layout']
+        assert tb.fixed_layout(*c['args']).tolist() == c['layout']
     for args in [(2, 8, 'fixed', 4, 'unidirectional', 1, 1), (4, 16, 'fixed', 4, 'bidirectional', 2, 2),
                  (4, 16, 'fixed', 8, 'unidirectional', 4, 2), (3, 32, 'fixed', 8, 'bidirectional', 8, 1),
                  (2, 8, 'dense', 4, 'unidirectional', 1, 1)]:
