@@ -25,6 +25,7 @@ typedef enum { BSP_F16 = 0, BSP_BF16 = 1, BSP_F32 = 2 } bsp_dtype;
 typedef enum {
   BSP_OK = 0,
   BSP_OK_WHOLE_LAYOUT = 1,   /* bsp_sdd_matmul only: the group plan was used, every block of the layout is written */
+  BSP_NEEDS_TABLE = 2,       /* bsp_sdd_matmul called with the plan alone: nothing launched, call again with the sdd table */
   BSP_ERR_ARG = -1,          /* null pointer, bad size, misaligned operand */
   BSP_ERR_UNSUPPORTED = -2,  /* block size / dtype / mode not built */
   BSP_ERR_CAPACITY = -3,     /* caller-provided table or workspace too small */
@@ -152,7 +153,10 @@ typedef enum {
  * groups and the number of block-rows per head (NULL / 0 / 0 if none); when given, a kernel that shares operand
  * tiles inside each group may take the launch.  The plan describes the whole layout, not one pack level: if that
  * kernel ran, the return value is BSP_OK_WHOLE_LAYOUT and the caller skips the remaining pack levels (pass the plan
- * with the first level only). */
+ * with the first level only).  A caller that has the plan but has not built the table yet (its greedy packing is the
+ * one sequential step of the builders) may call with d_lut = NULL, pack = 0, n_groups = 0: the result is
+ * BSP_OK_WHOLE_LAYOUT if a kernel that works from the plan alone took the product, else BSP_NEEDS_TABLE and nothing was
+ * launched. */
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
                    int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
                    int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,

@@ -19,6 +19,7 @@ extern "C" const char *bsp_strerror(int status) {
   switch (status) {
     case BSP_OK: return "ok";
     case BSP_OK_WHOLE_LAYOUT: return "ok, every block of the layout written (skip the remaining pack levels)";
+    case BSP_NEEDS_TABLE: return "nothing launched: this product needs the sdd table (call again with it)";
     case BSP_ERR_ARG: return "invalid argument (null pointer, bad size or operand not 16-byte aligned)";
     case BSP_ERR_UNSUPPORTED: return "unsupported block size, dtype or problem size";
     case BSP_ERR_CAPACITY: return "caller-provided table or workspace too small";
@@ -36,7 +37,8 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
                               int64_t ldb, int64_t c_stride_z, int block, int pack, const int32_t *d_lut,
                               const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups,
                               int plan_lines, int flags, void *stream) {
-  if (!a || !b || !c || !d_lut || Z <= 0 || K <= 0 || n_groups < 0) return BSP_ERR_ARG;
+  if (!a || !b || !c || Z <= 0 || K <= 0 || n_groups < 0) return BSP_ERR_ARG;
+  if (!d_lut && (!d_gplan || no_groups(flags) || general_only(flags))) return d_gplan ? BSP_NEEDS_TABLE : BSP_ERR_ARG;
   if (!block_ok(block)) return BSP_ERR_UNSUPPORTED;
   if (K % 16) return BSP_ERR_K_MULTIPLE;   // reference matmul.py:318-319
   const int u = elems16(dtype);
@@ -55,6 +57,7 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   int rc = general_only(flags) ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
   if (rc < 0) return rc;
   if (rc >= 1) { BSP_LAUNCH_CHECK(); return rc == 2 ? BSP_OK_WHOLE_LAYOUT : BSP_OK; }
+  if (!d_lut) return BSP_NEEDS_TABLE;      // a call with the plan alone, and no kernel that works from the plan applies
   switch (dtype) {
     case BSP_F16: rc = sdd_generic_f16(g, block, pack, a_kc, b_kc, st); break;
     case BSP_BF16: rc = sdd_generic_bf16(g, block, pack, a_kc, b_kc, st); break;

@@ -1189,14 +1189,16 @@ template <typename T> int sdd_small_t(const SddArgs &g, int block, hipStream_t s
   return BSP_OK;
 }
 
+// -> 2: the plan kernel wrote the whole layout; BSP_OK: the per-block kernel took this pack level; 1: nothing applies
 template <typename T> int sdd_fast_t(const SddArgs &g, hipStream_t st) {
   if (g.gplan && g.n_pgroups > 0 && (g.K == 64 || g.K == 128) && !g.valid) {
     const int64_t n = (int64_t)g.n_pgroups * g.Z;
     if (n >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
     if (g.K == 64) hipLaunchKernelGGL((k_sdd64_rg<T, 64>), dim3((unsigned)n), dim3(256), 0, st, g);
     else hipLaunchKernelGGL((k_sdd64_rg<T, 128>), dim3((unsigned)n), dim3(256), 0, st, g);
-    return BSP_OK;
+    return 2;
   }
+  if (!g.lut) return 1;
   const int64_t n_wg = (g.n_groups * g.Z + 3) / 4;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
@@ -1248,9 +1250,10 @@ int sdd_fast64(int dtype, const SddArgs &g0, int block, int pack, bool a_kc, boo
     int rc = dtype == BSP_F16 ? sdd_small_t<f16>(g, block, st) : sdd_small_t<bf16>(g, block, st);
     return rc == BSP_OK ? 2 : rc;
   }
-  if (dtype == BSP_F32 || !fast_ok_sdd(g, block, pack, a_kc, b_kc)) return 0;
+  // (a call without the table, with the plan alone: pack is unknown, the plan kernel covers every pack level anyway)
+  if (dtype == BSP_F32 || !fast_ok_sdd(g, block, g.lut ? pack : 1, a_kc, b_kc)) return 0;
   int rc = dtype == BSP_F16 ? sdd_fast_t<f16>(g, st) : sdd_fast_t<bf16>(g, st);
-  return rc == BSP_OK ? 1 : rc;
+  return rc == BSP_OK ? 1 : rc == 1 ? 0 : rc;
 }
 // a plan over 64 x 64 tiles of a block-16 / block-32 layout (negative line count): the block-64 row-group kernel,
 // gathering each tile from its small blocks

@@ -19,6 +19,7 @@ FLAG_GENERAL_ONLY, FLAG_NO_GROUPS = 1, 2   # bsp_launch_flags
 
 OK = 0
 OK_WHOLE_LAYOUT = 1   # bsp_sdd_matmul: the group plan was used, every block of the layout is written
+NEEDS_TABLE = 2       # bsp_sdd_matmul called with the plan alone: nothing launched, the sdd table is needed
 ERR_CAPACITY = -3
 ERR_EMPTY_HEAD = -4
 ERR_ROW_TOO_LONG = -6

@@ -31,10 +31,30 @@ class _LayoutOnDevice:
         self.lay = _lib.layout_to_device(layout, self.device)
         self.ws, self.ws_bytes = _lib.workspace(self.lay, self.device)
         self.nnz = int((layout != 0).sum())
+        self._coarse = None
 
     @staticmethod
     def of(layout, device, ctx):
         return ctx if ctx is not None else _LayoutOnDevice(layout, device)
+
+    def coarse(self, S):
+        """The layout coarsened to tiles of S x S blocks (a tile is present if any of its blocks is), as a context of its
+        own, and per present tile the ids of its S * S blocks (-1 where absent), tiles in nonzero() order.  Made once
+        and shared by the plans over tiles of all three products."""
+        if self._coarse is None:
+            H, R, C = self.lay.shape
+            lay = self.lay != 0
+            tiles5 = lay.reshape(H, R // S, S, C // S, S)
+            present = tiles5.any(4).any(2)
+            cctx = _LayoutOnDevice.__new__(_LayoutOnDevice)
+            cctx.device, cctx.lay = self.device, present.to(torch.int32).contiguous()
+            cctx.ws, cctx.ws_bytes = _lib.workspace(cctx.lay, self.device)
+            cctx.nnz = int(present.sum())
+            cctx._coarse = None
+            fine = torch.where(lay, torch.cumsum(lay.reshape(-1), 0, dtype=torch.int32).reshape(lay.shape) - 1, -1).to(torch.int32)
+            ids = fine.reshape(H, R // S, S, C // S, S).permute(0, 1, 3, 2, 4)[present].reshape(-1, S * S)
+            self._coarse = (cctx, ids)
+        return self._coarse
 
 
 def _prep(x):
@@ -73,13 +93,13 @@ class GroupPlan:
         self._ws = None
 
     @staticmethod
-    def thin_min(layout, by_rows, block=64):
+    def thin_min(layout, by_rows, block=64, nnz=None):
         """Lines at least this long become chains: well above the average line, so that dense-ish layouts (whose
         groups share every dense tile four times) keep their groups and only outliers such as global columns split.
         The kernels for blocks 16 and 32 give a chain less than the block-64 kernel does (measured on the attention
         mask: chains of 98 blocks of 32 cost 3 us, chains of 196 blocks of 16 save 15), so only very long lines split."""
         H, R, C = layout.shape
-        mean = float((layout != 0).sum()) / max(1, H * (R if by_rows else C))
+        mean = float((layout != 0).sum() if nnz is None else nnz) / max(1, H * (R if by_rows else C))
         return max(16 if block >= 64 else 128, int(2 * mean + 0.5))
 
     # A chain with more entries than this is cut into parts that run as workgroups of their own (block-64 kernels).
@@ -114,7 +134,7 @@ class GroupPlan:
         return GroupPlan(table[:n.value], n_groups.value, R if by_rows else C, n_split.value)
 
     @staticmethod
-    def build_coarse(layout, block, by_rows, device, for_sdd=False):
+    def build_coarse(layout, block, by_rows, device, for_sdd=False, ctx=None):
         """Plan of a block-16 layout over 64 x 64 tiles: the groups, chains and order of `build` on the layout coarsened
         to 64 (a tile is present if any of its S x S blocks is, S = 64 / block), with entries that carry the ids of the
         small blocks: (position, 4 tile ids, 4 x S*S block ids, -1 where absent).  The launchers are told by a
@@ -126,23 +146,18 @@ class GroupPlan:
         H, R, C = layout.shape
         if R % S or C % S:
             return None
-        dev = torch.device(device)
-        lay = (layout != 0)
-        coarse = lay.reshape(H, R // S, S, C // S, S).any(4).any(2).to(torch.int64)
-        plan = GroupPlan.build(coarse, by_rows, dev, thin_min=0 if for_sdd else GroupPlan.thin_min(coarse, by_rows, 64),
+        ctx = _LayoutOnDevice.of(layout, device, ctx)
+        cctx, tiles = ctx.coarse(S)
+        coarse = cctx.lay
+        plan = GroupPlan.build(coarse, by_rows, ctx.device, thin_min=0 if for_sdd else GroupPlan.thin_min(coarse, by_rows, 64, nnz=cctx.nnz),
                                order_buckets=2 if for_sdd else GroupPlan.order_buckets(coarse, by_rows, 64),
-                               split_len=0 if for_sdd else GroupPlan.SPLIT_LEN)
+                               split_len=0 if for_sdd else GroupPlan.SPLIT_LEN, ctx=cctx)
         ng, G = plan.n_groups, 4
         table = plan.table
         header, entries = table[:4 * ng], table[4 * ng:].view(-1, G + 1)
-        # ids of the small blocks of every present tile, tiles in nonzero() order like the plan's tile ids
-        layd = lay.to(dev)
-        fine = torch.where(layd, torch.cumsum(layd.reshape(-1).to(torch.int64), 0).reshape(layd.shape) - 1,
-                           torch.full((), -1, dtype=torch.int64, device=dev)).to(torch.int32)
-        tiles = fine.reshape(H, R // S, S, C // S, S).permute(0, 1, 3, 2, 4)[coarse.to(dev).bool()].reshape(-1, S * S)
         ids = entries[:, 1:].to(torch.int64)                                    # [entries, G] tile ids or -1
-        sub = torch.where((ids >= 0).unsqueeze(2), tiles[ids.clamp(min=0)], torch.full((), -1, dtype=torch.int32, device=dev))
-        wide = torch.cat([entries, sub.reshape(entries.shape[0], G * S * S)], 1).to(torch.int32)
+        sub = torch.where((ids >= 0).unsqueeze(2), tiles[ids.clamp(min=0)], -1)
+        wide = torch.cat([entries, sub.reshape(entries.shape[0], G * S * S)], 1)
         out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines, plan.n_split)
         out.coarse = True
         return out
@@ -202,9 +217,22 @@ def _check_sparse(name, x, nnz, block, Z):
 
 class SddTables(list):
     """The per-pack sdd tables, in the reference's order; `nnz` is the number of blocks of the output, `gplan` the
-    optional row-group plan of the layout."""
+    optional row-group plan of the layout.  Built by `MatMul.make_lut` the list starts empty and `build` fills it when a
+    product first needs the tables: the greedy packing behind them is the one sequential step of the builders
+    (milliseconds at block 16), and the kernels that work from the plan alone never read them."""
     nnz = 0
     gplan = None
+    spdims = None
+    build = None          # callable -> (tables, widths, packs), or None when the list is complete
+    widths = None
+    packs = None
+
+    def materialize(self):
+        if self.build is not None:
+            tables, self.widths, self.packs = self.build()
+            self.extend(tables)
+            self.build = None
+        return self.widths, self.packs
 
 
 class _sparse_matmul(torch.autograd.Function):
@@ -213,52 +241,63 @@ class _sparse_matmul(torch.autograd.Function):
     # SPARSE = DENSE x DENSE #
     ##########################
     @staticmethod
-    def make_sdd_lut(layout, block, dtype, device, ctx=None):
+    def make_sdd_lut(layout, block, dtype, device, ctx=None, lazy=False):
         """-> (luts, None, widths, packs) as the reference (matmul.py:281-297); built on `device`.
 
         start_width is 64 // block in the reference, which is 0 for block 128 and leaves the table empty
         (matmul.py:283, csrc/utils.cpp:117); max(1, .) gives block 128 the single-block table it needs.
         Each table tensor carries `.valid` (None, or a uint8 tensor marking the rows that really are blocks).
+        lazy: return (luts, None, None, None) with the tables not built yet; `luts.materialize()` builds them (the
+        row-group plan, which the specialised kernels work from, is always built here).
         """
         lib = _lib.load()
         ctx = _LayoutOnDevice.of(layout, device, ctx)
         dev, lay, nnz = ctx.device, ctx.lay, ctx.nnz
         H, R, C = lay.shape
-        start_width = max(1, 64 // block)
-        cap = nnz + nnz // 8 + 64
-        n_levels = ctypes.c_int(0)
-        packs = (ctypes.c_int * 8)()
-        rows = (ctypes.c_int64 * 8)()
-        total = ctypes.c_int64(0)
-        all_valid = ctypes.c_int(1)
-        for attempt in range(2):
-            lut = torch.empty((cap, 4), dtype=torch.int32, device=dev)
-            valid = torch.empty((cap,), dtype=torch.uint8, device=dev)
-            rc = lib.bsp_sdd_lut_build(_lib.ptr(lay), H, R, C, start_width, _lib.ptr(lut), _lib.ptr(valid), cap, _lib.ptr(ctx.ws),
-                                       ctx.ws_bytes, ctypes.byref(n_levels), packs, rows, ctypes.byref(total),
-                                       ctypes.byref(all_valid), _lib.stream_ptr(dev))
-            if rc == _lib.ERR_CAPACITY and attempt == 0:
-                cap = int(total.value)
-                continue
-            _lib.check(rc, 'bsp_sdd_lut_build')
-            break
-        luts, widths, out_packs = SddTables(), [], []
+
+        def build_tables():
+            start_width = max(1, 64 // block)
+            cap = nnz + nnz // 8 + 64
+            n_levels = ctypes.c_int(0)
+            packs = (ctypes.c_int * 8)()
+            rows = (ctypes.c_int64 * 8)()
+            total = ctypes.c_int64(0)
+            all_valid = ctypes.c_int(1)
+            for attempt in range(2):
+                lut = torch.empty((cap, 4), dtype=torch.int32, device=dev)
+                valid = torch.empty((cap,), dtype=torch.uint8, device=dev)
+                rc = lib.bsp_sdd_lut_build(_lib.ptr(lay), H, R, C, start_width, _lib.ptr(lut), _lib.ptr(valid), cap, _lib.ptr(ctx.ws),
+                                           ctx.ws_bytes, ctypes.byref(n_levels), packs, rows, ctypes.byref(total),
+                                           ctypes.byref(all_valid), _lib.stream_ptr(dev))
+                if rc == _lib.ERR_CAPACITY and attempt == 0:
+                    cap = int(total.value)
+                    continue
+                _lib.check(rc, 'bsp_sdd_lut_build')
+                break
+            tables, widths, out_packs = [], [], []
+            done = 0
+            for k in range(n_levels.value):
+                p, r = int(packs[k]), int(rows[k])
+                t = lut[done:done + r].reshape(-1)
+                t.valid = None if all_valid.value else valid[done:done + r]
+                tables.append(t)
+                widths.append(r // (p * p))
+                out_packs.append(p)
+                done += r
+            return tables, widths, out_packs
+
+        luts = SddTables()
         luts.nnz = nnz
         luts.spdims = tuple(layout.shape)
+        luts.build = build_tables
         if block in (16, 32, 64):
-            luts.gplan = GroupPlan.build_coarse(layout, block, True, dev, for_sdd=True) if block == 16 else None
+            luts.gplan = GroupPlan.build_coarse(layout, block, True, dev, for_sdd=True, ctx=ctx) if block == 16 else None
             if luts.gplan is None:
                 luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0, ctx=ctx)
-        done = 0
-        for k in range(n_levels.value):
-            p, r = int(packs[k]), int(rows[k])
-            t = lut[done:done + r].reshape(-1)
-            t.valid = None if all_valid.value else valid[done:done + r]
-            luts.append(t)
-            widths.append(r // (p * p))
-            out_packs.append(p)
-            done += r
-        return luts, None, widths, out_packs
+        if lazy and luts.gplan is not None:
+            return luts, None, None, None
+        widths, packs = luts.materialize()
+        return luts, None, widths, packs
 
     @staticmethod
     def _sdd_matmul(a, b, trans_a, trans_b, trans_c, spdims, block, luts, num_locks, widths, packs, bench, time):
@@ -275,21 +314,32 @@ class _sparse_matmul(torch.autograd.Function):
         _check_dense('a', a, spdims[0], block * spdims[1], None, trans_a)
         _check_dense('b', b, spdims[0], None, block * spdims[2], trans_b)
         lib = _lib.load()
-        total_width = luts.nnz if isinstance(luts, SddTables) else sum(w * p * p for w, p in zip(widths, packs))
+        lazy = isinstance(luts, SddTables)
+        total_width = luts.nnz if lazy else sum(w * p * p for w, p in zip(widths, packs))
         c = torch.empty((AS0, total_width, block, block), dtype=a.dtype, device=a.device)
         timer = _Timer(bench, a.device)
-        # the group plan describes the whole layout: it goes with the first pack level, and if the library used it
-        # (status OK_WHOLE_LAYOUT) every block is written and the other levels are skipped
+        operands = (_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
+                    AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2), c.stride(0), block)
+        # The group plan describes the whole layout.  If the tables are not built yet it goes first on its own: a kernel
+        # that works from the plan writes every block (status OK_WHOLE_LAYOUT) and the tables are never needed; otherwise
+        # nothing was launched (NEEDS_TABLE), the tables are built and the plan goes with the first pack level.
         gplan = GroupPlan.args(getattr(luts, 'gplan', None))
-        for lut, width, pack in zip(luts, widths, packs):
-            rc = lib.bsp_sdd_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
-                                    AS0, AS3, a.stride(0), a.stride(1), a.stride(2), b.stride(0), b.stride(1), b.stride(2),
-                                    c.stride(0), block, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
-                                    gplan[0], gplan[1], gplan[2], KERNEL_FLAGS, _lib.stream_ptr(a.device))
-            if rc == _lib.OK_WHOLE_LAYOUT:
-                break
-            _lib.check(rc, 'bsp_sdd_matmul')
-            gplan = GroupPlan.args(None)
+        rc = _lib.NEEDS_TABLE
+        if lazy and luts.build is not None and luts.gplan is not None:
+            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), 0, gplan[0], gplan[1], gplan[2], KERNEL_FLAGS,
+                                    _lib.stream_ptr(a.device))
+            if rc not in (_lib.OK_WHOLE_LAYOUT, _lib.NEEDS_TABLE):
+                _lib.check(rc, 'bsp_sdd_matmul')
+        if rc == _lib.NEEDS_TABLE:
+            if lazy:
+                widths, packs = luts.materialize()
+            for lut, width, pack in zip(luts, widths, packs):
+                rc = lib.bsp_sdd_matmul(*operands, pack, _lib.ptr(lut), _lib.ptr(getattr(lut, 'valid', None)), width,
+                                        gplan[0], gplan[1], gplan[2], KERNEL_FLAGS, _lib.stream_ptr(a.device))
+                if rc == _lib.OK_WHOLE_LAYOUT:
+                    break
+                _lib.check(rc, 'bsp_sdd_matmul')
+                gplan = GroupPlan.args(None)
         time[0] = timer.done()
         return c
 
@@ -326,9 +376,9 @@ class _sparse_matmul(torch.autograd.Function):
         lut.plan = planbuf[first:first + 2 * nnz].view(nnz, 2)
         lut.nnz = nnz
         lut.spdims = tuple(layout.shape)
-        lut.gplan = GroupPlan.build_coarse(layout, block, trans, dev) if block == 16 else None
+        lut.gplan = GroupPlan.build_coarse(layout, block, trans, dev, ctx=ctx) if block == 16 else None
         if lut.gplan is None and block in (16, 32, 64):
-            lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block),
+            lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block, nnz=nnz),
                                         order_buckets=GroupPlan.order_buckets(layout, trans, block),
                                         split_len=GroupPlan.SPLIT_LEN if block == 64 else 0, ctx=ctx)
         return lut, num_locks.value, width.value, None
@@ -448,7 +498,7 @@ class MatMul:
         layout, block = self.layout, self.block
         step = 8 if dtype == torch.float32 else 16             # matmul.py:617
         ctx = _LayoutOnDevice(layout, device)                  # one upload of the layout and one workspace for all tables
-        sdd = lambda: _sparse_matmul.make_sdd_lut(layout, block, dtype, device, ctx=ctx)
+        sdd = lambda: _sparse_matmul.make_sdd_lut(layout, block, dtype, device, ctx=ctx, lazy=True)
         dxx = lambda trans: _sparse_matmul.make_dxx_lut(layout, block, step, trans, device, ctx=ctx)
         if self.mode == 'sdd':                                 # matmul.py:618-637
             c, da, db = sdd(), dxx(True), dxx(False)
