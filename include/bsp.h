@@ -142,7 +142,8 @@ int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_ro
  * ------------------------------------------------------------------------------------------------- */
 typedef enum {
   BSP_FLAG_GENERAL_ONLY = 1,  /* take the general kernels even where a specialised one would serve (for cross-checks) */
-  BSP_FLAG_NO_GROUPS = 2      /* ignore the group plan (the per-block / per-segment kernels run instead) */
+  BSP_FLAG_NO_GROUPS = 2,     /* ignore the group plan (the per-block / per-segment kernels run instead) */
+  BSP_FLAG_NO_WIDE = 4        /* skip the kernels specialised for a wide free dimension (dsd / dds, blocks 64 and 128) */
 } bsp_launch_flags;
 
 /* sparse = dense x dense: replaces _sparse_matmul._sdd_matmul + the SDD branch of the kernel

@@ -8,6 +8,7 @@ using namespace bsp;
 namespace {
 bool no_groups(int flags) { return (flags & BSP_FLAG_NO_GROUPS) != 0; }
 bool general_only(int flags) { return (flags & BSP_FLAG_GENERAL_ONLY) != 0; }
+bool no_wide(int flags) { return (flags & (BSP_FLAG_NO_WIDE | BSP_FLAG_GENERAL_ONLY)) != 0; }
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool block_ok(int block) { return block == 16 || block == 32 || block == 64 || block == 128; }
 int elems16(int dtype) { return dtype == BSP_F32 ? 4 : 8; }   // elements per 16 bytes
@@ -91,7 +92,11 @@ static int xsd_workspace(XsdArgs &g, int n_split, int free_dim, void *d_ws, int6
 
 static int xsd_dispatch(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, int flags, void *stream) {
   hipStream_t st = as_stream(stream);
-  int rc = general_only(flags) ? 0 : xsd_fast64(dtype, g, block, sp_trans, dn_kc, out_nc, st);
+  // a wide free dimension at blocks 64 / 128: the kernels bound by the matrix cores and the feed from L2
+  int rc = no_wide(flags) ? 0 : xsd_dl(dtype, g, block, sp_trans, dn_kc, out_nc, st);
+  if (rc < 0) return rc;
+  if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
+  rc = general_only(flags) ? 0 : xsd_fast64(dtype, g, block, sp_trans, dn_kc, out_nc, st);
   if (rc < 0) return rc;
   if (rc == 1) { BSP_LAUNCH_CHECK(); return BSP_OK; }
   switch (dtype) {

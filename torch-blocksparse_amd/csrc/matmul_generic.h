@@ -685,5 +685,7 @@ int xsd_generic_f32(const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool
 // specialised block-64 16-bit kernels (matmul_fast64.hip): 1 = launched, 0 = not applicable, < 0 = error
 int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool b_kc, hipStream_t st);
 int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
+// dsd / dds for a wide free dimension at blocks 64 / 128, 16-bit (matmul_dl.hip): same return convention
+int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
 
 }  // namespace bsp

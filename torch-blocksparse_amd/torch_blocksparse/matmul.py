@@ -381,7 +381,24 @@ class _sparse_matmul(torch.autograd.Function):
             lut.gplan = GroupPlan.build(layout, trans, dev, thin_min=GroupPlan.thin_min(layout, trans, block, nnz=nnz),
                                         order_buckets=GroupPlan.order_buckets(layout, trans, block),
                                         split_len=GroupPlan.SPLIT_LEN if block == 64 else 0, ctx=ctx)
+        # blocks of 32 with a wide free dimension take a kernel of their own (dense tiles shared by the four lines of a
+        # group): its plan has no chains and runs head by head; built when such a product first comes
+        lut.gplan_wide = None
+        if block == 32:
+            lut.build_wide = lambda: GroupPlan.build(layout, trans, dev, thin_min=0, order_buckets=1, ctx=ctx)
         return lut, num_locks.value, width.value, None
+
+    @staticmethod
+    def _plan_for(lut, block, free_dim, dtype, dense_k_contiguous):
+        """The group plan that goes with a dsd / dds launch: the wide-free-dimension plan for blocks of 32 (16-bit types,
+        256 dense rows or more, dense operand with the reduction contiguous: the products the wide kernel takes), else
+        the table's ordinary plan."""
+        if (block == 32 and free_dim >= 256 and dtype != torch.float32 and dense_k_contiguous
+                and getattr(lut, 'build_wide', None) is not None):
+            if lut.gplan_wide is None:
+                lut.gplan_wide = lut.build_wide()
+            return lut.gplan_wide
+        return getattr(lut, 'gplan', None)
 
     @staticmethod
     def _pad_free_dim(x, dim, v):
@@ -409,7 +426,7 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dds_matmul(_lib.DTYPES[a.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), a.size(0), M, a.stride(0), a.stride(1), a.stride(2), b_sz, c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
-                                        *GroupPlan.xsd_args(getattr(lut, 'gplan', None), M, a.size(0)), KERNEL_FLAGS,
+                                        *GroupPlan.xsd_args(_sparse_matmul._plan_for(lut, block, M, a.dtype, not trans_a), M, a.size(0)), KERNEL_FLAGS,
                                         _lib.stream_ptr(a.device))
         _lib.check(rc, 'bsp_dds_matmul')
         time[0] = timer.done()
@@ -434,7 +451,7 @@ class _sparse_matmul(torch.autograd.Function):
         rc = _lib.load().bsp_dsd_matmul(_lib.DTYPES[b.dtype], _lib.ptr(a), _lib.ptr(b), _lib.ptr(c), int(trans_a), int(trans_b),
                                         int(trans_c), b.size(0), N, a_sz, b.stride(0), b.stride(1), b.stride(2), c.stride(0),
                                         c.stride(1), c.stride(2), block, _lib.ptr(lut), _lib.ptr(lut.planbuf), width,
-                                        *GroupPlan.xsd_args(getattr(lut, 'gplan', None), N, b.size(0)), KERNEL_FLAGS,
+                                        *GroupPlan.xsd_args(_sparse_matmul._plan_for(lut, block, N, b.dtype, bool(trans_b)), N, b.size(0)), KERNEL_FLAGS,
                                         _lib.stream_ptr(b.device))
         _lib.check(rc, 'bsp_dsd_matmul')
         time[0] = timer.done()
