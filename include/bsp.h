@@ -155,7 +155,8 @@ typedef enum {
  * tiles inside each group may take the launch.  The plan describes the whole layout, not one pack level: if that
  * kernel ran, the return value is BSP_OK_WHOLE_LAYOUT and the caller skips the remaining pack levels (pass the plan
  * with the first level only).  A caller that has the plan but has not built the table yet (its greedy packing is the
- * one sequential step of the builders) may call with d_lut = NULL, pack = 0, n_groups = 0: the result is
+ * one sequential step of the builders) may call with d_lut = NULL, pack = 0 and n_groups = the number of block-columns
+ * of the layout (0 if unknown: the kernels for long reductions at blocks of 32 then do not apply): the result is
  * BSP_OK_WHOLE_LAYOUT if a kernel that works from the plan alone took the product, else BSP_NEEDS_TABLE and nothing was
  * launched. */
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,

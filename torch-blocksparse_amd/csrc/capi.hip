@@ -55,7 +55,14 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   // op(A)[m][k]: reduction contiguous unless A is read transposed; op(B)[k][n]: contiguous when B is read transposed
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);
-  int rc = general_only(flags) ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
+  int rc = 0;
+  if (!d_lut) {   // the plan alone: n_groups then carries the number of block-columns of the layout
+    g.cols = (int)n_groups; g.n_groups = 0;
+    rc = no_wide(flags) ? 0 : sdd_dl(dtype, g, block, a_kc, b_kc, st);
+    if (rc < 0) return rc;
+    if (rc == 2) { BSP_LAUNCH_CHECK(); return BSP_OK_WHOLE_LAYOUT; }
+  }
+  rc = general_only(flags) ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
   if (rc < 0) return rc;
   if (rc >= 1) { BSP_LAUNCH_CHECK(); return rc == 2 ? BSP_OK_WHOLE_LAYOUT : BSP_OK; }
   if (!d_lut) return BSP_NEEDS_TABLE;      // a call with the plan alone, and no kernel that works from the plan applies

@@ -447,6 +447,184 @@ template <typename T> int launch_rg_dl(const XsdArgs &g, bool sp_trans, bool dn_
   return BSP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// sdd with a long reduction (hundreds of elements or more), blocks of 32, fp16 / bf16.  One output block is a 32 x 32
+// product: a workgroup per block (or per 2 x 2 pack of the reference's table) fetches 2 + 2 KiB per 65 kflop and is bound
+// by the feed from L2 at a thirteenth of the matrix peak.  Here a workgroup takes a group of four consecutive block-rows
+// (128 rows of A, the group plan of bsp_group_plan_build) and eight of the block-columns in which any of them has a
+// block (256 rows of B, gathered), and runs the dense 128 x 256 product over the whole reduction with the pipeline
+// of k_xsd_dl; only the blocks that exist are written.  Computing the absent ones as well costs matrix time that the
+// launch has to spare (it waits for operands either way) and removes all bookkeeping from the reduction loop: no
+// table is read in it.  Operand bytes per useful flop drop by 2 at a quarter of the blocks kept.
+// ---------------------------------------------------------------------------------------------------------
+constexpr int kSddCols = 8;      // block-columns per workgroup
+
+template <typename T, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) k_sdd_rg_dl(SddArgs g, int chunks) {
+  typedef Mma<T, 32> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int B = 32, G = BSP_GROUP, J = kSddCols, TM = G * B, TN = J * B;
+  static_assert(TN == kTN, "the gathered B tile is the dense tile of the other kernels");
+  typedef DlTile<T, TM, A_KC> XT;
+  typedef DlTile<T, TN, B_KC> YT;
+  constexpr int STAGE = XT::BYTES + YT::BYTES;
+  constexpr int XL = XT::LOADS / 4, YL = YT::LOADS / 4, L = XL + YL;
+  constexpr int RM = 2, RN = 4;                       // 2 x 2 wavefronts of 64 x 128
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t per_z = (int64_t)g.n_pgroups * chunks;
+  const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
+  const int z = (int)(w / per_z);
+  const int chunk = (int)((w % per_z) % chunks);      // chunk fastest: the chunks of a group share its rows of A in L2
+  const table_ptr hd = as_table(g.gplan) + 4 * ((w % per_z) / chunks);
+  const int e0 = hd[0], ne = hd[1], h = hd[2], code = hd[3];
+  if (chunk * J >= ne) return;                        // (the grid is sized for the longest possible group)
+  const int left = ne - chunk * J;                    // entries of this chunk: min(left, J)
+  const int line0 = (code & 0xffffff) * G;
+  const int rows_a = g.lines * B;                     // rows of op(A) per head
+  const int64_t lda = g.lda, ldb = g.ldb;
+  const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh;
+  const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh;
+
+  // Loop-invariant part of every load address.  A: rows line0 * 32 .. + 127 (rows past the end of the matrix read its
+  // last rows; their blocks do not exist).  B: row n of the tile is row n % 32 of block-column pos[n / 32].
+  int64_t xoff[XL], yoff[YL];
+#pragma unroll
+  for (int i = 0; i < XL; i++) {
+    const int ld = wave * XL + i;
+    if constexpr (A_KC) {
+      const int row = ld * 16 + (lane >> 2), chunk16 = (lane & 3) ^ ((row >> 1) & 3);
+      const int r = line0 * B + row < rows_a ? line0 * B + row : rows_a - 1;
+      xoff[i] = (int64_t)r * lda + chunk16 * 8;
+    } else {
+      constexpr int CPR = TM / 8;
+      const int j = ld * 64 + lane, k = j / CPR, slot = j % CPR;
+      const int c = (((slot >> 1) ^ ks_swz<TM>(k)) << 1) | (slot & 1);
+      const int r = line0 * B + c * 8 < rows_a ? line0 * B + c * 8 : rows_a - 8;
+      xoff[i] = (int64_t)k * lda + r;
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < YL; i++) {
+    const int ld = wave * YL + i;
+    if constexpr (B_KC) {
+      const int row = ld * 16 + (lane >> 2), chunk16 = (lane & 3) ^ ((row >> 1) & 3);
+      const int jj = row >> 5;
+      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J + (jj < left ? jj : left - 1))];
+      yoff[i] = ((int64_t)pos * B + (row & 31)) * ldb + chunk16 * 8;
+    } else {
+      constexpr int CPR = TN / 8;
+      const int j = ld * 64 + lane, k = j / CPR, slot = j % CPR;
+      const int c = (((slot >> 1) ^ ks_swz<TN>(k)) << 1) | (slot & 1);
+      const int jj = c >> 2;                          // four chunks of 8 columns per block-column
+      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J + (jj < left ? jj : left - 1))];
+      yoff[i] = (int64_t)k * ldb + (int64_t)pos * B + (c & 3) * 8;
+    }
+  }
+  typename M::acc_t acc[RM][RN];
+#pragma unroll
+  for (int i = 0; i < RM; i++)
+#pragma unroll
+    for (int j = 0; j < RN; j++)
+#pragma unroll
+      for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
+  const int ksteps = g.K / kTK;
+  auto issue = [&](int s) {
+    const int64_t k0 = (int64_t)(s < ksteps ? s : ksteps - 1) * kTK;
+    const T *xb = pa + (A_KC ? k0 : k0 * lda);
+    const T *yb = pb + (B_KC ? k0 : k0 * ldb);
+    unsigned char *st = smem + (s % kStages) * STAGE;
+#pragma unroll
+    for (int i = 0; i < XL; i++)
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(xb + xoff[i]), BSP_LDS_PTR(st + (wave * XL + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < YL; i++)
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(yb + yoff[i]), BSP_LDS_PTR(st + XT::BYTES + (wave * YL + i) * 1024), 16, 0, 0);
+  };
+#pragma unroll
+  for (int s = 0; s < kStages - 1; s++) issue(s);
+  for (int s = 0; s < ksteps; s++) {
+    BSP_WAIT_VM(L * (kStages - 2));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    issue(s + kStages - 1);
+    const unsigned char *st = smem + (s % kStages) * STAGE;
+#pragma unroll
+    for (int kk = 0; kk < kTK / 16; kk++) {
+      frag_t xf[RM], yf[RN];
+#pragma unroll
+      for (int i = 0; i < RM; i++) xf[i] = XT::frag(st, (wm * RM + i) * 32, kk, lane);
+#pragma unroll
+      for (int j = 0; j < RN; j++) yf[j] = YT::frag(st + XT::BYTES, (wn * RN + j) * 32, kk, lane);
+#pragma unroll
+      for (int i = 0; i < RM; i++)
+#pragma unroll
+        for (int j = 0; j < RN; j++) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // 4 consecutive values run along the block's columns
+    }
+  }
+  BSP_WAIT_VM(0);
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  // epilogue: the 128 x 256 tile through LDS, then the blocks that exist, each 2 KiB of consecutive addresses
+  constexpr int LDR = TN + 8;
+  static_assert(TM * LDR * 2 <= kStages * STAGE, "the staged tile fits into the ring");
+  T *stage = reinterpret_cast<T *>(smem);
+#pragma unroll
+  for (int i = 0; i < RM; i++)
+#pragma unroll
+    for (int j = 0; j < RN; j++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int row = (wm * RM + i) * 32 + (lane & 31), col = (wn * RN + j) * 32 + 8 * g4 + 4 * (lane >> 5);
+        union { u32x2 raw; T e[4]; } u;
+#pragma unroll
+        for (int e = 0; e < 4; e++) u.e[e] = from_float<T>(acc[i][j][4 * g4 + e]);
+        *reinterpret_cast<u32x2 *>(stage + row * LDR + col) = u.raw;
+      }
+  __syncthreads();
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
+  const int32_t *ids = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J);   // vector loads: the id differs from lane to lane
+  constexpr int CPB = B * B / 8;                      // 16-byte chunks per block
+#pragma unroll 4
+  for (int c = tid; c < G * J * CPB; c += 256) {
+    const int blk = c / CPB, within = c % CPB;
+    const int m = blk / J, jj = blk % J;
+    const int id = jj < left ? ids[(G + 1) * jj + 1 + m] : -1;
+    if (id >= 0) {
+      const int r = within >> 2, cc = (within & 3) * 8;
+      *reinterpret_cast<u32x4 *>(pc + (int64_t)id * (B * B) + within * 8) = *reinterpret_cast<const u32x4 *>(stage + (m * B + r) * LDR + jj * B + cc);
+    }
+  }
+}
+
+template <typename T> int launch_sdd_rg_dl(const SddArgs &g, bool a_kc, bool b_kc, hipStream_t st) {
+  const int chunks = (g.cols + kSddCols - 1) / kSddCols;
+  const int64_t n_wg = (int64_t)g.n_pgroups * chunks * g.Z;
+  if (n_wg <= 0) return BSP_OK;
+  if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  constexpr int SMEM = kStages * (BSP_GROUP * 32 + kTN) * kTK * 2;
+  dim3 grid((unsigned)n_wg), wg(256);
+#define BSP_SDD_RG_LAUNCH(AK, BK)                                                                                       \
+  do {                                                                                                                  \
+    static bool attr_set = false;                                                                                       \
+    if (!attr_set) {                                                                                                    \
+      if (hipFuncSetAttribute((const void *)k_sdd_rg_dl<T, AK, BK>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != \
+          hipSuccess) return BSP_ERR_HIP;                                                                               \
+      attr_set = true;                                                                                                  \
+    }                                                                                                                   \
+    hipLaunchKernelGGL((k_sdd_rg_dl<T, AK, BK>), grid, wg, SMEM, st, g, chunks);                                       \
+  } while (0)
+  if (a_kc && b_kc) BSP_SDD_RG_LAUNCH(true, true);
+  else if (a_kc) BSP_SDD_RG_LAUNCH(true, false);
+  else if (b_kc) BSP_SDD_RG_LAUNCH(false, true);
+  else BSP_SDD_RG_LAUNCH(false, false);
+#undef BSP_SDD_RG_LAUNCH
+  return BSP_OK;
+}
+
 template <typename T, int BLOCK> int launch_dl(const XsdArgs &g0, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
   const int64_t n_wg = (int64_t)g0.width * ((g0.NF + kTN - 1) / kTN) * g0.Z;
   if (n_wg <= 0) return BSP_OK;
@@ -499,6 +677,15 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
   if (dtype == BSP_F16) rc = block == 128 ? launch_dl<f16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<f16, 64>(g, sp_trans, dn_kc, out_nc, st);
   else rc = block == 128 ? launch_dl<bf16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<bf16, 64>(g, sp_trans, dn_kc, out_nc, st);
   return rc == BSP_OK ? 1 : rc;
+}
+
+// sdd with a long reduction at blocks of 32 from the group plan alone: 2 = launched (every block of the layout is
+// written), 0 = not applicable, < 0 = error
+int sdd_dl(int dtype, const SddArgs &g, int block, bool a_kc, bool b_kc, hipStream_t st) {
+  if (dtype == BSP_F32 || block != 32 || !g.gplan || g.n_pgroups <= 0 || g.lines <= 0 || g.cols <= 0) return 0;
+  if (g.K < 256 || g.K % kTK) return 0;
+  const int rc = dtype == BSP_F16 ? launch_sdd_rg_dl<f16>(g, a_kc, b_kc, st) : launch_sdd_rg_dl<bf16>(g, a_kc, b_kc, st);
+  return rc == BSP_OK ? 2 : rc;
 }
 
 }  // namespace bsp

@@ -361,6 +361,7 @@ struct SddArgs {
   const int32_t *lut; const uint8_t *valid;
   int64_t n_groups;
   const int32_t *gplan; int n_pgroups; int lines;   // optional group plan (by rows), its groups, block-rows per head
+  int cols = 0;                                       // block-columns per head when known (a call with the plan alone), else 0
 };
 
 template <typename T, int BLOCK, int PACK, bool KCONTIG> struct SddView {
@@ -687,5 +688,7 @@ int sdd_fast64(int dtype, const SddArgs &g, int block, int pack, bool a_kc, bool
 int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
 // dsd / dds for a wide free dimension at blocks 64 / 128, 16-bit (matmul_dl.hip): same return convention
 int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
+// sdd with a long reduction at blocks of 32, from the group plan alone (matmul_dl.hip): 2 = launched and every block written
+int sdd_dl(int dtype, const SddArgs &g, int block, bool a_kc, bool b_kc, hipStream_t st);
 
 }  // namespace bsp

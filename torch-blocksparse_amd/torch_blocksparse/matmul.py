@@ -224,6 +224,8 @@ class SddTables(list):
     gplan = None
     spdims = None
     build = None          # callable -> (tables, widths, packs), or None when the list is complete
+    gplan_long = None     # block 32: the plan of the long-reduction kernel (head by head), built by build_long on demand
+    build_long = None
     widths = None
     packs = None
 
@@ -294,6 +296,12 @@ class _sparse_matmul(torch.autograd.Function):
             luts.gplan = GroupPlan.build_coarse(layout, block, True, dev, for_sdd=True, ctx=ctx) if block == 16 else None
             if luts.gplan is None:
                 luts.gplan = GroupPlan.build(layout, True, dev, thin_min=0, ctx=ctx)
+        # blocks of 32 with a long reduction take a kernel of their own, whose plan runs head by head (the workgroups on
+        # an XCD at one time then read the same rows of B; the attention-shape kernels prefer the longest group first:
+        # measured 0.64 against 0.67 ms per attention step); built when such a product first comes
+        luts.gplan_long = None
+        if block == 32:
+            luts.build_long = lambda: GroupPlan.build(layout, True, dev, thin_min=0, order_buckets=1, ctx=ctx)
         if lazy and luts.gplan is not None:
             return luts, None, None, None
         widths, packs = luts.materialize()
@@ -325,9 +333,17 @@ class _sparse_matmul(torch.autograd.Function):
         # nothing was launched (NEEDS_TABLE), the tables are built and the plan goes with the first pack level.
         gplan = GroupPlan.args(getattr(luts, 'gplan', None))
         rc = _lib.NEEDS_TABLE
-        if lazy and luts.build is not None and luts.gplan is not None:
-            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), 0, gplan[0], gplan[1], gplan[2], KERNEL_FLAGS,
-                                    _lib.stream_ptr(a.device))
+        long_k = lazy and block == 32 and AS3 >= 256 and a.dtype != torch.float32 and getattr(luts, 'build_long', None) is not None
+        if long_k:
+            # the kernel for long reductions works from its own plan, whether the tables exist or not
+            if luts.gplan_long is None:
+                luts.gplan_long = luts.build_long()
+            lp = GroupPlan.args(luts.gplan_long)
+            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), spdims[2], lp[0], lp[1], lp[2],
+                                    KERNEL_FLAGS, _lib.stream_ptr(a.device))
+        elif lazy and luts.gplan is not None and luts.build is not None:
+            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), spdims[2], gplan[0], gplan[1], gplan[2],
+                                    KERNEL_FLAGS, _lib.stream_ptr(a.device))
             if rc not in (_lib.OK_WHOLE_LAYOUT, _lib.NEEDS_TABLE):
                 _lib.check(rc, 'bsp_sdd_matmul')
         if rc == _lib.NEEDS_TABLE:
