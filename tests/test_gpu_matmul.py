@@ -292,3 +292,70 @@ def test_random_attention_shapes_specialised_against_general(monkeypatch):
         monkeypatch.setattr(matmul, 'KERNEL_FLAGS', 0)
         tol = (2e-2 if dtype == torch.bfloat16 else 4e-3) * (float(y.abs().max()) + 1e-6)
         assert torch.isfinite(x).all() and float((x - y).abs().max()) <= tol, (it, mode, block, H, R, C, Z, free, dtype)
+
+
+@pytest.mark.parametrize('block', [32, 64, 128])
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_wide_free_dimension_kernels(block, dtype):
+    # dsd / dds with 256 dense rows or more take the kernels that load straight into LDS (blocks 64 and 128; block 32
+    # through row groups that share the dense tiles): every orientation, a free dimension that does not fill its last
+    # 256-wide tile (328) and one of exactly two tiles, an empty line, a full line, a number of lines that is not a
+    # multiple of the group size
+    n = 9 if block == 128 else 11
+    lay = random_layout((2, n, n), 0.35, 900 + block)
+    lay[:, 3, :] = 0
+    lay[:, :, 4] = 0
+    lay[0, 5, :] = 1
+    lay[1, :, 6] = 1
+    lay[:, 3, :] = 0
+    lay[:, :, 4] = 0
+    lay[:, 0, 0] = 1
+    for free in (328, 512):
+        for ta in (False, True):
+            for tb_ in (False, True):
+                run_case('dsd', ta, tb_, block, dtype, Z=2, H=2, M=n * block, K=n * block, N=free, layout=lay, seed=free + block, dist='randn',
+                         scale=0.2, backward=False)
+                run_case('dds', ta, tb_, block, dtype, Z=2, H=2, M=free, K=n * block, N=n * block, layout=lay, seed=free + block + 1,
+                         dist='randn', scale=0.2, backward=False)
+    # forward and backward once (the backward products are dsd / dds / sdd calls of their own, written transposed)
+    run_case('dsd', False, False, block, dtype, Z=2, H=2, M=n * block, K=n * block, N=320, layout=lay, seed=block, dist='randn', scale=0.2)
+    run_case('dds', False, True, block, dtype, Z=2, H=2, M=320, K=n * block, N=n * block, layout=lay, seed=block + 5, dist='randn', scale=0.2)
+
+
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_sdd_with_a_long_reduction_at_block_32(dtype):
+    # reductions of 256 and more at blocks of 32 run dense 128 x 256 tiles over a row group and eight of its block-columns
+    # and write only the blocks that exist: 22 block-rows (the last group has two lines), 19 block-columns (three chunks,
+    # the last one ragged), an empty row, an empty column, a full row; all four operand orientations
+    lay = random_layout((3, 22, 19), 0.3, 3232)
+    lay[:, 7, :] = 0
+    lay[:, :, 11] = 0
+    lay[1, 20, :] = 1
+    lay[:, 7, :] = 0
+    lay[:, :, 11] = 0
+    lay[:, 0, 0] = 1
+    for K in (256, 352):
+        for ta in (False, True):
+            for tb_ in (False, True):
+                run_case('sdd', ta, tb_, 32, dtype, Z=2, H=3, M=22 * 32, N=19 * 32, K=K, layout=lay, seed=K, dist='randn', scale=0.2, backward=False)
+    run_case('sdd', False, True, 32, dtype, Z=2, H=3, M=22 * 32, N=19 * 32, K=320, layout=lay, seed=7, dist='randn', scale=0.2)
+
+
+def test_wide_kernels_agree_with_the_general_ones(monkeypatch):
+    # the same launches with and without the wide-free-dimension / long-reduction kernels (a launch flag of the C ABI)
+    from torch_blocksparse import _lib, matmul
+    torch.manual_seed(77)
+    for block in (32, 64, 128):
+        lay = random_layout((2, 6, 7), 0.4, 70 + block)
+        nnz = int(lay.sum())
+        sp = torch.randn(2, nnz, block, block, device=DEV, dtype=torch.float16)
+        dn = torch.randn(2, 2, 7 * block, 512, device=DEV, dtype=torch.float16)
+        a, b = torch.randn(2, 2, 6 * block, 512, device=DEV, dtype=torch.float16), torch.randn(2, 2, 7 * block, 512, device=DEV, dtype=torch.float16)
+        outs = []
+        for flags in (0, _lib.FLAG_NO_WIDE):
+            monkeypatch.setattr(matmul, 'KERNEL_FLAGS', flags)
+            outs.append((tb.MatMul(lay, block, 'dsd')(sp, dn), tb.MatMul(lay, block, 'sdd', trans_b=True)(a, b)))
+        monkeypatch.setattr(matmul, 'KERNEL_FLAGS', 0)
+        for x, y in zip(*outs):
+            tol = 4e-3 * (float(y.float().abs().max()) + 1e-6)
+            assert float((x.float() - y.float()).abs().max()) <= tol

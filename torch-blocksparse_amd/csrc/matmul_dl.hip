@@ -673,6 +673,9 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
     return rc == BSP_OK ? 1 : rc;
   }
   if (block != 64 && block != 128) return 0;
+  // (sparse operand transposed and dense operand with the reduction contiguous, the dX product of a sparse linear layer:
+  // measured 0.064 ms here against 0.059 ms for the general kernel at block 128, equal at block 64: left where it was)
+  if (sp_trans && dn_kc) return 0;
   int rc;
   if (dtype == BSP_F16) rc = block == 128 ? launch_dl<f16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<f16, 64>(g, sp_trans, dn_kc, out_nc, st);
   else rc = block == 128 ? launch_dl<bf16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<bf16, 64>(g, sp_trans, dn_kc, out_nc, st);
