@@ -494,16 +494,22 @@ def record_traffic(fetch_dir, write_dir):
         return 268435456.0 / (sum(vals) / len(vals))
     fs, ws = copy_scale(fetch), copy_scale(write)
 
-    def kernel_bytes(sub, *more):
+    split = {}
+
+    def kernel_bytes(name, sub, *more):
         def pick(per):
             vals = [v for k, vs in per.items() if sub in k and all(m in k for m in more) for v in vs]
             return sum(vals) / len(vals)
-        return int(pick(fetch) * fs + pick(write) * ws)
-    per_kernel = {'k_sdd64_rg': kernel_bytes('k_sdd64_rg'), 'k_xsd64_rg<sparse operand as stored>': kernel_bytes('k_xsd64_rg', 'Lb0E'),
-                  'k_xsd64_rg<sparse operand transposed>': kernel_bytes('k_xsd64_rg', 'Lb1E'),
-                  'k_softmax_fwd': kernel_bytes('k_softmax_fwd'), 'k_softmax_bwd': kernel_bytes('k_softmax_bwd')}
+        split[name] = {'FETCH_SIZE_KiB': round(pick(fetch)), 'WRITE_SIZE_KiB': round(pick(write)),
+                       'read_bytes': int(pick(fetch) * fs), 'written_bytes': int(pick(write) * ws)}
+        return split[name]['read_bytes'] + split[name]['written_bytes']
+    per_kernel = {name: kernel_bytes(name, *subs) for name, subs in (
+        ('k_sdd64_rg', ('k_sdd64_rg',)), ('k_xsd64_rg<sparse operand as stored>', ('k_xsd64_rg', 'Lb0E')),
+        ('k_xsd64_rg<sparse operand transposed>', ('k_xsd64_rg', 'Lb1E')), ('k_softmax_fwd', ('k_softmax_fwd',)),
+        ('k_softmax_bwd', ('k_softmax_bwd',)))}
     rec = {'kernel_sources_sha256': kernel_sources_sha(), 'bytes_per_counted_KiB': {'FETCH_SIZE': round(fs, 1), 'WRITE_SIZE': round(ws, 1)},
-           'bytes_per_kernel_launch': per_kernel, 'bytes_per_launch': {name: per_kernel[k] for name, k in KERNEL_OF.items()},
+           'bytes_per_kernel_launch': per_kernel, 'counters_per_kernel_launch': split,
+           'bytes_per_launch': {name: per_kernel[k] for name, k in KERNEL_OF.items()},
            'note': 'averages over the launches of each kernel in a 3-step run; launches of one kernel share a figure'}
     with open(TRAFFIC_FILE, 'w') as f:
         json.dump(rec, f, indent=1)

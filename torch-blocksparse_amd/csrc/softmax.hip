@@ -131,16 +131,25 @@ template <typename T, int BLOCK> struct Unit {
     const int64_t u = wg * wpg + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     ok = u < n_units;
     const int lane = threadIdx.x & 63;
-    const int g = (int)(u % GE::G);
+    int g = (int)(u % GE::G);
     const int64_t t = u / GE::G;
     // Block-rows are taken from the last one down.  The matmul kernels on either side of this one walk a causal
     // layout from its longest rows (the last ones) to its shortest, so this order reads first what the producer wrote
     // last; measured in the attention chain it makes this kernel and its consumer 3-5 % faster than the ascending order.
     if (shared_masks) {
-      const int R = HR / H;
-      z = (int)(t % Z);
-      const int64_t t2 = t / Z;
-      hr = (int)(t2 % H) * R + (R - 1 - (int)((t2 / H) % R));
+      // (batch, head) fastest: the wavefronts of a workgroup then read the same mask rows at the same time, and all but
+      // the first find them in the vector cache of their CU instead of fetching them from L2 again
+      const int R = HR / H, ZH = Z * H;
+      const int zh = (int)(u % ZH);
+      const int64_t t2 = u / ZH;
+      z = zh % Z;
+      g = (int)(t2 % GE::G);
+      // An XCD works on a contiguous eighth of the units.  Block-rows are dealt to the eighths in turn, so that each XCD
+      // gets short and long rows of a causal layout alike (an XCD draws about its share of the memory bandwidth: the one
+      // with the longest rows would finish last).
+      int br = (int)((t2 / GE::G) % R);
+      if (R % 8 == 0) br = (br % (R / 8)) * 8 + br / (R / 8);
+      hr = (zh / Z) * R + (R - 1 - br);
     } else {
       hr = HR - 1 - (int)(t % HR);
       z = (int)(t / HR);
