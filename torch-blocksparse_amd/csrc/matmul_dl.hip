@@ -16,9 +16,22 @@
 // A standalone dense probe of this pipeline (128 x 256 x 32 tiles) reaches 0.9 PFLOP/s on an 8192 x 4096 x 4096
 // product where the register-staged general kernel reaches 0.75.
 #include "matmul_generic.h"
+#include <atomic>
 
 namespace bsp {
 namespace {
+
+// The kernels of this file use more dynamic LDS than a launch may ask for by default: the limit of a kernel is raised
+// once per device (a bit per device; devices past the 64th set it at every launch), from whichever thread gets there.
+inline bool raise_lds_limit(const void *kernel, int bytes, std::atomic<uint64_t> &done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = dev < 64 ? uint64_t(1) << dev : 0;
+  if (bit && (done.load(std::memory_order_acquire) & bit)) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) return false;
+  done.fetch_or(bit, std::memory_order_release);
+  return true;
+}
 
 #define BSP_GLOBAL_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
 #define BSP_LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
@@ -424,12 +437,8 @@ template <typename T> int launch_rg_dl(const XsdArgs &g, bool sp_trans, bool dn_
   dim3 grid((unsigned)n_wg), wg(256);
 #define BSP_RG_LAUNCH(ST, DK, ON)                                                                                       \
   do {                                                                                                                  \
-    static bool attr_set = false;                                                                                       \
-    if (!attr_set) {                                                                                                    \
-      if (hipFuncSetAttribute((const void *)k_xsd_rg_dl<T, ST, DK, ON>, hipFuncAttributeMaxDynamicSharedMemorySize,     \
-                              SMEM) != hipSuccess) return BSP_ERR_HIP;                                                  \
-      attr_set = true;                                                                                                  \
-    }                                                                                                                   \
+    static std::atomic<uint64_t> done{0};                                                                               \
+    if (!raise_lds_limit((const void *)k_xsd_rg_dl<T, ST, DK, ON>, SMEM, done)) return BSP_ERR_HIP;                     \
     hipLaunchKernelGGL((k_xsd_rg_dl<T, ST, DK, ON>), grid, wg, SMEM, st, g);                                           \
   } while (0)
   const int key = (sp_trans ? 4 : 0) | (dn_kc ? 2 : 0) | (out_nc ? 1 : 0);
@@ -529,6 +538,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     for (int j = 0; j < RN; j++)
 #pragma unroll
       for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
+  // which of this wavefront's 2 x 4 blocks exist: the others are neither multiplied nor (if a whole row or column of
+  // them is absent) read from LDS.  The loads into LDS stay dense: their count per stage is fixed.
+  unsigned present = 0;
+  {
+    const table_ptr ids = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J);
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+#pragma unroll
+      for (int j = 0; j < RN; j++) {
+        const int m = wm * RM + i, jj = wn * RN + j;
+        const int id = ids[(G + 1) * (jj < left ? jj : left - 1) + 1 + m];
+        present |= (jj < left && id >= 0) ? 1u << (i * RN + j) : 0u;
+      }
+  }
   const int ksteps = g.K / kTK;
   auto issue = [&](int s) {
     const int64_t k0 = (int64_t)(s < ksteps ? s : ksteps - 1) * kTK;
@@ -553,15 +576,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const unsigned char *st = smem + (s % kStages) * STAGE;
 #pragma unroll
     for (int kk = 0; kk < kTK / 16; kk++) {
-      frag_t xf[RM], yf[RN];
+      frag_t xf[RM] = {}, yf[RN] = {};
 #pragma unroll
-      for (int i = 0; i < RM; i++) xf[i] = XT::frag(st, (wm * RM + i) * 32, kk, lane);
+      for (int i = 0; i < RM; i++)
+        if ((present >> (i * RN)) & ((1u << RN) - 1)) xf[i] = XT::frag(st, (wm * RM + i) * 32, kk, lane);
 #pragma unroll
-      for (int j = 0; j < RN; j++) yf[j] = YT::frag(st + XT::BYTES, (wn * RN + j) * 32, kk, lane);
+      for (int j = 0; j < RN; j++)
+        if ((present >> j) & 0x11u) yf[j] = YT::frag(st + XT::BYTES, (wn * RN + j) * 32, kk, lane);
+      static_assert(RM == 2 && RN == 4, "the column test above reads bits j and j + RN");
 #pragma unroll
       for (int i = 0; i < RM; i++)
 #pragma unroll
-        for (int j = 0; j < RN; j++) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // 4 consecutive values run along the block's columns
+        for (int j = 0; j < RN; j++)
+          if ((present >> (i * RN + j)) & 1u) acc[i][j] = M::run(yf[j], xf[i], acc[i][j]);   // 4 consecutive values run along the block's columns
     }
   }
   BSP_WAIT_VM(0);
@@ -609,12 +636,8 @@ template <typename T> int launch_sdd_rg_dl(const SddArgs &g, bool a_kc, bool b_k
   dim3 grid((unsigned)n_wg), wg(256);
 #define BSP_SDD_RG_LAUNCH(AK, BK)                                                                                       \
   do {                                                                                                                  \
-    static bool attr_set = false;                                                                                       \
-    if (!attr_set) {                                                                                                    \
-      if (hipFuncSetAttribute((const void *)k_sdd_rg_dl<T, AK, BK>, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != \
-          hipSuccess) return BSP_ERR_HIP;                                                                               \
-      attr_set = true;                                                                                                  \
-    }                                                                                                                   \
+    static std::atomic<uint64_t> done{0};                                                                               \
+    if (!raise_lds_limit((const void *)k_sdd_rg_dl<T, AK, BK>, SMEM, done)) return BSP_ERR_HIP;                         \
     hipLaunchKernelGGL((k_sdd_rg_dl<T, AK, BK>), grid, wg, SMEM, st, g, chunks);                                       \
   } while (0)
   if (a_kc && b_kc) BSP_SDD_RG_LAUNCH(true, true);
@@ -635,12 +658,8 @@ template <typename T, int BLOCK> int launch_dl(const XsdArgs &g0, bool sp_trans,
   dim3 grid((unsigned)n_wg), wg(256);
 #define BSP_DL_LAUNCH(ST, DK, ON)                                                                                       \
   do {                                                                                                                  \
-    static bool attr_set = false;   /* once per instantiation: more dynamic LDS than the default limit */              \
-    if (!attr_set) {                                                                                                    \
-      if (hipFuncSetAttribute((const void *)k_xsd_dl<T, BLOCK, ST, DK, ON>, hipFuncAttributeMaxDynamicSharedMemorySize, \
-                              SMEM) != hipSuccess) return BSP_ERR_HIP;                                                  \
-      attr_set = true;                                                                                                  \
-    }                                                                                                                   \
+    static std::atomic<uint64_t> done{0};                                                                               \
+    if (!raise_lds_limit((const void *)k_xsd_dl<T, BLOCK, ST, DK, ON>, SMEM, done)) return BSP_ERR_HIP;                 \
     hipLaunchKernelGGL((k_xsd_dl<T, BLOCK, ST, DK, ON>), grid, wg, SMEM, st, g);                                       \
   } while (0)
   const int key = (sp_trans ? 4 : 0) | (dn_kc ? 2 : 0) | (out_nc ? 1 : 0);
