@@ -13,6 +13,24 @@ def pytest_configure(config):
     config.addinivalue_line('markers', 'gpu: needs a real MI355X (run with -m gpu on the GPU box)')
 
 
+def pytest_terminal_summary(terminalreporter):
+    """What each comparison against the oracle actually reached (tests/helpers.py): the largest relative error where the
+    bound is purely relative, the largest used share of the tolerance where it has an absolute term."""
+    try:
+        from helpers import ACHIEVED
+    except ImportError:
+        return
+    if not ACHIEVED:
+        return
+    bound = {'float32': 1e-5, 'float16': 1e-2, 'bfloat16': 2e-2}
+    terminalreporter.write_sep('-', 'parity against the oracle: what the comparisons reached')
+    for (dtype, what, form), val in sorted(ACHIEVED.items()):
+        if form == 'pure':
+            terminalreporter.write_line('%-9s %-12s max relative error %.3g (bound %g, no absolute term)' % (dtype, what, val, bound[dtype]))
+        else:
+            terminalreporter.write_line('%-9s %-12s %.0f %% of the tolerance used at most' % (dtype, what, 100 * val))
+
+
 @pytest.fixture(scope='session')
 def golden():
     import json

@@ -119,6 +119,9 @@ class _sparse_softmax(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, dx):
+        """The gradient is computed in place, as in the reference (softmax.py:316-325): the tensor that comes in as the
+        gradient of the output holds the gradient of the input afterwards.  A caller that still needs the incoming
+        gradient after backward (retain_graph with a second backward, a hook that keeps it) passes a copy."""
         x, lut = ctx.saved_tensors
         if dx.shape != x.shape:
             raise ValueError('softmax gradient has shape %s, the output has %s' % (tuple(dx.shape), tuple(x.shape)))
