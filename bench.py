@@ -41,13 +41,26 @@ FP32_PEAK_TFLOPS = 157.3    # fp32 matrix
 
 TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'traffic_attention_seq4096_fp16_blk64.json')
 
-# kernel behind each launch of the step, for the per-kernel totals
+# kernel behind each launch of the step, for the per-kernel totals (the headline block size; kernel_of() for the others)
 KERNEL_OF = {
     'sdd_fwd  q.k^T': 'k_sdd64_rg', 'sdd_bwd  do.v^T': 'k_sdd64_rg',
     'dsd_fwd  p.v': 'k_xsd64_rg<sparse operand as stored>', 'dsd_bwd  ds.k': 'k_xsd64_rg<sparse operand as stored>',
     'dsd_bwd  p^T.do': 'k_xsd64_rg<sparse operand transposed>', 'dds_bwd  (q^T.ds)^T': 'k_xsd64_rg<sparse operand transposed>',
     'softmax_fwd': 'k_softmax_fwd', 'softmax_bwd': 'k_softmax_bwd',
 }
+
+
+def kernel_of(block):
+    """--block 32 runs the one-member-per-wavefront kernels, --block 16 the block-64 kernels on gathered 4 x 4 tiles."""
+    if block == 64:
+        return KERNEL_OF
+    def ren(k):
+        if block == 32:
+            return k.replace('k_sdd64_rg', 'k_sdd_rg_small').replace('k_xsd64_rg', 'k_xsd_rg_small')
+        if '64_rg' not in k:
+            return k
+        return k.replace('>', ', tiles of 4 x 4 blocks>') if '<' in k else k + '<tiles of 4 x 4 blocks>'
+    return {name: ren(k) for name, k in KERNEL_OF.items()}
 
 
 def kernel_sources_sha():
@@ -141,7 +154,7 @@ def main():
     # the dominant kernel = the one with the largest total time per step over all its launches
     per_kernel = {}
     for name, ent in kernels.items():
-        k = per_kernel.setdefault(KERNEL_OF[name], {'launches_per_step': 0, 'ms_per_step': 0.0, 'bytes': 0, 'traffic': 0, 'have_traffic': True})
+        k = per_kernel.setdefault(kernel_of(args.block)[name], {'launches_per_step': 0, 'ms_per_step': 0.0, 'bytes': 0, 'traffic': 0, 'have_traffic': True})
         k['launches_per_step'] += 1
         k['ms_per_step'] += ent['ms']
         k['bytes'] += ent['bytes']
