@@ -246,11 +246,42 @@ def test_separate_projection_weights_and_no_bias():
     assert_close(got, ref.float(), torch.float16, 'separate projection weights')
 
 
-def test_extra_key_position_is_refused():
-    lay = torch.ones(2, 4, 4, dtype=torch.int64)
-    for kw in (dict(add_bias_kv=True), dict(add_zero_attn=True)):
-        with pytest.raises(NotImplementedError):
-            tb.MultiheadAttention(64, 2, lay, 16, **kw)
+@pytest.mark.parametrize('bias_kv,zero_attn', [(True, False), (False, True), (True, True)])
+def test_extra_key_positions_against_torch(bias_kv, zero_attn):
+    # add_bias_kv / add_zero_attn append one key position each, visible to every query.  Against nn.MultiheadAttention
+    # itself in fp32 with the same weights: the block layout (banded, with a global first column) is handed to torch as
+    # an additive mask, which torch pads with zeros for the appended positions; with a key padding mask, forward and
+    # backward.  The sparse module keeps the positions in one more block-column whose padding it hides itself.
+    import copy
+    torch.manual_seed(41)
+    E, heads, L, B, block = 64, 2, 128, 3, 16
+    nb = L // block
+    lay = torch.zeros(heads, nb, nb, dtype=torch.int64)
+    for i in range(nb):
+        lay[:, i, max(0, i - 1):i + 1] = 1
+    lay[:, :, 0] = 1
+    lay[1, 2, 5] = 1
+    dense = torch.nn.MultiheadAttention(E, heads, add_bias_kv=bias_kv, add_zero_attn=zero_attn).to(DEV)
+    sparse = tb.MultiheadAttention(E, heads, lay, block, add_bias_kv=bias_kv, add_zero_attn=zero_attn,
+                                   key_padding_mask_mode='mul', attn_mask_mode='add').to(DEV)
+    sparse.load_state_dict(dense.state_dict())
+    x = torch.randn(L, B, E, device=DEV)
+    pad = torch.zeros(B, L, dtype=torch.bool, device=DEV)
+    pad[2, 90:] = True
+    outside = (lay == 0).repeat_interleave(block, 1).repeat_interleave(block, 2)          # [heads, L, L]
+    layout_mask = torch.zeros(heads, L, L).masked_fill(outside, float('-inf')).to(DEV)
+    xd, xs = x.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    yd, _ = dense(xd, xd, xd, key_padding_mask=pad, attn_mask=layout_mask.repeat(B, 1, 1), need_weights=False)
+    ys, _ = sparse(xs, xs, xs, key_padding_mask=(~pad).float())
+    g = torch.randn_like(yd)
+    yd.backward(g)
+    ys.backward(g)
+    pairs = [('output', ys, yd), ('input gradient', xs.grad, xd.grad), ('in_proj gradient', sparse.in_proj_weight.grad, dense.in_proj_weight.grad)]
+    if bias_kv:
+        pairs += [('bias_k gradient', sparse.bias_k.grad, dense.bias_k.grad), ('bias_v gradient', sparse.bias_v.grad, dense.bias_v.grad)]
+    for name, got, ref in pairs:
+        err = float((got.detach() - ref.detach()).abs().max())
+        assert err <= 1e-4 * float(ref.detach().abs().max()), 'extra key positions, %s: max err %g' % (name, err)
 
 
 def test_multihead_attention_with_dropout():

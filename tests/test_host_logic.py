@@ -43,8 +43,6 @@ def test_constructor_errors():
         tb.SparsityConfig(mode='bigbird')
     with pytest.raises(NotImplementedError):
         tb.SparsityConfig(attention='causal')
-    with pytest.raises(NotImplementedError):
-        tb.MultiheadAttention(32, 2, lay, 16, add_zero_attn=True)
     with pytest.raises(ValueError):
         tb.Softmax(lay, 16)(torch.zeros(1, 4, 16, 16, dtype=torch.float16), attn_mask=torch.zeros(32, 32))
     with pytest.raises(ValueError):

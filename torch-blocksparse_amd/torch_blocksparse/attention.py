@@ -21,8 +21,14 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
                                  key_padding_mask=None, need_weights=True, attn_mask=None,
                                  use_separate_proj_weight=False, q_proj_weight=None, k_proj_weight=None,
                                  v_proj_weight=None, static_k=None, static_v=None, key_padding_mask_mode='add',
-                                 attn_mask_mode='add'):
-    """Same signature and result as the reference (attention.py:9-202): returns (attn_output, None)."""
+                                 attn_mask_mode='add', key_block_pad=0):
+    """Same signature and result as the reference (attention.py:9-202): returns (attn_output, None).
+
+    bias_k / bias_v and add_zero_attn append one key position each, as in nn.functional.multi_head_attention_forward; the
+    masks grow by columns that leave those positions visible (0 in 'add' mode, 1 in 'mul' mode).  key_block_pad more
+    zero positions are then appended and hidden through the key-padding mask (one is made if the caller passed none), so
+    that the keys fill a whole number of blocks; the sparse operators passed in must be built on a layout with the
+    matching number of block-columns (MultiheadAttention does both)."""
     tgt_len, bsz, embed_dim = query.size()
     assert embed_dim == embed_dim_to_check
     assert key.size() == value.size()
@@ -53,16 +59,17 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
         v = linear(value, v_proj_weight, bias_slice(2 * E, None))
     q = q * scaling                                      # attention.py:127, so softmax runs with scale 1
 
-    def grow(mask, n):
+    def grow(mask, n, mode, visible=True):
         if mask is None:
             return None
-        return torch.cat([mask, mask.new_zeros((mask.size(0), n))], dim=1)
+        shown, hidden = (0., float('-inf')) if mode == 'add' else (1., 0.)
+        return torch.cat([mask, mask.new_full((mask.size(0), n), shown if visible else hidden)], dim=1)
 
     if bias_k is not None and bias_v is not None:
         assert static_k is None and static_v is None, 'bias cannot be added to static key/value.'
         k = torch.cat([k, bias_k.repeat(1, bsz, 1)])
         v = torch.cat([v, bias_v.repeat(1, bsz, 1)])
-        attn_mask, key_padding_mask = grow(attn_mask, 1), grow(key_padding_mask, 1)
+        attn_mask, key_padding_mask = grow(attn_mask, 1, attn_mask_mode), grow(key_padding_mask, 1, key_padding_mask_mode)
     else:
         assert bias_k is None and bias_v is None
 
@@ -79,12 +86,20 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
     if key_padding_mask is not None:
         assert key_padding_mask.size(0) == bsz and key_padding_mask.size(1) == src_len
     if attn_mask is not None:
-        assert attn_mask.size(0) == src_len and attn_mask.size(1) == src_len
+        assert attn_mask.size(0) == tgt_len and attn_mask.size(1) == src_len
     if add_zero_attn:
         src_len += 1
         k = torch.cat([k, k.new_zeros((k.size(0), 1) + k.size()[2:])], dim=1)
         v = torch.cat([v, v.new_zeros((v.size(0), 1) + v.size()[2:])], dim=1)
-        attn_mask, key_padding_mask = grow(attn_mask, 1), grow(key_padding_mask, 1)
+        attn_mask, key_padding_mask = grow(attn_mask, 1, attn_mask_mode), grow(key_padding_mask, 1, key_padding_mask_mode)
+    if key_block_pad:
+        k = torch.cat([k, k.new_zeros((k.size(0), key_block_pad) + k.size()[2:])], dim=1)
+        v = torch.cat([v, v.new_zeros((v.size(0), key_block_pad) + v.size()[2:])], dim=1)
+        if key_padding_mask is None:
+            key_padding_mask = q.new_full((bsz, src_len), 0. if key_padding_mask_mode == 'add' else 1.)
+        key_padding_mask = grow(key_padding_mask, key_block_pad, key_padding_mask_mode, visible=False)
+        attn_mask = grow(attn_mask, key_block_pad, attn_mask_mode)
+        src_len += key_block_pad
 
     q = q.reshape(bsz, num_heads, q.shape[1], q.shape[2]).contiguous()
     k = k.reshape(bsz, num_heads, k.shape[1], k.shape[2]).contiguous()
@@ -104,19 +119,26 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
 
 class MultiheadAttention(nn.modules.activation.MultiheadAttention):
 
+    def extra_keys(self):
+        """Key positions appended to the sequence: one for bias_k / bias_v, one for add_zero_attn."""
+        return int(self.bias_k is not None) + int(bool(self.add_zero_attn))
+
     def get_ops(self, L):
         if L not in self._ops:
-            self._ops[L] = (MatMul(self.layout, self.block, 'sdd', trans_a=False, trans_b=True),
-                            MatMul(self.layout, self.block, 'dsd', trans_a=False, trans_b=False),
-                            Softmax(self.layout, self.block))
+            layout = self.layout
+            if self.extra_keys():
+                # The appended positions get a block-column of their own, present in every block-row of every head
+                # (nn.MultiheadAttention shows them to every query); the rest of that block is padding, hidden through
+                # the key-padding mask.  The reference accepts the two flags and then runs its kernels on a key length
+                # that is not a whole number of blocks (attention.py:140-186).
+                layout = torch.cat([layout, torch.ones_like(layout[:, :, :1])], dim=2)
+            self._ops[L] = (MatMul(layout, self.block, 'sdd', trans_a=False, trans_b=True),
+                            MatMul(layout, self.block, 'dsd', trans_a=False, trans_b=False),
+                            Softmax(layout, self.block))
         return self._ops[L]
 
     def __init__(self, embed_dim, num_heads, layout, block, dropout=0., bias=True, add_bias_kv=False, add_zero_attn=False,
                  kdim=None, vdim=None, key_padding_mask_mode='add', attn_mask_mode='mul'):
-        if add_bias_kv or add_zero_attn:
-            # one more key position than the sequence has: L + 1 is not a whole number of blocks, so no [L/block, L/block]
-            # layout can describe the scores (the reference accepts the flags and then fails inside its kernels)
-            raise NotImplementedError('add_bias_kv / add_zero_attn append a key position, which a square block layout cannot hold')
         super(MultiheadAttention, self).__init__(embed_dim, num_heads, dropout, bias, add_bias_kv, add_zero_attn, kdim, vdim)
         self.layout = layout
         self.block = block
@@ -137,8 +159,10 @@ class MultiheadAttention(nn.modules.activation.MultiheadAttention):
             query, key, value = [t.transpose(0, 1) for t in (query, key, value)]
         sdd_nt, dsd_nn, softmax = self.get_ops(query.shape[0])
         extra = dict()
+        if self.extra_keys():
+            extra['key_block_pad'] = self.block - self.extra_keys()
         if not self._qkv_same_embed_dim:
-            extra = dict(use_separate_proj_weight=True, q_proj_weight=self.q_proj_weight,
+            extra.update(use_separate_proj_weight=True, q_proj_weight=self.q_proj_weight,
                          k_proj_weight=self.k_proj_weight, v_proj_weight=self.v_proj_weight)
         out, _ = multi_head_attention_forward(
             query, key, value, self.embed_dim, self.num_heads, self.in_proj_weight, self.in_proj_bias,
