@@ -96,6 +96,9 @@ def main():
     ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
                     help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
     ap.add_argument('--calibrate', action='store_true')
+    ap.add_argument('--kernel-flags', type=int, default=0,
+                    help='--config runs only: the flags argument of the matmul launchers (include/bsp.h: 1 general kernels only, '
+                         '2 no group plans, 4 no direct-to-LDS kernels), to time one kernel family against another')
     ap.add_argument('--record-traffic', nargs=2, metavar=('FETCH_DIR', 'WRITE_DIR'))
     args = ap.parse_args()
     if args.gpus != 1:
@@ -105,11 +108,16 @@ def main():
         return record_traffic(*args.record_traffic)
     if args.calibrate:
         return calibrate(args)
+    if args.kernel_flags and args.config == 3:
+        sys.exit('--kernel-flags is for --config 1|2|4|5 runs: the headline figure is always taken with the default kernels')
     if args.config != 3:
+        from torch_blocksparse import matmul as _mm
+        _mm.KERNEL_FLAGS = args.kernel_flags
         res = other_config(args.config, min(args.steps, 50), max(1, min(args.warmup, 5)))
         print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
                           'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic',
-                          'config': {'workload': res['workload'], 'config': args.config}, 'launches': res['launches']}))
+                          'config': {'workload': res['workload'], 'config': args.config, 'kernel_flags': args.kernel_flags},
+                          'launches': res['launches']}))
         return
 
     import torch
