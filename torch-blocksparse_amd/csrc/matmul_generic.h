@@ -88,7 +88,11 @@ template <typename T, int ROWS, int NT, bool KCONTIG> struct TileLoader {
   // its MFMA operand is a single element per lane, (row lane % MS, reduction index lane / MS), read where it lies.
   static constexpr bool ASIS = !KCONTIG;
   static constexpr bool TR = ASIS && sizeof(T) == 2;
-  static constexpr int LDR = ROWS + 8;
+  // Padding of a row of the as-is layout.  16-bit: the transposing read of a 16-lane group takes 32 contiguous bytes from
+  // each of four consecutive reduction rows, and two groups half a row block apart are served together; with rows of
+  // 64 bytes more than a multiple of 256 these eight pieces fall into different banks (the LDS serves 256 bytes per
+  // clock: measured, bank-conflict cycles 46-50 % -> 10-20 % of the LDS-active cycles against a padding of 16 bytes).
+  static constexpr int LDR = ROWS + (sizeof(T) == 2 ? 32 : 8);
   static constexpr int ELEMS = ASIS ? TK * LDR : ROWS * LDK;
   u32x4 reg[ITER];
   bool ok[ITER];
