@@ -189,18 +189,33 @@ def test_dropout_rate_and_repeatability():
     assert torch.equal(sm(x.clone(), dropout_p=0.0), sm(x.clone()))
 
 
-def test_backward_overwrites_the_incoming_gradient_like_the_reference():
-    # softmax.py:316-325 of the reference runs its backward kernel in place on the incoming gradient and returns it; so
-    # does this one: after backward the tensor handed in as dy holds dx (and x.grad is that very result)
+def test_backward_overwrites_only_a_private_gradient():
+    # The reference runs its backward kernel in place on whatever gradient comes in (softmax.py:316-325).  This one does so
+    # only when nobody else holds that tensor: (1) the tensor a user hands to backward() stays as it was; (2) a gradient
+    # that an addition passes on to a second branch reaches that branch unchanged; (3) inside the attention chain, where
+    # the gradient is a fresh result of the next operator's backward, the in-place path is the one taken.
+    from torch_blocksparse.softmax import _sparse_softmax
     lay = random_layout((2, 4, 4), 0.6, 3)
     nnz = int(lay.sum())
     torch.manual_seed(0)
     x = torch.rand(2, nnz, 32, 32, dtype=torch.float16)
     dy = torch.rand(2, nnz, 32, 32, dtype=torch.float16)
     _, rdx = D.softmax(x, lay, 32, scale=0.7, dy=dy)
+    op = tb.Softmax(lay, 32)
     xg = x.to(DEV).requires_grad_(True)
-    y = tb.Softmax(lay, 32)(xg * 1.0, scale=0.7)
     g = dy.to(DEV)
-    y.backward(g)
-    assert_close(g, rdx, torch.float16, 'softmax dy-buffer-after-backward')
+    op(xg * 1.0, scale=0.7).backward(g)
+    assert torch.equal(g.cpu(), dy), 'the gradient passed to backward() was modified'
     assert_close(xg.grad, rdx, torch.float16, 'softmax dx')
+    xg = x.to(DEV).requires_grad_(True)
+    w = torch.zeros_like(xg, requires_grad=True)
+    (op(xg * 1.0, scale=0.7) + w).backward(g)
+    assert torch.equal(w.grad.cpu(), dy), 'the other branch of an addition saw the softmax gradient instead of its own'
+    assert_close(xg.grad, rdx, torch.float16, 'softmax dx-with-a-shared-gradient')
+    before = _sparse_softmax.in_place_backwards
+    H, L, dh = 2, 128, 64
+    sdd, dsd = tb.MatMul(lay, 32, 'sdd', trans_b=True), tb.MatMul(lay, 32, 'dsd')
+    q, k, v = [torch.randn(2, H, L, dh, device=DEV, dtype=torch.float16, requires_grad=True) for _ in range(3)]
+    o = dsd(op(sdd(q, k), scale=0.125), v)
+    o.backward(torch.randn_like(o))
+    assert _sparse_softmax.in_place_backwards == before + 1, 'the chain did not take the in-place path'
