@@ -95,6 +95,7 @@ def main():
                     help='config 3 only: express the same attention mask in smaller blocks (64 = the headline workload)')
     ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
                     help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
+    ap.add_argument('--dtype', default='f16', choices=['f16', 'bf16'], help='config 3 only: the 16-bit type of the workload (the headline is quoted on f16)')
     ap.add_argument('--calibrate', action='store_true')
     ap.add_argument('--kernel-flags', type=int, default=0,
                     help='--config runs only: the flags argument of the matmul launchers (include/bsp.h: 1 general kernels only, '
@@ -122,7 +123,7 @@ def main():
 
     import torch
     import torch_blocksparse as tb
-    w = Attention(args.batch, args.block)
+    w = Attention(args.batch, args.block, args.dtype)
     step = w.step
     for _ in range(args.warmup):
         step()
@@ -148,7 +149,7 @@ def main():
                 if it >= 3:
                     events[name].append((e0, e1))
     torch.cuda.synchronize()
-    traffic = recorded_traffic() if (args.batch == 8 and args.block == 64) else {}
+    traffic = recorded_traffic() if (args.batch == 8 and args.block == 64 and args.dtype == 'f16') else {}
     kernels = {}
     for name, _, flops, nbytes in launches:
         ms = sum(a.elapsed_time(b) for a, b in events[name]) / len(events[name])
@@ -180,10 +181,10 @@ def main():
 
     block, B = args.block, args.batch
     out = {
-        'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, fp16 blk%d' % block,
+        'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, %s blk%d' % ({'f16': 'fp16', 'bf16': 'bf16'}[args.dtype], block),
         'value': round(6 * w.flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
-        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': 'f16', 'data': 'synthetic',
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': args.dtype, 'data': 'synthetic',
         'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block %d, fixed '
                                'layout (local 4 blocks + 1 global per 16 at block 64, causal), scale 1/8, additive key-padding mask' % (B, block),
                    'nnz_blocks': w.nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
@@ -205,7 +206,7 @@ def main():
 class Attention:
     """The headline workload: operands, operators, the autograd step and its eight launches one by one."""
 
-    def __init__(self, B=8, block=64):
+    def __init__(self, B=8, block=64, dtype='f16'):
         import torch
         import torch_blocksparse as tb
         from torch_blocksparse.matmul import _sparse_matmul
@@ -213,7 +214,7 @@ class Attention:
         dev = torch.device('cuda:0')
         torch.manual_seed(0)
         H, L, dh = 16, 4096, 64
-        dtype = torch.float16
+        dtype = {'f16': torch.float16, 'bf16': torch.bfloat16}[dtype]
         self.scale, self.dh, self.block = 0.125, dh, block
         lay = tb.sparse_transformer_layout(H, L // 64, 4, 16, True)
         if block != 64:   # the same mask, every 64-block split into (64 / block)^2 blocks: same flops, same bytes
