@@ -161,3 +161,31 @@ def test_workspace_size_of_split_chains():
     assert lib.bsp_xsd_workspace_bytes(0, 64, 8) == 0
     # 3 split chains x 2 tiles x 2 batches = 12 slots of 8 fp32 tiles of 64 x 64
     assert lib.bsp_xsd_workspace_bytes(3, 128, 2) == 12 * 8 * 64 * 64 * 4
+
+
+def test_private_gradient_detection():
+    # the softmax backward may overwrite its incoming gradient only if nobody else holds it: the detector (reference
+    # count of the tensor as the autograd engine hands it over, calibrated with a probe graph) on the CPU
+    from torch_blocksparse.softmax import _gradient_is_private, _private_use_count
+    assert _private_use_count() >= 1
+    seen = {}
+
+    class Spy(torch.autograd.Function):
+        @staticmethod
+        def forward(ctx, t, tag):
+            ctx.tag = tag
+            return t * 1.0
+
+        @staticmethod
+        def backward(ctx, g):
+            seen[ctx.tag] = _gradient_is_private(g)
+            return g * 1.0, None
+    x = torch.ones(4, requires_grad=True)
+    w = torch.ones(4, requires_grad=True)
+    (Spy.apply(x, 'fresh') * 2.0).sum().backward()                 # gradient made by the multiplication's backward
+    g = torch.ones(4)
+    Spy.apply(x, 'user').backward(g)                               # the user's own tensor
+    (Spy.apply(x, 'shared') + w).backward(torch.ones(4))           # one tensor handed to two branches by the addition
+    big = torch.ones(2, 4)
+    Spy.apply(x, 'view').backward(big[0])                          # a view of a larger tensor
+    assert seen == {'fresh': True, 'user': False, 'shared': False, 'view': False}
