@@ -192,11 +192,14 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     lookup(kStages - 1, pos, bid);                     // the table runs one step ahead of the loads that use it: its
     for (int s = 0; s < ksteps; s++) {                 // (scalar) latency is not between the barrier and the loads
-      BSP_WAIT_VM(L * (kStages - 2));                  // this wavefront's loads of step s have landed
+      // this wavefront's loads of step s have landed: all but those of the one step issued after them, or, at the
+      // last step, all (no load is issued for steps past the end)
+      if (s + 1 < ksteps) BSP_WAIT_VM(L * (kStages - 2));
+      else BSP_WAIT_VM(0);
       asm volatile("" ::: "memory");                   // (the compiler must not move LDS accesses across the barrier)
       __builtin_amdgcn_s_barrier();                    // everybody's have, and everybody is done reading step s - 1
       asm volatile("" ::: "memory");
-      issue(s + kStages - 1, pos, bid);                // into the stage that step s - 1 used
+      if (s + kStages - 1 < ksteps) issue(s + kStages - 1, pos, bid);   // into the stage that step s - 1 used
       lookup(s + kStages, pos, bid);
       const unsigned char *st = smem + (s % kStages) * STAGE;
       // operands of the second half of the step are fetched from LDS before the matrix instructions of the first
@@ -218,7 +221,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             else acc[i][j] = M::run(xf[kk][i], yf[kk][j], acc[i][j]);                    // ... along m
           }
     }
-    BSP_WAIT_VM(0);                                    // the padding loads past the end still target LDS
+    BSP_WAIT_VM(0);                                    // (nothing is in flight any more unless the segment had a single step)
   }
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
