@@ -326,14 +326,15 @@ def other_config(config, steps, warmup):
                         lay[h, r, int(torch.randint(0, shape[2], (1,), generator=g))] = 1
         return lay
 
-    def mm(name, mode, ta, tb_, block, dtype, Z, H, M, N, K, lay, scale=1.0):
+    def mm(name, mode, ta, tb_, block, dtype, Z, H, M, N, K, lay, scale=1.0, sp_scale=1.0):
+        # operands N(0, scale) (dense) and N(0, sp_scale) (sparse): the matrix pipes' clock under load depends on the data
         nnz = int(lay.sum())
         a = torch.randn((Z, H) + ((K, M) if ta else (M, K)), device=dev, dtype=dtype) * scale
         b = torch.randn((Z, H) + ((N, K) if tb_ else (K, N)), device=dev, dtype=dtype) * scale
         if mode == 'dsd':
-            a = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype)
+            a = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype) * sp_scale
         if mode == 'dds':
-            b = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype)
+            b = torch.randn(Z, nnz, block, block, device=dev, dtype=dtype) * sp_scale
         op = tb.MatMul(lay, block, mode, trans_a=ta, trans_b=tb_)
         with torch.no_grad():
             ms = timeit(lambda: op(a, b))
@@ -359,16 +360,16 @@ def other_config(config, steps, warmup):
         lay = bernoulli((16, 64, 64), 0.25, 2, one_per_row=True)
         for ta in (False, True):
             for tb_ in (False, True):
-                mm('dsd trans_a=%d trans_b=%d' % (ta, tb_), 'dsd', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
-                mm('dds trans_a=%d trans_b=%d' % (ta, tb_), 'dds', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.25)
-        mm('sdd (gradient of the sparse operand)', 'sdd', False, True, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay)
-        workload = 'fp16 block 32, Z 8, H 16, M=N=K=2048, Bernoulli(0.25) layout; bound: MFMA'
+                mm('dsd trans_a=%d trans_b=%d' % (ta, tb_), 'dsd', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.5)
+                mm('dds trans_a=%d trans_b=%d' % (ta, tb_), 'dds', ta, tb_, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.5)
+        mm('sdd (gradient of the sparse operand)', 'sdd', False, True, 32, torch.float16, 8, 16, 2048, 2048, 2048, lay, 2048 ** -0.5)
+        workload = 'fp16 block 32, Z 8, H 16, M=N=K=2048, Bernoulli(0.25) layout, dense operands N(0,1)/sqrt(K), sparse N(0,1); bound: MFMA'
     elif config == 5:
         lay = bernoulli((1, 32, 32), 0.1, 5)
-        mm('dds trans_b (y = x.W^T)', 'dds', False, True, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
-        mm('dds (dx = dy.W)', 'dds', False, False, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 0.1)
-        mm('sdd trans_a (dW = dy^T.x on the layout)', 'sdd', True, False, 128, torch.float16, 1, 1, 4096, 4096, 8192, lay, 0.1)
-        workload = 'block-sparse linear layer: 8192 tokens, 4096x4096 weight, block 128, 10 % density, fp16; bound: MFMA'
+        mm('dds trans_b (y = x.W^T)', 'dds', False, True, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 1.0, 0.02)
+        mm('dds (dx = dy.W)', 'dds', False, False, 128, torch.float16, 1, 1, 8192, 4096, 4096, lay, 1.0, 0.02)
+        mm('sdd trans_a (dW = dy^T.x on the layout)', 'sdd', True, False, 128, torch.float16, 1, 1, 4096, 4096, 8192, lay, 1.0)
+        workload = 'block-sparse linear layer: 8192 tokens, 4096x4096 weight N(0, 0.02), block 128, 10 % density, activations and gradients N(0,1), fp16; bound: MFMA'
     else:
         lay = tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True)
         B, H, L, dh, block = 2, 12, 16384, 64, 64

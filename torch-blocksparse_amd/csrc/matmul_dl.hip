@@ -114,32 +114,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const int wm = wave / WGN, wn = wave % WGN;
 
   const int n_tiles = (g.NF + kTN - 1) / kTN;
-  const int64_t per_z = (int64_t)g.width * n_tiles;
-  const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
-  int z = (int)(w / per_z);
-  int nt = (int)((w % per_z) / g.width);
-  int seg0 = (int)((w % per_z) % g.width);
-  // Longest segments first (g.order) means first on every XCD: an XCD works on a contiguous eighth of the launch, so
-  // inside its eighth the segment index is the slow one and the tile of the free dimension the fast one.  One batch
-  // with a number of tiles that divides by 8: every XCD gets all segments for its own tiles; batches that divide by 8:
-  // every XCD gets whole batches.
-  if (g.order) {
-    const int64_t total = per_z * g.Z;
-    if (total % 8 == 0) {
-      const int64_t chunk = total / 8, p = w % chunk;
-      const int x = (int)(w / chunk);
-      if (g.Z == 1 && n_tiles % 8 == 0) {
-        const int tpx = n_tiles / 8;
-        seg0 = (int)(p / tpx);
-        nt = x * tpx + (int)(p % tpx);
-      } else if (g.Z % 8 == 0) {
-        const int64_t q = p % per_z;
-        z = x * (g.Z / 8) + (int)(p / per_z);
-        seg0 = (int)(q / n_tiles);
-        nt = (int)(q % n_tiles);
-      }
-    }
-  }
+  int z, nt, seg0;
+  xsd_work_item(g, n_tiles, z, nt, seg0);
   const int seg = g.order ? as_table(g.order)[seg0] : seg0;
   const table_ptr hd = as_table(g.lut) + 6 * (int64_t)seg;
   const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];

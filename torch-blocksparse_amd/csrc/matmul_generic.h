@@ -534,6 +534,35 @@ template <int BLOCK, bool WIDE> struct XsdShape {
   static constexpr int WGN = 4 / WGM;
 };
 
+// Which (batch, tile of the free dimension, position in the dispatch order) a workgroup of the dsd / dds kernels takes.
+// Segment index fastest: consecutive workgroups (same XCD after the re-numbering) walk the segments of a head against one
+// slab of columns of the dense operand, which then stays in L2 between its uses.  With a dispatch order (g.order:
+// longest segments first, short launches only) "first" has to mean first on every XCD: an XCD works on a contiguous
+// eighth of the launch, so inside its eighth the position in the order is the slow index and the tile the fast one.
+// One batch with a number of tiles that divides by 8: every XCD gets all segments for its own tiles; a batch that
+// divides by 8: every XCD gets whole batches.
+__device__ __forceinline__ void xsd_work_item(const XsdArgs &g, int n_tiles, int &z, int &nt, int &seg0) {
+  const int64_t per_z = (int64_t)g.width * n_tiles, total = per_z * g.Z;
+  const int64_t w = xcd_remap(blockIdx.x, total);
+  z = (int)(w / per_z);
+  nt = (int)((w % per_z) / g.width);
+  seg0 = (int)((w % per_z) % g.width);
+  if (g.order && total % 8 == 0) {
+    const int64_t chunk = total / 8, p = w % chunk;
+    const int x = (int)(w / chunk);
+    if (g.Z == 1 && n_tiles % 8 == 0) {
+      const int tpx = n_tiles / 8;
+      seg0 = (int)(p / tpx);
+      nt = x * tpx + (int)(p % tpx);
+    } else if (g.Z % 8 == 0) {
+      const int64_t q = p % per_z;
+      z = x * (g.Z / 8) + (int)(p / per_z);
+      seg0 = (int)(q / n_tiles);
+      nt = (int)(q % n_tiles);
+    }
+  }
+}
+
 // (at least two wavefronts per SIMD: the 128 x 256 tile of block 128 would otherwise take 266 registers and run alone)
 template <typename T, int BLOCK, bool WIDE, bool SP_TRANS, bool DN_KCONTIG, bool OUT_NCONTIG>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k_xsd(XsdArgs g) {
@@ -541,13 +570,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) k
   typedef TileGemm<T, BLOCK, S::TN, S::WGM, S::WGN, !SP_TRANS, DN_KCONTIG, OUT_NCONTIG> G;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   const int n_tiles = (g.NF + S::TN - 1) / S::TN;
-  const int64_t per_z = (int64_t)g.width * n_tiles;
-  const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
-  const int z = (int)(w / per_z);
-  // segment index fastest: consecutive workgroups (same XCD after the re-numbering) walk the segments of a head
-  // against one slab of TN columns of the dense operand, which then stays in L2 between its uses
-  const int nt = (int)((w % per_z) / g.width);
-  const int seg0 = (int)((w % per_z) % g.width);
+  int z, nt, seg0;
+  xsd_work_item(g, n_tiles, z, nt, seg0);
   const int seg = g.order ? as_table(g.order)[seg0] : seg0;   // longest first only where the launch is short (see the dispatcher)
   const table_ptr hd = as_table(g.lut) + 6 * (int64_t)seg;
   const int offset = hd[0], seglen = hd[1], column = hd[2], depth = hd[3];
