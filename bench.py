@@ -128,7 +128,7 @@ def main():
     # Per-launch timing with HIP events on the launch stream, the eight launches of a step issued back to back in
     # step order (so each kernel sees the cache state its predecessor leaves), K steps, one synchronisation at the end.
     launches = w.launches() + [('calibration_copy', w.k_copy, 0.0, 2 * w.x_bytes)]
-    reps = max(args.steps, 10)
+    reps = max(args.steps, 50)                    # at least ~40 ms of work: past the power-management transient that follows an idle GPU
     events = {name: [] for name, _, _, _ in launches}
     with torch.no_grad():
         for it in range(10 + reps):                  # the first ten passes are not recorded
