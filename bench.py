@@ -41,6 +41,8 @@ FP32_PEAK_TFLOPS = 157.3    # fp32 matrix
 
 TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'traffic_attention_seq4096_fp16_blk64.json')
 
+SETTLE_STEPS = 30         # untimed steps in front of the warm-up steps (see main)
+
 # kernel behind each launch of the step, for the per-kernel totals (the headline block size; kernel_of() for the others)
 KERNEL_OF = {
     'sdd_fwd  q.k^T': 'k_sdd64_rg', 'sdd_bwd  do.v^T': 'k_sdd64_rg',
@@ -128,6 +130,11 @@ def main():
     # Per-launch timing with HIP events on the launch stream, the eight launches of a step issued back to back in
     # step order (so each kernel sees the cache state its predecessor leaves), K steps, one synchronisation at the end.
     launches = w.launches() + [('calibration_copy', w.k_copy, 0.0, 2 * w.x_bytes)]
+    # No garbage collection inside the measured regions: a full collection stops the host for tens of milliseconds, the
+    # launch queue runs dry, and the idle time lands between the two events of whichever launch comes next.
+    import gc
+    gc.collect()
+    gc.disable()
     reps = max(args.steps, 50)                    # at least ~40 ms of work: past the power-management transient that follows an idle GPU
     events = {name: [] for name, _, _, _ in launches}
     with torch.no_grad():
@@ -142,6 +149,11 @@ def main():
     torch.cuda.synchronize()
     # The step itself: W untimed steps, then exactly K steps between two synchronisations.  (The per-launch pass above
     # runs first so that clocks, caches and the allocator are in their steady state whatever W is.)
+    # After any change of the launch pattern (an idle GPU, or the per-launch pass above) the step time needs about 25
+    # steps to settle (0.63 -> 0.59 ms here, the GPU's power management): SETTLE_STEPS more untimed steps in front of the
+    # W warm-up steps, so that the K timed steps measure the steady state whatever W is.  Reported as config.settle_steps.
+    for _ in range(SETTLE_STEPS):
+        step()
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -150,11 +162,18 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    gc.enable()
 
     traffic = recorded_traffic() if (args.batch == 8 and args.block == 64 and args.dtype == 'f16') else {}
     kernels = {}
+    stalls = 0
     for name, _, flops, nbytes in launches:
-        ms = sum(a.elapsed_time(b) for a, b in events[name]) / len(events[name])
+        # mean over the passes; a sample more than three times the median is not a launch duration but a launch that the
+        # GPU had to wait for (the host was held up: the events bracket the wait too) and is left out, and counted
+        samples = sorted(a.elapsed_time(b) for a, b in events[name])
+        kept = [t for t in samples if t <= 3.0 * samples[len(samples) // 2]]
+        stalls += len(samples) - len(kept)
+        ms = sum(kept) / len(kept)
         ent = {'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
                'bytes': nbytes, 'traffic': traffic.get(name)}
         if flops:
@@ -189,7 +208,8 @@ def main():
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': args.dtype, 'data': 'synthetic',
         'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block %d, fixed '
                                'layout (local 4 blocks + 1 global per 16 at block 64, causal), scale 1/8, additive key-padding mask' % (B, block),
-                   'nnz_blocks': w.nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4)},
+                   'nnz_blocks': w.nnz, 'sum_of_kernel_ms': round(sum(e['ms'] for e in kernels.values()), 4),
+                   'per_launch_samples_left_out_as_host_stalls': stalls, 'settle_steps': SETTLE_STEPS},
         'matmul_TFLOP/s_kernel_time_only': round(6 * w.flops_mm / sum(e['ms'] for n, e in kernels.items() if 'softmax' not in n) * 1e-9, 2),
         'softmax_GB/s': {'fwd': kernels['softmax_fwd']['GB/s'], 'bwd': kernels['softmax_bwd']['GB/s']},
         'roofline': roofline, 'kernels': kernels, 'calibration_copy': calib,
