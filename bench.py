@@ -328,14 +328,29 @@ def other_config(config, steps, warmup):
     out = []
 
     def timeit(f):
+        import gc
+        # warm-up by time, not by count: after a change of the launch pattern the GPU needs about 20 ms of the new work
+        # before its launch times settle (see SETTLE_STEPS), whether that is 15 launches or 400
         for _ in range(max(warmup, 1)):
             f()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        f()
+        torch.cuda.synchronize()
+        one = max(time.perf_counter() - t0, 2e-5)
+        for _ in range(min(2000, int(0.025 / one) + 1)):
             f()
-        e1.record()
-        e1.synchronize()
+        gc.collect()
+        gc.disable()                                   # (a collection pause would leave the GPU waiting inside the timed loop)
+        try:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                f()
+            e1.record()
+            e1.synchronize()
+        finally:
+            gc.enable()
         return e0.elapsed_time(e1) / steps
 
     def bernoulli(shape, density, seed, one_per_row=False):
