@@ -27,6 +27,9 @@ def pytest_terminal_summary(terminalreporter):
     for (dtype, what, form), val in sorted(ACHIEVED.items()):
         if form == 'pure':
             terminalreporter.write_line('%-9s %-12s max relative error %.3g (bound %g, no absolute term)' % (dtype, what, val, bound[dtype]))
+        elif form == 'terms':
+            terminalreporter.write_line('%-9s %-12s %.0f %% of the tolerance used at most (bound %g of the summed |terms|, no absolute term)'
+                                        % (dtype, what, 100 * val, bound[dtype]))
         else:
             terminalreporter.write_line('%-9s %-12s %.0f %% of the tolerance used at most' % (dtype, what, 100 * val))
 

@@ -9,7 +9,7 @@ import torch
 
 import torch_blocksparse as tb
 from oracle import dense_oracle as D
-from helpers import assert_close, random_layout, run_matmul_case as run_case
+from helpers import assert_close, guard_allocations, random_layout, run_matmul_case as run_case
 
 pytestmark = pytest.mark.gpu
 DEV = 'cuda'
@@ -20,6 +20,84 @@ def head_blocks(lay, h):
     per_head = lay.reshape(lay.shape[0], -1).sum(1)
     lo = int(per_head[:h].sum())
     return lo, lo + int(per_head[h])
+
+
+def test_config1_readme_sdd_then_softmax_fp32():
+    # README shape: sdd with trans_a, fp32, Z=4, H=2, M=256, N=512, K=384, block 16, operands uniform in [0, 1), layout
+    # Bernoulli(0.5) of shape [H, M/16, N/16]; then Softmax(layout, 16) on the sparse result.  1e-5 relative at every
+    # stage: (1) the product against the oracle (sums of positive terms: pure relative bound); (2) the softmax kernel
+    # against the oracle's softmax of the very logits the GPU produced (pure relative bound); (3) the chain against the
+    # oracle's chain.  For (3) the bound has to follow the arithmetic: a softmax turns an ABSOLUTE perturbation d of its
+    # logits into a RELATIVE one of its result, |dy/y| <= 2 max|d|, and stage (1) leaves d <= 1e-5 |c| with c ~ K/4 = 96
+    # here, so the chain is held to 1e-5 (1 + 2 scale max|c|) relative, with max|c| taken per row of the oracle's logits.
+    torch.manual_seed(0)
+    Z, H, M, N, K, block = 4, 2, 256, 512, 384, 16
+    lay = torch.randint(0, 2, (H, M // block, N // block))
+    for h in range(H):
+        for r in range(M // block):
+            if lay[h, r].sum() == 0:
+                lay[h, r, 0] = 1
+    a = torch.rand(Z, H, K, M)
+    b = torch.rand(Z, H, K, N)
+    scale = 1.0                                              # Softmax's default, as in the README
+    rc = D.matmul(a, b, 'sdd', True, False, lay, block)
+    ry = D.softmax(rc, lay, block, scale=scale)
+    sdd = tb.MatMul(lay, block, 'sdd', trans_a=True, trans_b=False)
+    sm = tb.Softmax(lay, block)
+    with guard_allocations('config 1'):
+        c = sdd(a.to(DEV), b.to(DEV))
+        c_gpu = c.clone()
+        y = sm(c, scale=scale)
+    assert y.data_ptr() == c.data_ptr()                      # in place, as the reference
+    assert_close(c_gpu, rc, torch.float32, 'config 1 sdd', no_cancellation=True)
+    assert_close(y, D.softmax(c_gpu, lay, block, scale=scale), torch.float32, 'config 1 softmax of the GPU logits', no_cancellation=True)
+    row_max = D.sparse_to_dense(rc, lay, block).abs().amax(-1, keepdim=True)                  # [Z, H, M, 1]
+    row_max = D.dense_to_sparse(row_max.expand(-1, -1, -1, N), lay, block)
+    bound = 1e-5 * (1 + 2 * scale * row_max) * ry
+    err = (y.cpu() - ry).abs()
+    assert bool((err <= bound).all()), 'config 1 chain: max err / bound = %g' % float((err / bound.clamp(min=1e-45)).max())
+    # rows of the result sum to one
+    sums = D.sparse_to_dense(y.cpu(), lay, block).sum(-1)
+    assert float((sums - 1).abs().max()) < 1e-5
+
+
+def test_config3_sparse_transformer_attention_full_size_with_mask_and_backward():
+    # The benchmark configuration itself: batch 8, 16 heads, seq 4096, head_dim 64, block 64, fp16, fixed Sparse-Transformer
+    # layout (local window of 4 blocks + one global block per 16, causal), scale 1/8, additive key-padding mask with the
+    # last 0-25 % of the keys of every sequence padded (random per sequence), forward and backward.  With batch 8 the
+    # launches put one batch on each XCD (z = workgroup index mod 8), the scheduling the benchmark figure relies on.
+    # Dense oracle on three (batch, head) slices including the first and the last.
+    B, H, L, dh, block = 8, 16, 4096, 64, 64
+    lay = tb.sparse_transformer_layout(H, L // block, 4, 16, True)
+    g = torch.Generator().manual_seed(33)
+    q, k, v, do = [torch.randn(B, H, L, dh, generator=g).half() for _ in range(4)]
+    kpm = torch.zeros(B, L)
+    padded = torch.randint(0, L // 4 + 1, (B,), generator=g)
+    for z in range(B):
+        if padded[z] > 0:
+            kpm[z, L - int(padded[z]):] = float('-inf')
+    sdd = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=True)
+    dsd = tb.MatMul(lay, block, 'dsd')
+    sm = tb.Softmax(lay, block)
+    kpm_dev, do_dev = kpm.half().to(DEV), do.to(DEV)
+
+    def chain():
+        qg, kg, vg = [t.to(DEV).requires_grad_(True) for t in (q, k, v)]
+        o = dsd(sm(sdd(qg, kg), scale=0.125, key_padding_mask=kpm_dev), vg)
+        o.backward(do_dev)
+        torch.cuda.synchronize()
+        return [t.detach().cpu() for t in (o, qg.grad, kg.grad, vg.grad)]
+    got = chain()                                 # as the benchmark runs it (the softmax gradient computed in place)
+    with guard_allocations('config 3'):           # and with every output, gradient and workspace inside guard bands
+        guarded = chain()
+    for x, y in zip(got, guarded):
+        assert torch.equal(x, y)
+    for z, h in ((0, 0), (B - 1, H - 1), (int(padded.argmax()), 6)):
+        sl = (slice(z, z + 1), slice(h, h + 1))
+        ref = D.attention(q[sl], k[sl], v[sl], lay[h:h + 1], block, 0.125, key_padding_mask=kpm[z:z + 1], do=do[sl])
+        for name, x, r in zip(('out', 'dq', 'dk', 'dv'), got, ref):
+            assert not torch.isnan(r).any()
+            assert_close(x[sl], r, torch.float16, 'config 3 z=%d h=%d %s' % (z, h, name))
 
 
 def test_config2_dsd_dds_all_transpositions_full_size():

@@ -54,3 +54,51 @@ def test_attention_chain_captured_and_replayed(block, dtype):
         torch.cuda.synchronize()
         for name, a, b in zip(('out', 'dq', 'dk', 'dv'), static_out, eager):
             assert torch.equal(a, b), 'replay %d differs from the eager run: %s (block %d)' % (rep, name, block)
+
+
+def test_split_chains_captured_then_a_larger_eager_call_between_replays():
+    # A layout with a line of more than 128 blocks: the chain is cut into parts whose fp32 partial tiles live in the
+    # plan's workspace, and a captured launch carries that buffer's address.  An eager call with a larger batch between
+    # the replays makes the plan take a larger workspace; the one the graph uses must stay alive and untouched by
+    # other tensors, so every replay still equals the eager result.
+    torch.manual_seed(11)
+    n, block, dtype = 300, 64, torch.float16
+    lay = torch.zeros(2, n, 4, dtype=torch.int64)
+    lay[:, :, 1] = 1
+    lay[0, ::7, 0] = 1
+    lay[1, ::5, 3] = 1
+    op = tb.MatMul(lay, block, 'dsd', trans_a=True)
+    nnz = int(lay.sum())
+    a = (0.1 * torch.randn(2, nnz, block, block, device=DEV)).to(dtype)
+    b = torch.randn(2, 2, n * block, 64, device=DEV, dtype=dtype)
+    a_big = (0.1 * torch.randn(5, nnz, block, block, device=DEV)).to(dtype)
+    b_big = torch.randn(5, 2, n * block, 128, device=DEV, dtype=dtype)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            op(a, b)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    plan = op.make_lut(dtype, a.device)[0].gplan
+    assert plan.n_split == 2
+    small_ws = plan._ws
+    sa, sb = a.clone(), b.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = op(sa, sb)
+    assert plan._ws is small_ws                         # the capture allocated nothing new for the chains
+    for rep in range(3):
+        big = op(a_big, b_big)                          # larger batch and free dimension: the workspace grows
+        assert plan._ws is not small_ws and any(w is small_ws for w in plan._ws_retired)
+        filler = [torch.full((small_ws.numel() // 4,), float(rep), device=DEV) for _ in range(4)]   # would land in a freed buffer
+        fa, fb = torch.randn_like(sa) * 0.1, torch.randn_like(sb)
+        eager = op(fa, fb)
+        torch.cuda.synchronize()
+        sa.copy_(fa)
+        sb.copy_(fb)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), 'replay %d differs from the eager run' % rep
+        assert all(bool((f == float(rep)).all()) for f in filler)
+        del big, filler

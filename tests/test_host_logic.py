@@ -188,4 +188,61 @@ def test_private_gradient_detection():
     (Spy.apply(x, 'shared') + w).backward(torch.ones(4))           # one tensor handed to two branches by the addition
     big = torch.ones(2, 4)
     Spy.apply(x, 'view').backward(big[0])                          # a view of a larger tensor
-    assert seen == {'fresh': True, 'user': False, 'shared': False, 'view': False}
+    g2 = torch.ones(4)
+    Spy.apply(x, 'detached').backward(g2.detach())                 # another tensor object over the user's storage: no base,
+    Spy.apply(x, 'data').backward(g2.data)                         # few owners of the object, but the memory is shared
+    assert seen == {'fresh': True, 'user': False, 'shared': False, 'view': False, 'detached': False, 'data': False}
+
+
+def test_sdd_long_reduction_branch_raises_on_a_failed_launch(monkeypatch):
+    # the block-32 long-reduction sdd goes to the library with the plan alone; a negative status must raise instead of
+    # returning the uninitialised output (library mocked: no GPU needed)
+    from torch_blocksparse import matmul as M
+
+    class FakeLib:
+        def bsp_sdd_matmul(self, *args):
+            return -5
+
+        def bsp_strerror(self, code):
+            return b'HIP runtime error'
+    monkeypatch.setattr(_lib, 'load', lambda: FakeLib())
+    monkeypatch.setattr(_lib, 'ptr', lambda t: 0)
+    monkeypatch.setattr(_lib, 'stream_ptr', lambda d: 0)
+    monkeypatch.setattr(M, '_Timer', lambda bench, device: type('T', (), {'done': lambda self: None})())
+    luts = M.SddTables()
+    luts.nnz, luts.spdims = 4, (1, 2, 2)
+    plan = M.GroupPlan(torch.zeros(8, dtype=torch.int32), 1, 2)
+    luts.gplan, luts.gplan_long = plan, plan
+    luts.build = lambda: ([], [], [])
+    luts.build_long = lambda: plan
+    a = torch.zeros(1, 1, 64, 256, dtype=torch.float16)
+    b = torch.zeros(1, 1, 256, 64, dtype=torch.float16)
+    with pytest.raises(_lib.BlocksparseLibraryError, match='bsp_sdd_matmul'):
+        M._sparse_matmul._sdd_matmul(a, b, False, False, False, (1, 2, 2), 32, luts, 1, None, None, False, [None])
+    # the sibling branch (plan alone, short reduction) raises the same way
+    luts.build_long = None
+    a = torch.zeros(1, 1, 64, 64, dtype=torch.float16)
+    b = torch.zeros(1, 1, 64, 64, dtype=torch.float16)
+    with pytest.raises(_lib.BlocksparseLibraryError, match='bsp_sdd_matmul'):
+        M._sparse_matmul._sdd_matmul(a, b, False, False, False, (1, 2, 2), 32, luts, 1, None, None, False, [None])
+
+
+def test_replace_mha_takes_the_reference_form_with_one_info_argument():
+    # replace_mha(model, info) of the reference (attention.py:267-281): info carries layout and block
+    import types
+    import torch_blocksparse as tb
+    block, heads, E, L = 16, 2, 32, 64
+    layout = torch.ones(heads, L // block, L // block, dtype=torch.int64)
+    for info in (types.SimpleNamespace(layout=layout, block=block), dict(layout=layout, block=block), (layout, block)):
+        model = torch.nn.TransformerEncoderLayer(E, heads, dim_feedforward=64, dropout=0.0)
+        before = {k: v.clone() for k, v in model.self_attn.state_dict().items()}
+        tb.replace_mha(model, info)
+        assert isinstance(model.self_attn, tb.MultiheadAttention) and model.self_attn.block == block
+        assert torch.equal(model.self_attn.layout, layout)
+        for k, v in model.self_attn.state_dict().items():
+            assert torch.equal(v, before[k])
+    model = torch.nn.TransformerEncoderLayer(E, heads, dim_feedforward=64, dropout=0.0)
+    tb.replace_mha(model, layout, block)
+    assert isinstance(model.self_attn, tb.MultiheadAttention)
+    with pytest.raises(TypeError):
+        tb.replace_mha(model, layout)

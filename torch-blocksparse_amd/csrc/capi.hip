@@ -142,6 +142,18 @@ extern "C" int bsp_dsd_matmul(int dtype, const void *a, const void *b, void *c, 
   return xsd_dispatch(dtype, g, block, trans_a != 0, trans_b != 0, !trans_c, flags, stream);
 }
 
+// Whether a dsd launch with these properties is taken by a kernel that runs split chains and so uses the workspace:
+// the row-group kernels on 64 x 64 tiles (block 64, or block 16 with a plan over tiles: negative line count), 16-bit
+// types, dense operand not reduction-contiguous, output rows contiguous, whole 64-wide tiles of the free dimension,
+// and at block 64 a free dimension the wide kernel (xsd_dl, which comes first in xsd_dispatch) leaves alone.
+static bool split_chains_run(int dtype, int block, int N, bool dn_kc, bool out_nc, int plan_lines, int flags) {
+  if (dtype == BSP_F32 || dn_kc || !out_nc || N % 64) return false;
+  if (no_groups(flags) || general_only(flags)) return false;
+  if (block == 16) return plan_lines < 0;
+  if (block == 64) return plan_lines > 0 && (N < 256 || no_wide(flags));
+  return false;
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // The allocation-free variant of bsp_dsd_matmul: the workspace of the split chains is a static device array.
 // In host code the array's name only stands for the symbol; its device address differs from GPU to GPU and is looked
@@ -178,6 +190,11 @@ extern "C" int bsp_dsd_matmul_noalloc(int dtype, const void *a, const void *b, v
   if (n_split < 0 || Z <= 0 || N <= 0) return BSP_ERR_ARG;
   void *ws = nullptr;
   int64_t ws_bytes = 0;
+  if (d_gplan && n_split > 0 && !split_chains_run(dtype, block, N, trans_b != 0, !trans_c, plan_lines, flags)) {
+    // A kernel that does not know split chains takes this launch (the wide kernel, the general one, fp32, ...): it
+    // needs no scratch memory whatever the sizes, and must not see a plan whose chains are cut into parts.
+    d_gplan = nullptr; n_plan_groups = 0; plan_lines = 0; n_split = 0;
+  }
   if (d_gplan && n_split > 0) {
     if (xsd_ws_slots(n_split, N, Z) > BSP_NOALLOC_MAX_SLOTS) return BSP_ERR_SCRATCH_LIMIT;
     ws = scratch_address();

@@ -173,12 +173,30 @@ class MultiheadAttention(nn.modules.activation.MultiheadAttention):
         return (out.transpose(0, 1) if self.batch_first else out), None
 
 
-def replace_mha(model, layout, block):
+def _layout_and_block(info, block):
+    """(layout, block) from either calling form of replace_mha: (layout, block), or one `info` carrying both: an
+    object with attributes `layout` and `block`, a mapping with those keys, or a (layout, block) pair."""
+    if block is not None:
+        return info, block
+    if isinstance(info, dict):
+        return info['layout'], info['block']
+    if hasattr(info, 'layout') and hasattr(info, 'block'):
+        return info.layout, info.block
+    if isinstance(info, (tuple, list)) and len(info) == 2:
+        return info[0], info[1]
+    raise TypeError('replace_mha(model, info): info must carry `layout` and `block` (attributes, keys or a pair); '
+                    'or call replace_mha(model, layout, block)')
+
+
+def replace_mha(model, layout, block=None):
     """Swap every nn.MultiheadAttention inside `model` for the block-sparse one, keeping its parameters, dtype, device
-    and batch_first setting.  The reference's replace_mha(model, info) hands `info` to a constructor that needs layout
-    AND block (attention.py:267-281) and cannot run; this one takes both.  Like the reference it builds the replacement
-    with key_padding_mask_mode='mul' and attn_mask_mode='add', the conventions of nn.MultiheadAttention's masks
-    (boolean / 0-1 padding mask, additive float attention mask); masks must have the dtype of the activations."""
+    and batch_first setting.  Two calling forms: replace_mha(model, layout, block), and the reference's
+    replace_mha(model, info) (attention.py:267-281), where `info` carries the layout and the block size (the reference
+    hands `info` to a constructor that needs both and cannot run as written).  Like the reference it builds the
+    replacement with key_padding_mask_mode='mul' and attn_mask_mode='add', the conventions of
+    nn.MultiheadAttention's masks (boolean / 0-1 padding mask, additive float attention mask); masks must have the
+    dtype of the activations."""
+    layout, block = _layout_and_block(layout, block)
     for child_name, child in model.named_children():
         if isinstance(child, nn.modules.activation.MultiheadAttention) and not isinstance(child, MultiheadAttention):
             ref = child.in_proj_weight if child.in_proj_weight is not None else child.q_proj_weight

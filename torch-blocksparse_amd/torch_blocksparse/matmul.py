@@ -91,6 +91,7 @@ class GroupPlan:
         self.table, self.n_groups, self.lines, self.n_split = table, n_groups, lines, n_split
         self.coarse = False
         self._ws = None
+        self._ws_retired = []
 
     @staticmethod
     def thin_min(layout, by_rows, block=64, nnz=None):
@@ -165,11 +166,15 @@ class GroupPlan:
     def workspace(self, free_dim, Z):
         """(pointer, bytes) of the scratch buffer the split chains of this plan need for a launch with this free dimension
         and batch (fp32 partial tiles; kept for the next call, contents never matter); (NULL, 0) for a plan without
-        split chains.  One buffer per plan: launches of one operator are assumed to be ordered on one stream."""
+        split chains.  One buffer per plan: launches of one operator are assumed to be ordered on one stream.
+        A launch that needs more than the buffer holds gets a larger one, and the smaller one stays allocated for the
+        life of the plan: a captured HIP graph replays launches that carry its address."""
         if self.n_split == 0:
             return ctypes.c_void_p(0), 0
         need = _lib.load().bsp_xsd_workspace_bytes(self.n_split, int(free_dim), int(Z))
         if self._ws is None or self._ws.numel() < need:
+            if self._ws is not None:
+                self._ws_retired.append(self._ws)
             self._ws = torch.empty(need, dtype=torch.uint8, device=self.table.device)
         return _lib.ptr(self._ws), self._ws.numel()
 
@@ -341,6 +346,8 @@ class _sparse_matmul(torch.autograd.Function):
             lp = GroupPlan.args(luts.gplan_long)
             rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), spdims[2], lp[0], lp[1], lp[2],
                                     KERNEL_FLAGS, _lib.stream_ptr(a.device))
+            if rc not in (_lib.OK_WHOLE_LAYOUT, _lib.NEEDS_TABLE):
+                _lib.check(rc, 'bsp_sdd_matmul')
         elif lazy and luts.gplan is not None and luts.build is not None:
             rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), spdims[2], gplan[0], gplan[1], gplan[2],
                                     KERNEL_FLAGS, _lib.stream_ptr(a.device))

@@ -38,10 +38,28 @@ def _private_use_count():
     return _PRIVATE_USE_COUNT
 
 
+def _storage_owners(g):
+    """How many tensors share g's storage (g itself counts), or a large number when that cannot be told."""
+    try:
+        return int(torch._C._storage_Use_Count(g.untyped_storage()._cdata))
+    except Exception:
+        return 1 << 30
+
+
+_PRIVATE_STORAGE_COUNT = None
+
+
 def _gradient_is_private(g):
-    """True when no one but the autograd engine holds g (then overwriting it cannot be observed)."""
+    """True when no one but the autograd engine holds g (then overwriting it cannot be observed): neither the tensor
+    object (its own reference count), nor a view of it, nor its storage through another tensor object such as
+    `g.detach()` or `g.data`, which share the memory but have no base."""
+    global _PRIVATE_STORAGE_COUNT
     base = _private_use_count()
-    return base > 0 and hasattr(g, '_use_count') and g._use_count() <= base and g._base is None
+    if not (base > 0 and hasattr(g, '_use_count') and g._use_count() <= base and g._base is None):
+        return False
+    if _PRIVATE_STORAGE_COUNT is None:
+        _PRIVATE_STORAGE_COUNT = _storage_owners(torch.ones(2))      # what a tensor nobody shares reads
+    return _storage_owners(g) <= _PRIVATE_STORAGE_COUNT
 
 
 class _sparse_softmax(torch.autograd.Function):
@@ -145,24 +163,29 @@ class _sparse_softmax(torch.autograd.Function):
             rc = _lib.load().bsp_softmax_dropout_fwd(_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(out), float(scale), _lib.ptr(lut), maxlut,
                                                      *common, out.stride(0), float(p), int(seed), int(offset), _lib.stream_ptr(x.device))
             _lib.check(rc, 'bsp_softmax_dropout_fwd')
+            ctx.mark_dirty(x)      # x now holds the softmax: autograd must know, as on the path without dropout
         time[0] = timer.done()
         ctx.save_for_backward(x, lut)
         ctx.spdims, ctx.block, ctx.maxlut, ctx.scale = spdims, block, maxlut, scale
-        return out
+        return out if dropout is None else (out, x)
 
     @staticmethod
-    def backward(ctx, dx):
-        """The kernel computes the gradient in place, as the reference does on every incoming gradient (softmax.py:316-325).
+    def backward(ctx, dx, dy_plain=None):
+        """dx: gradient of the (dropped) result; dy_plain: with dropout, the gradient of the second output, the softmax
+        itself that x was overwritten with (None unless the caller went on using x).
+        The kernel computes the gradient in place, as the reference does on every incoming gradient (softmax.py:316-325).
         Here that happens only when the incoming tensor is private to this call: a gradient that something else still
         holds (the tensor the user handed to backward(), a gradient that an addition passes to two branches) is copied
         first, so nobody else sees it change."""
         x, lut = ctx.saved_tensors
+        if dx is None:             # with dropout: only the softmax left in x was used
+            dx = torch.zeros_like(x)
         if dx.shape != x.shape:
             raise ValueError('softmax gradient has shape %s, the output has %s' % (tuple(dx.shape), tuple(x.shape)))
         private = _gradient_is_private(dx)
         dx = dx.contiguous()
         if dx.data_ptr() % 16 != 0 or not private:
-            dx = dx.clone()
+            dx = torch.empty_like(dx).copy_(dx)
         _sparse_softmax.in_place_backwards += int(private)
         args = (_lib.DTYPES[x.dtype], _lib.ptr(x), _lib.ptr(dx), float(ctx.scale), _lib.ptr(lut), ctx.maxlut, x.size(0),
                 ctx.spdims[0], ctx.spdims[1], ctx.block, x.stride(0), dx.stride(0))
@@ -172,6 +195,11 @@ class _sparse_softmax(torch.autograd.Function):
             p, seed, offset = ctx.dropout
             rc = _lib.load().bsp_softmax_dropout_bwd(*args, float(p), int(seed), int(offset), _lib.stream_ptr(x.device))
         _lib.check(rc, 'bsp_softmax_bwd')
+        if dy_plain is not None:
+            extra = torch.empty_like(x).copy_(dy_plain)
+            rc = _lib.load().bsp_softmax_bwd(*(args[:2] + (_lib.ptr(extra),) + args[3:-1] + (extra.stride(0),)), _lib.stream_ptr(x.device))
+            _lib.check(rc, 'bsp_softmax_bwd')
+            dx = dx + extra
         return (dx,) + (None,) * 13
 
 
@@ -220,4 +248,4 @@ class Softmax:
         x = Softmax.sparse_softmax(x, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode,
                                    self.spdims, self.block, lut, maxlut, self.bench, time_y, dropout)
         self.time_y = time_y[0]
-        return x
+        return x if dropout is None else x[0]
