@@ -95,8 +95,9 @@ def main():
     ap.add_argument('--batch', type=int, default=8)
     ap.add_argument('--block', type=int, default=64, choices=[16, 32, 64],
                     help='config 3 only: express the same attention mask in smaller blocks (64 = the headline workload)')
-    ap.add_argument('--config', type=int, default=3, choices=[1, 2, 3, 4, 5],
-                    help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one')
+    ap.add_argument('--config', default='3', choices=['1', '2', '3', '4', '5', 'ref'],
+                    help='3 = the headline workload (default); 1, 2, 4, 5 = the other configurations, matmul/softmax launches timed one by one; '
+                         'ref = the shapes of the reference\'s own benchmark functions (tests/test_matmul.py:105-122, tests/test_softmax.py:92-128)')
     ap.add_argument('--dtype', default='f16', choices=['f16', 'bf16'], help='config 3 only: the 16-bit type of the workload (the headline is quoted on f16)')
     ap.add_argument('--calibrate', action='store_true')
     ap.add_argument('--kernel-flags', type=int, default=0,
@@ -111,12 +112,17 @@ def main():
         return record_traffic(*args.record_traffic)
     if args.calibrate:
         return calibrate(args)
+    if args.config != 'ref':
+        args.config = int(args.config)
     if args.kernel_flags and args.config == 3:
         sys.exit('--kernel-flags is for --config 1|2|4|5 runs: the headline figure is always taken with the default kernels')
     if args.config != 3:
         from torch_blocksparse import matmul as _mm
         _mm.KERNEL_FLAGS = args.kernel_flags
-        res = other_config(args.config, min(args.steps, 50), max(1, min(args.warmup, 5)))
+        if args.config == 'ref':
+            res = reference_bench_shapes(min(args.steps, 50), max(1, min(args.warmup, 5)))
+        else:
+            res = other_config(args.config, min(args.steps, 50), max(1, min(args.warmup, 5)))
         print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
                           'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic',
                           'config': {'workload': res['workload'], 'config': args.config, 'kernel_flags': args.kernel_flags},
@@ -127,6 +133,20 @@ def main():
     import torch_blocksparse as tb
     w = Attention(args.batch, args.block, args.dtype)
     step = w.step
+    # The literal reading of the command line first: W warm-up steps and K timed steps on a GPU that has done nothing
+    # else in this process (tables built, no settle steps, no per-launch pass before).  Reported as
+    # `ms_per_step_first_window`; `ms_per_step` further down is the steady state.
+    import gc
+    gc.collect()
+    gc.disable()
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_first_window = (time.perf_counter() - t0) * 1e3 / args.steps
     # Per-launch timing with HIP events on the launch stream, the eight launches of a step issued back to back in
     # step order (so each kernel sees the cache state its predecessor leaves), K steps, one synchronisation at the end.
     launches = w.launches() + [('calibration_copy', w.k_copy, 0.0, 2 * w.x_bytes)]
@@ -205,6 +225,7 @@ def main():
         'metric': 'effective TFLOP/s (nonzero blocks) sdd/dsd/dds + softmax GB/s, %s blk%d' % ({'f16': 'fp16', 'bf16': 'bf16'}[args.dtype], block),
         'value': round(6 * w.flops_mm / ms_per_step * 1e-9, 3), 'unit': 'TFLOP/s',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup, 'ms_per_step': round(ms_per_step, 4),
+        'ms_per_step_first_window': round(ms_first_window, 4),
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None, 'dtype': args.dtype, 'data': 'synthetic',
         'config': {'workload': 'sparse self-attention fwd+bwd: batch %d, 16 heads, seq 4096, head_dim 64, block %d, fixed '
                                'layout (local 4 blocks + 1 global per 16 at block 64, causal), scale 1/8, additive key-padding mask' % (B, block),
@@ -317,6 +338,39 @@ class Attention:
                 ('dds_bwd  (q^T.ds)^T', self.k_dds_bwd, f, b), ('dsd_bwd  ds.k', self.k_dsd_bwd, f, b)]
 
 
+def launch_roofline(kernel, flops, nbytes, ms, peak_tflops=MFMA_PEAK_TFLOPS):
+    """The roofline object of one launch.  A product is bound by min(matrix peak, arithmetic intensity x HBM peak) with the
+    intensity taken from the algorithmic bytes (every tensor touched once); a softmax by the HBM peak.  `frac` is the
+    achieved rate over that binding roof; products also carry their fraction of the raw matrix peak."""
+    if not flops:
+        gbs = nbytes / ms * 1e-6
+        return {'kernel': kernel, 'bound': 'hbm', 'achieved': round(gbs, 1), 'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+                'frac': round(gbs / HBM_PEAK_GBS, 4), 'traffic': None}
+    tf = flops / ms * 1e-9
+    hbm_roof = flops / nbytes * HBM_PEAK_GBS * 1e-3            # TFLOP/s at 8 TB/s for this flop : byte ratio
+    roof = min(peak_tflops, hbm_roof)
+    return {'kernel': kernel, 'bound': 'mfma' if peak_tflops <= hbm_roof else 'hbm', 'achieved': round(tf, 2), 'peak': round(roof, 1),
+            'unit': 'TFLOP/s', 'frac': round(tf / roof, 4), 'frac_of_matrix_peak': round(tf / peak_tflops, 4),
+            'flop_per_byte': round(flops / nbytes, 1), 'traffic': None}
+
+
+def xsd_kernel_name(block, dtype_bits, free_dim, sp_trans, dn_kc):
+    """Which kernel the library's dispatch gives a dsd/dds launch (csrc/capi.hip xsd_dispatch, in its order)."""
+    if dtype_bits == 16 and free_dim >= 256:
+        if block == 32 and dn_kc:
+            return 'k_xsd_rg_dl'
+        if block in (64, 128) and not (sp_trans and dn_kc):
+            return 'k_xsd_dl<%d>' % block
+    if dtype_bits == 16 and not dn_kc and free_dim % 64 == 0:
+        if block == 64:
+            return 'k_xsd64_rg<sparse operand %s>' % ('transposed' if sp_trans else 'as stored')
+        if block == 16:
+            return 'k_xsd64_rg<tiles of 4 x 4 blocks>'
+        if block == 32 and free_dim <= 128:
+            return 'k_xsd_rg_small'
+    return 'k_xsd (general)'
+
+
 def other_config(config, steps, warmup):
     """The configurations the headline metric is not quoted on: every launch timed on its own (HIP events, mean of
     `steps` back-to-back launches), effective throughput over the nonzero blocks, as a fraction of the fp16 MFMA peak
@@ -380,8 +434,18 @@ def other_config(config, steps, warmup):
         es = a.element_size()
         nbytes = es * (Z * nnz * block * block + Z * H * (M * K if mode != 'dsd' else K * N) + Z * H * (M * N if mode != 'sdd' else K * N))
         peak = FP32_PEAK_TFLOPS if dtype == torch.float32 else MFMA_PEAK_TFLOPS
+        bits = 32 if dtype == torch.float32 else 16
+        if mode == 'sdd':
+            kernel = ('k_sdd_rg_dl' if (block == 32 and K >= 256 and bits == 16) else
+                      'k_sdd64_rg' if (block in (16, 64) and bits == 16 and K in (64, 128) and not ta and tb_) else
+                      'k_sdd_rg_small' if (block == 32 and bits == 16 and K == 64 and not ta and tb_) else 'k_sdd (general)')
+        elif mode == 'dsd':      # kernel rows = rows of op(A); dense operand reduction-contiguous when B is read transposed
+            kernel = xsd_kernel_name(block, bits, N, ta, tb_)
+        else:                    # dds = dsd on the transposed problem
+            kernel = xsd_kernel_name(block, bits, M, not tb_, not ta)
         out.append({'launch': name, 'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'mfma_frac': round(fl / ms * 1e-9 / peak, 4),
-                    'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)})
+                    'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4),
+                    'roofline': launch_roofline(kernel, fl, nbytes, ms, peak)})
 
     if config == 1:
         torch.manual_seed(0)
@@ -391,7 +455,8 @@ def other_config(config, steps, warmup):
         sm = tb.Softmax(lay, 16)
         with torch.no_grad():
             ms = timeit(lambda: sm(x))
-        out.append({'launch': 'softmax fwd fp32 blk16', 'ms': round(ms, 4), 'GB/s': round(2 * x.numel() * 4 / ms * 1e-6, 1)})
+        out.append({'launch': 'softmax fwd fp32 blk16', 'ms': round(ms, 4), 'GB/s': round(2 * x.numel() * 4 / ms * 1e-6, 1),
+                    'roofline': launch_roofline('k_softmax_fwd', 0, 2 * x.numel() * 4, ms)})
         workload = 'README shape: sdd trans_a fp32 block 16 + softmax'
     elif config == 2:
         lay = bernoulli((16, 64, 64), 0.25, 2, one_per_row=True)
@@ -449,11 +514,108 @@ def other_config(config, steps, warmup):
                 ent = {'launch': name, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1), 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4)}
                 if flops:
                     ent['TFLOP/s'] = round(flops / ms * 1e-9, 2)
+                kernel = ('k_softmax_fwd' if 'softmax fwd' in name else 'k_softmax_bwd' if 'softmax bwd' in name else 'k_sdd64_rg' if name.startswith('sdd')
+                          else 'k_xsd64_rg<sparse operand %s>' % ('transposed' if '^T.' in name else 'as stored'))
+                ent['roofline'] = launch_roofline(kernel, flops, nbytes, ms)
                 out.append(ent)
         workload = ('BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, '
                     'forward and backward launches; bound: HBM (softmax bytes: 2|x| + the mask and rpe bytes the layout touches)')
     torch.cuda.empty_cache()
     return {'workload': workload, 'launches': out}
+
+
+def reference_bench_shapes(steps, warmup):
+    """The shapes the reference's own benchmark functions run (they are all it ever names; it publishes no numbers):
+      * tests/test_matmul.py:105-122  sdd, batch 1, 12 heads, hidden 512, block 16, 'fixed' layout of stride 64 with 4
+        vertical blocks, bidirectional, seq 4096, fp16, operands uniform in [0, 1); reported as the reference does:
+        2 * Z * K * nnz * block^2 flops over the time of the forward call
+      * tests/test_softmax.py:92-128  block 16, Z 2, H 4, density 0.4: 256 rows x (256 .. 3072) columns and (32 .. 480)
+        rows x 512 columns; block 64, Z 1, H 1, 'fixed' layout of stride 64 with 4 vertical blocks, unidirectional and
+        bidirectional, seq 1024 .. 8192; forward and backward; bytes counted as the reference counts them:
+        forward 2|x| + |attn_mask| + |kp_mask|, backward 3|x|  (tests/test_softmax.py:76-77)
+    Every launch timed on its own with HIP events, `steps` back-to-back launches after a warm-up."""
+    import gc
+    import torch
+    import torch_blocksparse as tb
+    dev = torch.device('cuda:0')
+    torch.manual_seed(1)
+
+    def timeit(f):
+        for _ in range(max(warmup, 3)):
+            f()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        f()
+        torch.cuda.synchronize()
+        one = max(time.perf_counter() - t0, 2e-5)
+        for _ in range(min(2000, int(0.025 / one) + 1)):
+            f()
+        gc.collect()
+        gc.disable()
+        try:
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                f()
+            e1.record()
+            e1.synchronize()
+        finally:
+            gc.enable()
+        return e0.elapsed_time(e1) / steps
+
+    out = []
+    # matmul: bench_op of tests/test_matmul.py
+    batch, heads, hidden, block, stride, L = 1, 12, 512, 16, 64, 4096
+    lay = tb.make_layout(heads, L // block, 'fixed', stride // block, False, 4, 1)
+    nnz = int(lay.sum())
+    x = torch.rand(batch, heads, L, hidden, device=dev, dtype=torch.float16)
+    w = torch.rand(batch, heads, hidden, L, device=dev, dtype=torch.float16)
+    op = tb.MatMul(lay, block, 'sdd', trans_a=False, trans_b=False)
+    with torch.no_grad():
+        ms = timeit(lambda: op(x, w))
+    fl = 2.0 * batch * hidden * nnz * block * block
+    nbytes = 2 * (batch * nnz * block * block + 2 * batch * heads * L * hidden)
+    out.append({'launch': 'sdd  batch 1, 12 heads, seq 4096, hidden 512, block 16, fixed layout (stride 64, 4 vertical), fp16', 'nnz_blocks': nnz,
+                'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'roofline': launch_roofline('k_sdd (general)', fl, nbytes, ms)})
+
+    # softmax: bench_op of tests/test_softmax.py
+    def softmax_case(label, Z, lay, block):
+        n = int(lay.sum())
+        N = lay.shape[2] * block
+        xs = torch.rand(Z, n, block, block, device=dev, dtype=torch.float16)
+        dx = torch.rand_like(xs)
+        sm = tb.Softmax(lay, block)
+        lut, maxlut = sm.make_lut(dev)
+        with torch.no_grad():
+            sm(xs, 0.4)                                     # leaves a softmax in xs: what the backward pass reads
+            ms_y = timeit(lambda: sm(xs, 0.4))
+            ms_dx = timeit(lambda: _bwd_softmax(tb, xs, dx, 0.4, lut, maxlut, lay.shape, block))
+        xb = xs.numel() * 2
+        gb_y, gb_dx = 2 * xb + N * N * 2 + Z * N * 2, 3 * xb      # as the reference counts (masks included although it passes none)
+        out.append({'launch': 'softmax ' + label, 'nnz_blocks': n, 'fwd_ms': round(ms_y, 4), 'bwd_ms': round(ms_dx, 4),
+                    'fwd_GB/s': round(gb_y / ms_y * 1e-6, 1), 'bwd_GB/s': round(gb_dx / ms_dx * 1e-6, 1),
+                    'fwd_GB/s_x_only': round(2 * xb / ms_y * 1e-6, 1),
+                    'roofline': launch_roofline('k_softmax_fwd', 0, 2 * xb, ms_y)})
+
+    def bernoulli(shape, density, seed):
+        g = torch.Generator().manual_seed(seed)
+        lay = (torch.rand(shape, generator=g) < density).long()
+        for h in range(shape[0]):
+            for r in range(shape[1]):
+                if lay[h, r].sum() == 0:
+                    lay[h, r, 0] = 1
+        return lay
+    for N in (256, 1024, 2048, 3072):                       # "# Columns" sweep (the reference runs every multiple of 256)
+        softmax_case('block 16, Z 2, H 4, 256 rows x %d columns, density 0.4' % N, 2, bernoulli((4, 16, N // 16), 0.4, N), 16)
+    for M in (32, 256, 480):                                # "# Rows" sweep
+        softmax_case('block 16, Z 2, H 4, %d rows x 512 columns, density 0.4' % M, 2, bernoulli((4, M // 16, 32), 0.4, M), 16)
+    for uni, tag in ((True, 'Sparse GPT2 (unidirectional)'), (False, 'Sparse BERT (bidirectional)')):
+        for ctx_len in (1024, 2048, 4096, 8192):
+            lay = tb.make_layout(1, ctx_len // 64, 'fixed', 1, uni, 4, 1)
+            softmax_case('%s, block 64, Z 1, H 1, seq %d' % (tag, ctx_len), 1, lay, 64)
+    torch.cuda.empty_cache()
+    return {'workload': "the reference's own benchmark shapes: tests/test_matmul.py:105-122 (sdd, block 16) and tests/test_softmax.py:92-128 "
+                        "(softmax sweeps); the reference publishes no numbers for them", 'launches': out}
 
 
 def _bwd_softmax(tb, y, dy, scale, lut, maxlut, spdims, block):
