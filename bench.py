@@ -673,8 +673,11 @@ def calibrate(args):
     w = Attention(8, 64)
     flush_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
 
-    def flush():
+    def flush():           # 1 GiB written: L2 and the memory-side cache end up full of DIRTY lines of another buffer
         probe.bsp_probe_stream(1, _lib.ptr(flush_buf), None, None, flush_buf.numel(), 256 * 16, stream)
+
+    def flush_clean():     # 1 GiB read: the caches end up full of CLEAN lines of another buffer (nothing to write back)
+        probe.bsp_probe_stream(0, _lib.ptr(flush_buf), None, None, flush_buf.numel(), 256 * 16, stream)
 
     launches = w.launches()
     with torch.no_grad():
@@ -686,9 +689,13 @@ def calibrate(args):
             prev = launches[i - 1][1]
             warm = timed(f, before=prev)        # the cache state of the step: the predecessor has just run
             cold = timed(f, before=flush)
+            flush()
+            torch.cuda.synchronize()
+            cold_clean = timed(f, before=flush_clean)
             res['launches'].append({'launch': name, 'bytes': nbytes, 'ms_after_predecessor': round(warm, 4),
                                     'GB/s_after_predecessor': round(nbytes / warm * 1e-6, 1), 'ms_cold': round(cold, 4),
-                                    'GB/s_cold': round(nbytes / cold * 1e-6, 1)})
+                                    'GB/s_cold': round(nbytes / cold * 1e-6, 1), 'ms_cold_clean': round(cold_clean, 4),
+                                    'GB/s_cold_clean': round(nbytes / cold_clean * 1e-6, 1)})
     print(json.dumps({'metric': 'streaming calibration, not the headline metric', 'n_gpus': 1, 'data': 'synthetic', **res}))
 
 

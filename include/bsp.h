@@ -143,7 +143,11 @@ int bsp_group_plan_build(const int32_t *d_layout, int H, int R, int C, int by_ro
 typedef enum {
   BSP_FLAG_GENERAL_ONLY = 1,  /* take the general kernels even where a specialised one would serve (for cross-checks) */
   BSP_FLAG_NO_GROUPS = 2,     /* ignore the group plan (the per-block / per-segment kernels run instead) */
-  BSP_FLAG_NO_WIDE = 4        /* skip the kernels specialised for a wide free dimension (dsd / dds, blocks 64 and 128) */
+  BSP_FLAG_NO_WIDE = 4,       /* skip the kernels specialised for a wide free dimension (dsd / dds, blocks 64 and 128) */
+  BSP_FLAG_PLAN_ROWPAIR = 8   /* bsp_sdd_matmul, block 16: d_gplan is a plan over PAIRS of block-rows (built by bsp_group_plan_build on
+                                 the layout with every two block-rows merged, entries widened to 13 ints: position, 4 member ids,
+                                 then the ids of the two blocks of each member, -1 where absent); plan_lines counts the pairs.  Such a
+                                 plan serves the long-reduction kernel (K >= 256, K % 32 == 0, 16-bit types) and nothing else */
 } bsp_launch_flags;
 
 /* sparse = dense x dense: replaces _sparse_matmul._sdd_matmul + the SDD branch of the kernel
@@ -155,8 +159,10 @@ typedef enum {
  * tiles inside each group may take the launch.  The plan describes the whole layout, not one pack level: if that
  * kernel ran, the return value is BSP_OK_WHOLE_LAYOUT and the caller skips the remaining pack levels (pass the plan
  * with the first level only).  A caller that has the plan but has not built the table yet (its greedy packing is the
- * one sequential step of the builders) may call with d_lut = NULL, pack = 0 and n_groups = the number of block-columns
- * of the layout (0 if unknown: the kernels for long reductions at blocks of 32 then do not apply): the result is
+ * one sequential step of the builders) may call with d_lut = NULL, pack = 0 and n_groups = an upper bound on the number of
+ * entries of any group of the plan: the number of block-columns of the layout always is one, the largest entry count
+ * among the plan's header rows is the tightest (it sizes the grid of the kernels for long reductions at blocks of 16
+ * and 32; 0 if unknown: those kernels then do not apply): the result is
  * BSP_OK_WHOLE_LAYOUT if a kernel that works from the plan alone took the product, else BSP_NEEDS_TABLE and nothing was
  * launched. */
 int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,

@@ -341,11 +341,34 @@ def test_sdd_with_a_long_reduction_at_block_32(dtype):
     run_case('sdd', False, True, 32, dtype, Z=2, H=3, M=22 * 32, N=19 * 32, K=320, layout=lay, seed=7, dist='randn', scale=0.2)
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_sdd_with_a_long_reduction_at_block_16(dtype):
+    # blocks of 16, reduction >= 256 and a multiple of 32: the same 128 x 256 products from a plan over pairs of
+    # block-rows, sixteen gathered block-columns per workgroup; every orientation, batch 2, layouts with an empty
+    # column, members with one of their two block-rows absent, a ragged last group (10 block-rows: 5 pairs) and
+    # more block-columns than one chunk (24 > 16); also the stripe layout of the reference's own benchmark
+    # (tests/test_matmul.py:105-122: 'fixed', one dense column in four, local windows of four blocks)
+    lay = random_layout((2, 10, 24), 0.3, 31)
+    lay[:, :, 5] = 0
+    lay[0, 3, :] = 0
+    lay[1, 8:, :] = 0
+    lay[1, 9, 2] = 1
+    for ta, tb_ in ((False, True), (True, False), (False, False), (True, True)):
+        run_case('sdd', ta, tb_, 16, dtype, Z=2, H=2, M=160, N=384, K=320, layout=lay, seed=40 + ta + 2 * tb_, dist='randn', scale=0.25)
+    stripes = tb.make_layout(3, 16, 'fixed', 4, False, 4, 1)
+    run_case('sdd', False, False, 16, dtype, Z=1, H=3, M=256, N=256, K=512, layout=stripes, seed=44, dist='randn', scale=0.25)
+    # reductions the kernel leaves to the others: not a multiple of 32, or short; and an odd number of block-rows
+    run_case('sdd', False, True, 16, dtype, Z=1, H=2, M=160, N=384, K=272, layout=lay, seed=45, dist='randn', scale=0.25)
+    run_case('sdd', False, True, 16, dtype, Z=1, H=2, M=160, N=384, K=64, layout=lay, seed=46, dist='randn', scale=0.25)
+    odd = random_layout((1, 7, 9), 0.5, 33)
+    run_case('sdd', False, True, 16, dtype, Z=1, H=1, M=112, N=144, K=256, layout=odd, seed=47, dist='randn', scale=0.25)
+
+
 def test_wide_kernels_agree_with_the_general_ones(monkeypatch):
     # the same launches with and without the wide-free-dimension / long-reduction kernels (a launch flag of the C ABI)
     from torch_blocksparse import _lib, matmul
     torch.manual_seed(77)
-    for block in (32, 64, 128):
+    for block in (16, 32, 64, 128):
         lay = random_layout((2, 6, 7), 0.4, 70 + block)
         nnz = int(lay.sum())
         sp = torch.randn(2, nnz, block, block, device=DEV, dtype=torch.float16)

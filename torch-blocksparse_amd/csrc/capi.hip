@@ -9,6 +9,7 @@ namespace {
 bool no_groups(int flags) { return (flags & BSP_FLAG_NO_GROUPS) != 0; }
 bool general_only(int flags) { return (flags & BSP_FLAG_GENERAL_ONLY) != 0; }
 bool no_wide(int flags) { return (flags & (BSP_FLAG_NO_WIDE | BSP_FLAG_GENERAL_ONLY)) != 0; }
+bool rowpair(int flags) { return (flags & BSP_FLAG_PLAN_ROWPAIR) != 0; }
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 bool block_ok(int block) { return block == 16 || block == 32 || block == 64 || block == 128; }
 int elems16(int dtype) { return dtype == BSP_F32 ? 4 : 8; }   // elements per 16 bytes
@@ -56,11 +57,15 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   const bool a_kc = !trans_a, b_kc = trans_b != 0;
   hipStream_t st = as_stream(stream);
   int rc = 0;
-  if (!d_lut) {   // the plan alone: n_groups then carries the number of block-columns of the layout
+  if (!d_lut) {   // the plan alone: n_groups then carries an upper bound on the entries of a group (at most the block-columns of the layout)
     g.cols = (int)n_groups; g.n_groups = 0;
-    rc = no_wide(flags) ? 0 : sdd_dl(dtype, g, block, a_kc, b_kc, st);
+    rc = no_wide(flags) ? 0 : sdd_dl(dtype, g, block, rowpair(flags), a_kc, b_kc, st);
     if (rc < 0) return rc;
     if (rc == 2) { BSP_LAUNCH_CHECK(); return BSP_OK_WHOLE_LAYOUT; }
+  }
+  if (rowpair(flags)) {   // a plan over pairs of block-rows serves the long-reduction kernel only
+    if (!d_lut) return BSP_NEEDS_TABLE;
+    g.gplan = nullptr;
   }
   rc = general_only(flags) ? 0 : sdd_fast64(dtype, g, block, pack, a_kc, b_kc, st);
   if (rc < 0) return rc;

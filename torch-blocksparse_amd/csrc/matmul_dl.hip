@@ -469,13 +469,21 @@ template <typename T> int launch_rg_dl(const XsdArgs &g, bool sp_trans, bool dn_
 // launch has to spare (it waits for operands either way) and removes all bookkeeping from the reduction loop: no
 // table is read in it.  Operand bytes per useful flop drop by 2 at a quarter of the blocks kept.
 // ---------------------------------------------------------------------------------------------------------
-constexpr int kSddCols = 8;      // block-columns per workgroup
+constexpr int kSddColsElems = 256;   // columns of the gathered B tile: 8 block-columns of 32, 16 of 16
 
-template <typename T, bool A_KC, bool B_KC>
+// BLOCK = 32: the group plan of the layout itself, entries (position, id of each member's block or -1).
+// BLOCK = 16: the same 128 x 256 product from blocks of 16.  The plan is over PAIRS of block-rows (a member = two
+// consecutive block-rows = 32 rows of A, present at a block-column if either has a block there), so that a group is
+// still 128 consecutive rows of A; a workgroup gathers sixteen block-columns of 16; an entry is (position, 4 member
+// flags, then the ids of the two blocks of each member, -1 where absent): 13 ints.
+template <typename T, bool A_KC, bool B_KC, int BLOCK>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) k_sdd_rg_dl(SddArgs g, int chunks) {
   typedef Mma<T, 32> M;
   typedef typename M::frag_t frag_t;
-  constexpr int B = 32, G = BSP_GROUP, J = kSddCols, TM = G * B, TN = J * B;
+  constexpr int B = 32, G = BSP_GROUP, CB = BLOCK, J = kSddColsElems / CB, TM = G * B, TN = J * CB;
+  constexpr int SUB = B / CB;                         // block-rows per member: 1 or 2
+  constexpr int ENT = SUB == 1 ? G + 1 : G + 1 + G * SUB;
+  static_assert(BLOCK == 16 || BLOCK == 32, "blocks of 16 or 32");
   static_assert(TN == kTN, "the gathered B tile is the dense tile of the other kernels");
   typedef DlTile<T, TM, A_KC> XT;
   typedef DlTile<T, TN, B_KC> YT;
@@ -492,6 +500,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const table_ptr hd = as_table(g.gplan) + 4 * ((w % per_z) / chunks);
   const int e0 = hd[0], ne = hd[1], h = hd[2], code = hd[3];
   if (chunk * J >= ne) return;                        // (the grid is sized for the longest possible group)
+  static_assert(J == kSddColsElems / BLOCK, "launch_sdd_rg_dl sizes the grid with the same J");
   const int left = ne - chunk * J;                    // entries of this chunk: min(left, J)
   const int line0 = (code & 0xffffff) * G;
   const int rows_a = g.lines * B;                     // rows of op(A) per head
@@ -522,16 +531,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const int ld = wave * YL + i;
     if constexpr (B_KC) {
       const int row = ld * 16 + (lane >> 2), chunk16 = (lane & 3) ^ kc_swz(row);
-      const int jj = row >> 5;
-      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J + (jj < left ? jj : left - 1))];
-      yoff[i] = ((int64_t)pos * B + (row & 31)) * ldb + chunk16 * 8;
+      const int jj = row / CB;
+      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)ENT * (e0 + chunk * J + (jj < left ? jj : left - 1))];
+      yoff[i] = ((int64_t)pos * CB + (row % CB)) * ldb + chunk16 * 8;
     } else {
       constexpr int CPR = TN / 8;
       const int j = ld * 64 + lane, k = j / CPR, slot = j % CPR;
       const int c = (((slot >> 1) ^ ks_swz<TN>(k)) << 1) | (slot & 1);
-      const int jj = c >> 2;                          // four chunks of 8 columns per block-column
-      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J + (jj < left ? jj : left - 1))];
-      yoff[i] = (int64_t)k * ldb + (int64_t)pos * B + (c & 3) * 8;
+      const int jj = c / (CB / 8);                    // CB / 8 chunks of 8 columns per block-column
+      const int pos = as_table(g.gplan)[4 * (int64_t)g.n_pgroups + (int64_t)ENT * (e0 + chunk * J + (jj < left ? jj : left - 1))];
+      yoff[i] = (int64_t)k * ldb + (int64_t)pos * CB + (c % (CB / 8)) * 8;
     }
   }
   typename M::acc_t acc[RM][RN];
@@ -545,14 +554,21 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   // them is absent) read from LDS.  The loads into LDS stay dense: their count per stage is fixed.
   unsigned present = 0;
   {
-    const table_ptr ids = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J);
+    const table_ptr ids = as_table(g.gplan) + 4 * (int64_t)g.n_pgroups + (int64_t)ENT * (e0 + chunk * J);
 #pragma unroll
     for (int i = 0; i < RM; i++)
 #pragma unroll
       for (int j = 0; j < RN; j++) {
-        const int m = wm * RM + i, jj = wn * RN + j;
-        const int id = ids[(G + 1) * (jj < left ? jj : left - 1) + 1 + m];
-        present |= (jj < left && id >= 0) ? 1u << (i * RN + j) : 0u;
+        // a 32 x 32 tile of the product covers one member and 32 / CB entries; the member's flag of an entry says
+        // whether any of its blocks exists there
+        const int m = wm * RM + i;
+        bool any = false;
+#pragma unroll
+        for (int t = 0; t < B / CB; t++) {
+          const int jj = (wn * RN + j) * (B / CB) + t;
+          any = any || (jj < left && ids[ENT * (jj < left ? jj : left - 1) + 1 + m] >= 0);
+        }
+        present |= any ? 1u << (i * RN + j) : 0u;
       }
   }
   const int ksteps = g.K / kTK;
@@ -616,22 +632,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       }
   __syncthreads();
   T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz;
-  const int32_t *ids = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)(G + 1) * (e0 + chunk * J);   // vector loads: the id differs from lane to lane
-  constexpr int CPB = B * B / 8;                      // 16-byte chunks per block
+  const int32_t *ids = g.gplan + 4 * (int64_t)g.n_pgroups + (int64_t)ENT * (e0 + chunk * J);   // vector loads: the id differs from lane to lane
+  constexpr int CPB = CB * CB / 8;                    // 16-byte chunks per block
+  constexpr int MR = G * SUB;                         // block-rows of the tile
 #pragma unroll 4
-  for (int c = tid; c < G * J * CPB; c += 256) {
+  for (int c = tid; c < MR * J * CPB; c += 256) {
     const int blk = c / CPB, within = c % CPB;
-    const int m = blk / J, jj = blk % J;
-    const int id = jj < left ? ids[(G + 1) * jj + 1 + m] : -1;
+    const int mr = blk / J, jj = blk % J;             // block-row of the tile (member mr / SUB, its block-row mr % SUB), entry
+    const int id = jj < left ? ids[ENT * jj + (SUB == 1 ? 1 + mr : 1 + G + mr)] : -1;
     if (id >= 0) {
-      const int r = within >> 2, cc = (within & 3) * 8;
-      *reinterpret_cast<u32x4 *>(pc + (int64_t)id * (B * B) + within * 8) = *reinterpret_cast<const u32x4 *>(stage + (m * B + r) * LDR + jj * B + cc);
+      const int r = within / (CB / 8), cc = (within % (CB / 8)) * 8;
+      *reinterpret_cast<u32x4 *>(pc + (int64_t)id * (CB * CB) + within * 8) = *reinterpret_cast<const u32x4 *>(stage + (mr * CB + r) * LDR + jj * CB + cc);
     }
   }
 }
 
-template <typename T> int launch_sdd_rg_dl(const SddArgs &g, bool a_kc, bool b_kc, hipStream_t st) {
-  const int chunks = (g.cols + kSddCols - 1) / kSddCols;
+template <typename T, int BLOCK> int launch_sdd_rg_dl(const SddArgs &g, bool a_kc, bool b_kc, hipStream_t st) {
+  constexpr int J = kSddColsElems / BLOCK;
+  const int chunks = (g.cols + J - 1) / J;
   const int64_t n_wg = (int64_t)g.n_pgroups * chunks * g.Z;
   if (n_wg <= 0) return BSP_OK;
   if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
@@ -640,8 +658,8 @@ template <typename T> int launch_sdd_rg_dl(const SddArgs &g, bool a_kc, bool b_k
 #define BSP_SDD_RG_LAUNCH(AK, BK)                                                                                       \
   do {                                                                                                                  \
     static std::atomic<uint64_t> done{0};                                                                               \
-    if (!raise_lds_limit((const void *)k_sdd_rg_dl<T, AK, BK>, SMEM, done)) return BSP_ERR_HIP;                         \
-    hipLaunchKernelGGL((k_sdd_rg_dl<T, AK, BK>), grid, wg, SMEM, st, g, chunks);                                       \
+    if (!raise_lds_limit((const void *)k_sdd_rg_dl<T, AK, BK, BLOCK>, SMEM, done)) return BSP_ERR_HIP;                  \
+    hipLaunchKernelGGL((k_sdd_rg_dl<T, AK, BK, BLOCK>), grid, wg, SMEM, st, g, chunks);                                \
   } while (0)
   if (a_kc && b_kc) BSP_SDD_RG_LAUNCH(true, true);
   else if (a_kc) BSP_SDD_RG_LAUNCH(true, false);
@@ -706,10 +724,13 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
 
 // sdd with a long reduction at blocks of 32 from the group plan alone: 2 = launched (every block of the layout is
 // written), 0 = not applicable, < 0 = error
-int sdd_dl(int dtype, const SddArgs &g, int block, bool a_kc, bool b_kc, hipStream_t st) {
-  if (dtype == BSP_F32 || block != 32 || !g.gplan || g.n_pgroups <= 0 || g.lines <= 0 || g.cols <= 0) return 0;
+int sdd_dl(int dtype, const SddArgs &g, int block, bool rowpair_plan, bool a_kc, bool b_kc, hipStream_t st) {
+  if (dtype == BSP_F32 || (block != 32 && block != 16) || !g.gplan || g.n_pgroups <= 0 || g.lines <= 0 || g.cols <= 0) return 0;
+  if ((block == 16) != rowpair_plan) return 0;        // blocks of 16 come with the plan over pairs of block-rows, and only they
   if (g.K < 256 || g.K % kTK) return 0;
-  const int rc = dtype == BSP_F16 ? launch_sdd_rg_dl<f16>(g, a_kc, b_kc, st) : launch_sdd_rg_dl<bf16>(g, a_kc, b_kc, st);
+  int rc;
+  if (block == 32) rc = dtype == BSP_F16 ? launch_sdd_rg_dl<f16, 32>(g, a_kc, b_kc, st) : launch_sdd_rg_dl<bf16, 32>(g, a_kc, b_kc, st);
+  else rc = dtype == BSP_F16 ? launch_sdd_rg_dl<f16, 16>(g, a_kc, b_kc, st) : launch_sdd_rg_dl<bf16, 16>(g, a_kc, b_kc, st);
   return rc == BSP_OK ? 2 : rc;
 }
 

@@ -21,7 +21,12 @@ namespace {
 // 80.5 / 115 with 2, 82 / 116 with 1, 86 / 126 with 8.
 template <int NB> constexpr int waves_per_group_fwd() { return NB >= 32 ? 1 : NB >= 16 ? 2 : 4; }
 template <int NB> constexpr int waves_per_group_bwd() { return NB >= 32 ? 1 : NB > 0 ? 2 : 4; }
-constexpr int kChunk = 8;           // blocks per step of the streaming variants
+// Blocks per step of the streaming variants (rows longer than the register variants hold): all loads of a step are in
+// flight together.  Such rows come with few wavefronts per byte (a 8192-column row of blocks of 64 is 128 blocks for one
+// wavefront), so the bytes in flight per wavefront decide the rate: 16 blocks per step where the registers allow it
+// (no relative position embedding / attention mask beside x), 8 otherwise.
+constexpr int kChunk = 8;
+constexpr int kChunkPlain = 16;
 
 template <typename T, int EV> struct RawVec;
 template <> struct RawVec<f16, 8> { typedef u32x4 type; };
@@ -462,7 +467,7 @@ __global__ void __launch_bounds__(64 * waves_per_group_fwd<NB>()) k_softmax_fwd(
     // of a chunk in flight together.  Pass 1 keeps a running maximum and a running sum per lane (the sum is rescaled
     // when the maximum grows), pass 2 reads x again and writes the result: 2 reads + 1 write of x.
     typedef Pack<T, GE::EV> P;
-    constexpr int CH = kChunk, NX = EXTRA ? CH : 1;
+    constexpr int CH = EXTRA ? kChunk : kChunkPlain, NX = EXTRA ? CH : 1;
     const float unit = logit_unit<T>();
     const float sc = a.scale * unit;
     const T *xb = reinterpret_cast<const T *>(a.x) + (int64_t)u.z * a.x_sz + u.rxm * BLOCK + u.col;
@@ -669,8 +674,8 @@ __global__ void __launch_bounds__(64 * waves_per_group_bwd<NB>()) k_softmax_bwd(
         }
     }
   } else {
-    // longer rows: two passes, kChunk blocks at a time with all loads of a chunk in flight together
-    constexpr int CH = kChunk;
+    // longer rows: two passes, kChunkPlain blocks at a time with all loads of a chunk in flight together
+    constexpr int CH = kChunkPlain;
     P py[CH], pd[CH];
     int64_t off[CH];
     auto load_chunk = [&](int b0) {

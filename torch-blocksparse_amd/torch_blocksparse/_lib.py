@@ -15,7 +15,7 @@ LIB_PATH = os.path.join(os.path.dirname(_HERE), 'lib', 'libbsp_hip.so')
 F16, BF16, F32 = 0, 1, 2
 DTYPES = {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}
 
-FLAG_GENERAL_ONLY, FLAG_NO_GROUPS, FLAG_NO_WIDE = 1, 2, 4   # bsp_launch_flags
+FLAG_GENERAL_ONLY, FLAG_NO_GROUPS, FLAG_NO_WIDE, FLAG_PLAN_ROWPAIR = 1, 2, 4, 8   # bsp_launch_flags
 
 OK = 0
 OK_WHOLE_LAYOUT = 1   # bsp_sdd_matmul: the group plan was used, every block of the layout is written

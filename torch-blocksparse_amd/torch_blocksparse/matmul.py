@@ -90,6 +90,8 @@ class GroupPlan:
     def __init__(self, table, n_groups, lines, n_split=0):
         self.table, self.n_groups, self.lines, self.n_split = table, n_groups, lines, n_split
         self.coarse = False
+        self.rowpair = False
+        self._max_entries = None
         self._ws = None
         self._ws_retired = []
 
@@ -162,6 +164,42 @@ class GroupPlan:
         out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines, plan.n_split)
         out.coarse = True
         return out
+
+    @staticmethod
+    def build_rowpair(layout, device, ctx=None):
+        """Plan of a block-16 layout for the long-reduction sdd kernel: every two consecutive block-rows form a member of 32
+        rows (present at a block-column if either has a block there), four members a group (128 rows of A), no chains,
+        groups head by head.  Entries: (position, 4 member ids, then the ids of the two blocks of each member, -1 where
+        absent).  None if the layout has an odd number of block-rows."""
+        H, R, C = layout.shape
+        if R % 2:
+            return None
+        ctx = _LayoutOnDevice.of(layout, device, ctx)
+        lay = ctx.lay != 0
+        pairs = lay.reshape(H, R // 2, 2, C)
+        present = pairs.any(2)
+        pctx = _LayoutOnDevice.__new__(_LayoutOnDevice)
+        pctx.device, pctx.lay = ctx.device, present.to(torch.int32).contiguous()
+        pctx.ws, pctx.ws_bytes = _lib.workspace(pctx.lay, ctx.device)
+        pctx.nnz = int(present.sum())
+        pctx._coarse = None
+        fine = torch.where(lay, torch.cumsum(lay.reshape(-1), 0, dtype=torch.int32).reshape(lay.shape) - 1, -1).to(torch.int32)
+        ids2 = fine.reshape(H, R // 2, 2, C).permute(0, 1, 3, 2)[present].reshape(-1, 2)        # per present pair, in nonzero() order
+        plan = GroupPlan.build(pctx.lay, True, ctx.device, thin_min=0, order_buckets=1, ctx=pctx)
+        ng, G = plan.n_groups, 4
+        header, entries = plan.table[:4 * ng], plan.table[4 * ng:].view(-1, G + 1)
+        ids = entries[:, 1:].to(torch.int64)
+        sub = torch.where((ids >= 0).unsqueeze(2), ids2[ids.clamp(min=0)], -1)
+        wide = torch.cat([entries, sub.reshape(entries.shape[0], 2 * G)], 1)
+        out = GroupPlan(torch.cat([header, wide.reshape(-1)]).contiguous(), ng, plan.lines, 0)
+        out.rowpair = True
+        return out
+
+    def max_entries(self):
+        """The largest number of entries of any group of the plan (read back from the device once and kept)."""
+        if self._max_entries is None:
+            self._max_entries = int(self.table[:4 * self.n_groups].view(-1, 4)[:, 1].max()) if self.n_groups else 0
+        return self._max_entries
 
     def workspace(self, free_dim, Z):
         """(pointer, bytes) of the scratch buffer the split chains of this plan need for a launch with this free dimension
@@ -307,6 +345,9 @@ class _sparse_matmul(torch.autograd.Function):
         luts.gplan_long = None
         if block == 32:
             luts.build_long = lambda: GroupPlan.build(layout, True, dev, thin_min=0, order_buckets=1, ctx=ctx)
+        elif block == 16 and R % 2 == 0:
+            # blocks of 16: the same kernel on pairs of block-rows (a plan and a flag of its own)
+            luts.build_long = lambda: GroupPlan.build_rowpair(layout, dev, ctx=ctx)
         if lazy and luts.gplan is not None:
             return luts, None, None, None
         widths, packs = luts.materialize()
@@ -338,14 +379,17 @@ class _sparse_matmul(torch.autograd.Function):
         # nothing was launched (NEEDS_TABLE), the tables are built and the plan goes with the first pack level.
         gplan = GroupPlan.args(getattr(luts, 'gplan', None))
         rc = _lib.NEEDS_TABLE
-        long_k = lazy and block == 32 and AS3 >= 256 and a.dtype != torch.float32 and getattr(luts, 'build_long', None) is not None
+        long_k = (lazy and block in (16, 32) and AS3 >= 256 and AS3 % 32 == 0 and a.dtype != torch.float32
+                  and getattr(luts, 'build_long', None) is not None)
         if long_k:
             # the kernel for long reductions works from its own plan, whether the tables exist or not
             if luts.gplan_long is None:
                 luts.gplan_long = luts.build_long()
             lp = GroupPlan.args(luts.gplan_long)
-            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), spdims[2], lp[0], lp[1], lp[2],
-                                    KERNEL_FLAGS, _lib.stream_ptr(a.device))
+            flags = KERNEL_FLAGS | (_lib.FLAG_PLAN_ROWPAIR if luts.gplan_long.rowpair else 0)
+            # (the largest group of the plan sizes the grid: workgroups for block-columns that no group reaches are not launched)
+            rc = lib.bsp_sdd_matmul(*operands, 0, ctypes.c_void_p(0), ctypes.c_void_p(0), min(spdims[2], luts.gplan_long.max_entries()),
+                                    lp[0], lp[1], lp[2], flags, _lib.stream_ptr(a.device))
             if rc not in (_lib.OK_WHOLE_LAYOUT, _lib.NEEDS_TABLE):
                 _lib.check(rc, 'bsp_sdd_matmul')
         elif lazy and luts.gplan is not None and luts.build is not None:
