@@ -171,6 +171,19 @@ int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, int trans_a
                    const uint8_t *d_valid, int64_t n_groups, const int32_t *d_gplan, int n_plan_groups, int plan_lines, int flags,
                    void *stream);
 
+/* sparse = dense x dense over a long reduction into few blocks of 128, the reduction cut into `parts` parts that run side by
+ * side: replaces _sparse_matmul._sdd_matmul (matmul.py:299-364) where the reference would have used the split-K lock path of
+ * its kernel (matmul.py:186-203; dead there, no locks or atomics here).  Blocks of 128 and 16-bit types only, K a multiple
+ * of 32; d_lut / d_valid / n_groups: the pack-1 level of bsp_sdd_lut_build.  Each part leaves an fp32 partial block in d_ws
+ * (bsp_sdd_splitk_workspace_bytes(Z, n_groups, parts) bytes, 16-byte aligned, no initialisation needed; unused when parts == 1)
+ * and a second small kernel adds the parts of a block in part order: repeated launches agree bit for bit.
+ * BSP_ERR_UNSUPPORTED for any other block size or dtype (the caller takes bsp_sdd_matmul). */
+int64_t bsp_sdd_splitk_workspace_bytes(int Z, int64_t n_groups, int parts);
+int bsp_sdd_matmul_splitk(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
+                          int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
+                          int64_t ldb, int64_t c_stride_z, int block, const int32_t *d_lut, const uint8_t *d_valid,
+                          int64_t n_groups, int parts, void *d_ws, int64_t ws_bytes, int flags, void *stream);
+
 /* dense = sparse x dense: replaces _sparse_matmul._dsd_matmul + the DSD branch (matmul.py:507-552, 56-82).
  * C[z, h] = op(A_sparse)[h] . op(B)[z, h], written transposed when trans_c.  N = free dimension of op(B).
  * a_stride_z = 0 shares one sparse operand over the batch.  d_lut / d_plan / width from bsp_dxx_lut_build

@@ -80,6 +80,32 @@ def test_block128_sdd_one_or_four_workgroups_per_block(Z):
     run_case('sdd', False, True, 128, torch.bfloat16, Z=Z, H=2, M=1024, N=1024, K=48, layout=lay, seed=10, backward=False)
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16])
+def test_block128_sdd_long_reduction_cut_into_parts(dtype, monkeypatch):
+    # few blocks of 128 and a long reduction (the weight gradient of a sparse linear layer): the reduction is cut into
+    # parts whose fp32 partial blocks a second kernel adds in part order.  All four orientations; reductions of 1056
+    # (33 steps over 4 parts: the last part is shorter), 544 (2 parts) and 4096 (16 parts); batch 2; a layout with an empty
+    # row; repeated launches agree bit for bit; the workspace is reused by a smaller launch; and the same products
+    # with the parts switched off (one workgroup per block writes the block directly)
+    from torch_blocksparse.matmul import _sparse_matmul
+    lay = random_layout((2, 3, 4), 0.5, 128)
+    lay[0, 1, :] = 0
+    for ta, tb_ in ((False, True), (True, False), (False, False), (True, True)):
+        run_case('sdd', ta, tb_, 128, dtype, Z=2, H=2, M=384, N=512, K=1056, layout=lay, seed=50 + ta + 2 * tb_, dist='randn', scale=0.2, backward=False)
+    run_case('sdd', True, False, 128, dtype, Z=1, H=2, M=384, N=512, K=544, layout=lay, seed=54, dist='randn', scale=0.2, backward=False)
+    run_case('sdd', True, False, 128, dtype, Z=1, H=2, M=384, N=512, K=4096, layout=lay, seed=55, dist='randn', scale=0.05, backward=False)
+    op = tb.MatMul(lay, 128, 'sdd', trans_a=True)
+    g = torch.Generator().manual_seed(56)
+    a = (0.1 * torch.randn(2, 2, 2048, 384, generator=g)).to(dtype).to(DEV)
+    b = torch.randn(2, 2, 2048, 512, generator=g).to(dtype).to(DEV)
+    c1, c2 = op(a, b), op(a, b)
+    c3 = op(a[:1], b[:1])
+    assert torch.equal(c1, c2) and torch.equal(c3, c1[:1])
+    monkeypatch.setattr(_sparse_matmul, 'SPLITK_TARGET_WORKGROUPS', 1)        # no parts: the general path
+    c4 = tb.MatMul(lay, 128, 'sdd', trans_a=True)(a, b)
+    assert_close(c1, c4.float(), dtype, 'sdd in parts vs in one piece')
+
+
 @pytest.mark.parametrize('block', [16, 32, 64, 128])
 @pytest.mark.parametrize('mode,trans_a,trans_b', [('dsd', False, False), ('dsd', True, True), ('dds', False, True), ('dds', True, False)])
 def test_narrow_free_dimension(block, mode, trans_a, trans_b):

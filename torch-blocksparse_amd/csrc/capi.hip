@@ -82,6 +82,37 @@ extern "C" int bsp_sdd_matmul(int dtype, const void *a, const void *b, void *c, 
   return BSP_OK;
 }
 
+extern "C" int64_t bsp_sdd_splitk_workspace_bytes(int Z, int64_t n_groups, int parts) {
+  if (Z <= 0 || n_groups <= 0 || parts <= 1) return 0;
+  return (int64_t)Z * n_groups * parts * (int64_t)(128 * 128 * sizeof(float));
+}
+
+extern "C" int bsp_sdd_matmul_splitk(int dtype, const void *a, const void *b, void *c, int trans_a, int trans_b, int Z, int K,
+                                     int64_t a_stride_z, int64_t a_stride_h, int64_t lda, int64_t b_stride_z, int64_t b_stride_h,
+                                     int64_t ldb, int64_t c_stride_z, int block, const int32_t *d_lut, const uint8_t *d_valid,
+                                     int64_t n_groups, int parts, void *d_ws, int64_t ws_bytes, int flags, void *stream) {
+  if (!a || !b || !c || !d_lut || Z <= 0 || K <= 0 || n_groups < 0 || parts < 1 || parts > 64) return BSP_ERR_ARG;
+  if (block != 128 || (dtype != BSP_F16 && dtype != BSP_BF16) || general_only(flags) || no_wide(flags)) return BSP_ERR_UNSUPPORTED;
+  if (K % 16) return BSP_ERR_K_MULTIPLE;
+  if (K % 32) return BSP_ERR_UNSUPPORTED;
+  if (!aligned16(a) || !aligned16(b) || !aligned16(c)) return BSP_ERR_ARG;
+  if (a_stride_z % 8 || a_stride_h % 8 || lda % 8 || b_stride_z % 8 || b_stride_h % 8 || ldb % 8 || c_stride_z % 8) return BSP_ERR_ARG;
+  if (parts > 1) {
+    if (!d_ws || !aligned16(d_ws)) return BSP_ERR_ARG;
+    if (ws_bytes < bsp_sdd_splitk_workspace_bytes(Z, n_groups, parts)) return BSP_ERR_CAPACITY;
+  }
+  SddArgs g;
+  g.a = a; g.b = b; g.c = c; g.Z = Z; g.K = K;
+  g.a_sz = a_stride_z; g.a_sh = a_stride_h; g.lda = lda;
+  g.b_sz = b_stride_z; g.b_sh = b_stride_h; g.ldb = ldb; g.c_sz = c_stride_z;
+  g.lut = d_lut; g.valid = d_valid; g.n_groups = n_groups;
+  g.gplan = nullptr; g.n_pgroups = 0; g.lines = 0;
+  const int rc = sdd128_splitk(dtype, g, parts, reinterpret_cast<float *>(d_ws), !trans_a, trans_b != 0, as_stream(stream));
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
 // Workspace of a plan with split chains: BSP_CHAIN_PARTS fp32 tiles of 64 x 64 per (split chain, free tile, batch).
 static int64_t xsd_ws_slots(int n_split, int free_dim, int Z) { return (int64_t)n_split * ((free_dim + 63) / 64) * Z; }
 

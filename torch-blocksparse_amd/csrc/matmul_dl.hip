@@ -669,6 +669,189 @@ template <typename T, int BLOCK> int launch_sdd_rg_dl(const SddArgs &g, bool a_k
   return BSP_OK;
 }
 
+// ---------------------------------------------------------------------------------------------------------
+// sdd over a long reduction into few blocks of 128 (the weight gradient of a block-sparse linear layer: 102 blocks,
+// reduction over 8192 tokens).  One workgroup per block leaves most of the chip idle, four 64 x 64 workgroups per block
+// fetch every operand row twice.  Here a workgroup computes a whole 128 x 128 block over a PART of the reduction with
+// the pipeline of k_xsd_dl (128 x 128 x 32 steps, three LDS stages of 16 KiB, three workgroups per CU) and leaves an
+// fp32 partial block in the caller's workspace; k_sdd_splitk_sum adds the parts of a block in part order and writes
+// it.  Deterministic, no locks, no atomics: this is what the reference's split-K lock path (matmul.py:186-203, dead
+// there) was meant for.  With a single part the block is written directly.
+// Work item w: block fastest, then part, then batch: the workgroups that start together on an XCD (a contiguous range
+// of w) then work on the same part of the reduction, and blocks of one block-row (neighbours in the table) find the
+// rows of A they share in L2, as blocks of one block-column do with B.
+// ---------------------------------------------------------------------------------------------------------
+struct SplitK { int parts; int steps_per_part; float *ws; };
+
+template <typename T, bool A_KC, bool B_KC>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 3))) k_sdd128_splitk(SddArgs g, SplitK sk) {
+  typedef Mma<T, 32> M;
+  typedef typename M::frag_t frag_t;
+  constexpr int BL = 128;
+  typedef DlTile<T, BL, A_KC> XT;
+  typedef DlTile<T, BL, B_KC> YT;
+  constexpr int STAGE = XT::BYTES + YT::BYTES;
+  constexpr int XL = XT::LOADS / 4, YL = YT::LOADS / 4, L = XL + YL;
+  constexpr int RM = 2, RN = 2;                       // 2 x 2 wavefronts of 64 x 64
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  const int64_t per_z = g.n_groups * sk.parts;
+  const int64_t w = xcd_remap(blockIdx.x, per_z * g.Z);
+  const int z = (int)(w / per_z);
+  const int64_t grp = (w % per_z) % g.n_groups;
+  const int part = (int)((w % per_z) / g.n_groups);
+  if (g.valid && !g.valid[grp]) return;
+  const table_ptr e = as_table(g.lut) + grp * 4;
+  const int h = e[0], bi = e[1], bj = e[2], id = e[3];
+  const int64_t lda = g.lda, ldb = g.ldb;
+  const int ksteps_all = g.K / kTK;
+  const int s0 = part * sk.steps_per_part;
+  const int ksteps = min(sk.steps_per_part, ksteps_all - s0);
+  // (a part past the end of the reduction has nothing to add: it leaves a zero block, so that the sum reads no garbage)
+  const T *pa = reinterpret_cast<const T *>(g.a) + z * g.a_sz + h * g.a_sh + (A_KC ? (int64_t)bi * BL * lda : (int64_t)bi * BL);
+  const T *pb = reinterpret_cast<const T *>(g.b) + z * g.b_sz + h * g.b_sh + (B_KC ? (int64_t)bj * BL * ldb : (int64_t)bj * BL);
+  int64_t xoff[XL], yoff[YL];
+#pragma unroll
+  for (int i = 0; i < XL; i++) xoff[i] = A_KC ? XT::lane_offset(wave * XL + i, lane, lda, 1) : XT::lane_offset(wave * XL + i, lane, 1, lda);
+#pragma unroll
+  for (int i = 0; i < YL; i++) yoff[i] = B_KC ? YT::lane_offset(wave * YL + i, lane, ldb, 1) : YT::lane_offset(wave * YL + i, lane, 1, ldb);
+  typename M::acc_t acc[RM][RN];
+#pragma unroll
+  for (int i = 0; i < RM; i++)
+#pragma unroll
+    for (int j = 0; j < RN; j++)
+#pragma unroll
+      for (int v = 0; v < M::NACC; v++) acc[i][j][v] = 0.f;
+  auto issue = [&](int s) {
+    const int64_t k0 = (int64_t)(s0 + (s < ksteps ? s : ksteps - 1)) * kTK;
+    const T *xb = pa + (A_KC ? k0 : k0 * lda);
+    const T *yb = pb + (B_KC ? k0 : k0 * ldb);
+    unsigned char *st = smem + (s % kStages) * STAGE;
+#pragma unroll
+    for (int i = 0; i < XL; i++)
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(xb + xoff[i]), BSP_LDS_PTR(st + (wave * XL + i) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int i = 0; i < YL; i++)
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(yb + yoff[i]), BSP_LDS_PTR(st + XT::BYTES + (wave * YL + i) * 1024), 16, 0, 0);
+  };
+  if (ksteps > 0) {
+#pragma unroll
+    for (int s = 0; s < kStages - 1; s++) issue(s);
+    for (int s = 0; s < ksteps; s++) {
+      BSP_WAIT_VM(L * (kStages - 2));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      issue(s + kStages - 1);                          // (past the end: the last step again, a fixed number of loads per step)
+      const unsigned char *st = smem + (s % kStages) * STAGE;
+      frag_t xf[kTK / 16][RM], yf[kTK / 16][RN];
+#pragma unroll
+      for (int kk = 0; kk < kTK / 16; kk++) {
+#pragma unroll
+        for (int i = 0; i < RM; i++) xf[kk][i] = XT::frag(st, (wm * RM + i) * 32, kk, lane);
+#pragma unroll
+        for (int j = 0; j < RN; j++) yf[kk][j] = YT::frag(st + XT::BYTES, (wn * RN + j) * 32, kk, lane);
+      }
+#pragma unroll
+      for (int kk = 0; kk < kTK / 16; kk++)
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+          for (int j = 0; j < RN; j++) acc[i][j] = M::run(yf[kk][j], xf[kk][i], acc[i][j]);   // 4 consecutive values run along the block's columns
+    }
+    BSP_WAIT_VM(0);
+  }
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  // acc[i][j][4 * g4 + e] = C[row (wm * RM + i) * 32 + lane % 32][col (wn * RN + j) * 32 + 8 * g4 + 4 * (lane / 32) + e]
+  if (sk.parts > 1) {
+    // fp32 partial block, 16 bytes per lane (the parts of a block are summed by k_sdd_splitk_sum)
+    float *ws = sk.ws + (((int64_t)z * g.n_groups + grp) * sk.parts + part) * (BL * BL);
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+#pragma unroll
+      for (int j = 0; j < RN; j++)
+#pragma unroll
+        for (int g4 = 0; g4 < 4; g4++) {
+          const int row = (wm * RM + i) * 32 + (lane & 31), col = (wn * RN + j) * 32 + 8 * g4 + 4 * (lane >> 5);
+          const f32x4 v = {acc[i][j][4 * g4 + 0], acc[i][j][4 * g4 + 1], acc[i][j][4 * g4 + 2], acc[i][j][4 * g4 + 3]};
+          *reinterpret_cast<f32x4 *>(ws + row * BL + col) = v;
+        }
+    return;
+  }
+  constexpr int LDR = BL + 8;
+  static_assert(BL * LDR * 2 <= kStages * STAGE, "the staged block fits into the ring");
+  T *stage = reinterpret_cast<T *>(smem);
+#pragma unroll
+  for (int i = 0; i < RM; i++)
+#pragma unroll
+    for (int j = 0; j < RN; j++)
+#pragma unroll
+      for (int g4 = 0; g4 < 4; g4++) {
+        const int row = (wm * RM + i) * 32 + (lane & 31), col = (wn * RN + j) * 32 + 8 * g4 + 4 * (lane >> 5);
+        union { u32x2 raw; T e[4]; } u;
+#pragma unroll
+        for (int e2 = 0; e2 < 4; e2++) u.e[e2] = from_float<T>(acc[i][j][4 * g4 + e2]);
+        *reinterpret_cast<u32x2 *>(stage + row * LDR + col) = u.raw;
+      }
+  __syncthreads();
+  T *pc = reinterpret_cast<T *>(g.c) + z * g.c_sz + (int64_t)id * (BL * BL);
+#pragma unroll 4
+  for (int c = tid; c < BL * BL / 8; c += 256) {
+    const int row = c >> 4, cc = (c & 15) * 8;
+    *reinterpret_cast<u32x4 *>(pc + row * BL + cc) = *reinterpret_cast<const u32x4 *>(stage + row * LDR + cc);
+  }
+}
+
+// c[z, id] = sum over the parts, in part order, of the fp32 partial blocks; one thread per 8 elements
+template <typename T>
+__global__ void __launch_bounds__(256) k_sdd_splitk_sum(SddArgs g, SplitK sk) {
+  constexpr int BB = 128 * 128;
+  const int64_t chunk = (int64_t)blockIdx.x * 256 + threadIdx.x;      // 8 consecutive elements of one block
+  const int64_t blk = chunk / (BB / 8);                               // z * n_groups + grp
+  if (blk >= g.n_groups * g.Z) return;
+  const int64_t grp = blk % g.n_groups, z = blk / g.n_groups;
+  if (g.valid && !g.valid[grp]) return;
+  const int within = (int)(chunk % (BB / 8)) * 8;
+  const float *ws = sk.ws + blk * sk.parts * BB + within;
+  f32x4 lo = {0.f, 0.f, 0.f, 0.f}, hi = {0.f, 0.f, 0.f, 0.f};
+  for (int p = 0; p < sk.parts; p++) {
+    lo += __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ws + (int64_t)p * BB));
+    hi += __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(ws + (int64_t)p * BB + 4));
+  }
+  union { u32x4 raw; T e[8]; } u;
+#pragma unroll
+  for (int k = 0; k < 4; k++) { u.e[k] = from_float<T>(lo[k]); u.e[4 + k] = from_float<T>(hi[k]); }
+  const int id = as_table(g.lut)[grp * 4 + 3];
+  *reinterpret_cast<u32x4 *>(reinterpret_cast<T *>(g.c) + z * g.c_sz + (int64_t)id * BB + within) = u.raw;
+}
+
+template <typename T> int launch_sdd128_splitk(const SddArgs &g, const SplitK &sk, bool a_kc, bool b_kc, hipStream_t st) {
+  const int64_t n_wg = g.n_groups * g.Z * sk.parts;
+  if (n_wg <= 0) return BSP_OK;
+  if (n_wg >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  constexpr int SMEM = kStages * 2 * 128 * kTK * 2;
+  dim3 grid((unsigned)n_wg), wg(256);
+#define BSP_SPLITK_LAUNCH(AK, BK)                                                                                       \
+  do {                                                                                                                  \
+    static std::atomic<uint64_t> done{0};                                                                               \
+    if (!raise_lds_limit((const void *)k_sdd128_splitk<T, AK, BK>, SMEM, done)) return BSP_ERR_HIP;                     \
+    hipLaunchKernelGGL((k_sdd128_splitk<T, AK, BK>), grid, wg, SMEM, st, g, sk);                                       \
+  } while (0)
+  if (a_kc && b_kc) BSP_SPLITK_LAUNCH(true, true);
+  else if (a_kc) BSP_SPLITK_LAUNCH(true, false);
+  else if (b_kc) BSP_SPLITK_LAUNCH(false, true);
+  else BSP_SPLITK_LAUNCH(false, false);
+#undef BSP_SPLITK_LAUNCH
+  if (sk.parts > 1) {
+    const int64_t chunks = g.n_groups * g.Z * (128 * 128 / 8);
+    hipLaunchKernelGGL((k_sdd_splitk_sum<T>), dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, g, sk);
+  }
+  return BSP_OK;
+}
+
 template <typename T, int BLOCK> int launch_dl(const XsdArgs &g0, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st) {
   const int64_t n_wg = (int64_t)g0.width * ((g0.NF + kTN - 1) / kTN) * g0.Z;
   if (n_wg <= 0) return BSP_OK;
@@ -720,6 +903,16 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
   if (dtype == BSP_F16) rc = block == 128 ? launch_dl<f16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<f16, 64>(g, sp_trans, dn_kc, out_nc, st);
   else rc = block == 128 ? launch_dl<bf16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<bf16, 64>(g, sp_trans, dn_kc, out_nc, st);
   return rc == BSP_OK ? 1 : rc;
+}
+
+// sdd at blocks of 128 over a reduction cut into `parts` parts (pack-1 table rows; ws: parts fp32 blocks per table row and
+// batch, may be null when parts == 1): BSP_OK = launched, BSP_ERR_UNSUPPORTED = not this kernel's case
+int sdd128_splitk(int dtype, const SddArgs &g, int parts, float *ws, bool a_kc, bool b_kc, hipStream_t st) {
+  if (dtype == BSP_F32 || parts < 1 || g.K % kTK || (parts > 1 && !ws)) return BSP_ERR_UNSUPPORTED;
+  const int steps = g.K / kTK;
+  SplitK sk;
+  sk.parts = parts; sk.steps_per_part = (steps + parts - 1) / parts; sk.ws = ws;
+  return dtype == BSP_F16 ? launch_sdd128_splitk<f16>(g, sk, a_kc, b_kc, st) : launch_sdd128_splitk<bf16>(g, sk, a_kc, b_kc, st);
 }
 
 // sdd with a long reduction at blocks of 32 from the group plan alone: 2 = launched (every block of the layout is

@@ -718,5 +718,6 @@ int xsd_fast64(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc
 int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bool out_nc, hipStream_t st);
 // sdd with a long reduction at blocks of 32, from the group plan alone (matmul_dl.hip): 2 = launched and every block written
 int sdd_dl(int dtype, const SddArgs &g, int block, bool rowpair_plan, bool a_kc, bool b_kc, hipStream_t st);
+int sdd128_splitk(int dtype, const SddArgs &g, int parts, float *ws, bool a_kc, bool b_kc, hipStream_t st);
 
 }  // namespace bsp

@@ -20,6 +20,7 @@ FLAG_GENERAL_ONLY, FLAG_NO_GROUPS, FLAG_NO_WIDE, FLAG_PLAN_ROWPAIR = 1, 2, 4, 8 
 OK = 0
 OK_WHOLE_LAYOUT = 1   # bsp_sdd_matmul: the group plan was used, every block of the layout is written
 NEEDS_TABLE = 2       # bsp_sdd_matmul called with the plan alone: nothing launched, the sdd table is needed
+ERR_UNSUPPORTED = -2
 ERR_CAPACITY = -3
 ERR_EMPTY_HEAD = -4
 ERR_ROW_TOO_LONG = -6
@@ -47,6 +48,9 @@ SIGNATURES = {
     'bsp_xsd_workspace_bytes': (_i64, [_i, _i, _i]),
     'bsp_sdd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _i, _vp, _vp,
                             _i64, _vp, _i, _i, _i, _vp]),
+    'bsp_sdd_splitk_workspace_bytes': (_i64, [_i, _i64, _i]),
+    'bsp_sdd_matmul_splitk': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
+                                   _i64, _i, _vp, _i64, _i, _vp]),
     'bsp_dsd_matmul': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
                             _i, _vp, _i, _i, _i, _vp, _i64, _i, _vp]),
     'bsp_dsd_matmul_noalloc': (_i, [_i, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _i, _vp, _vp,
