@@ -83,6 +83,24 @@ def test_long_rows_streaming_variant(block, cols):
     run_case(1, 1, 2, cols, block, torch.float32, 0.95, cols + 1, scale=0.5)
 
 
+@pytest.mark.parametrize('dtype', [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize('block,cols', [(16, 70), (16, 200), (32, 70), (32, 140), (64, 20), (64, 40), (64, 100), (128, 20), (128, 60)])
+def test_long_rows_one_wavefront_per_row(block, cols, dtype):
+    # rows of more blocks than the register variants hold: one wavefront per row with 4, 8 or 16 sixteen-byte pieces per
+    # lane (every step count for every block size); rows of ragged lengths in one launch (a full row, a short one, an
+    # empty one, a single block); every mask at once in both modes; batch 2, 2 heads.  The longest rows of fp32 at
+    # block 128 (60 blocks = 7680 elements, more than 16 steps hold) fall back to the variant that re-reads x.
+    lay = random_layout((2, 4, cols), 0.7, cols + block)
+    lay[0, 0, :] = 1
+    lay[0, 1, :] = 0
+    lay[0, 1, cols // 2] = 1
+    lay[1, 2, :] = 0
+    lay[1, 3, :3] = 1
+    run_case(2, 2, 4, cols, block, dtype, 0, 400 + cols, scale=0.3, layout=lay)
+    run_case(1, 2, 4, cols, block, dtype, 0, 500 + cols, scale=0.5, rpe=True, kpm='add', attn='mul', layout=lay)
+    run_case(1, 2, 4, cols, block, dtype, 0, 600 + cols, scale=0.5, kpm='mul', attn='add', layout=lay)
+
+
 @pytest.mark.parametrize('longest', [1, 2, 3, 4, 5, 6, 7, 8, 9, 16, 17, 18, 19, 22, 27, 30, 32, 33])
 def test_every_row_length_bucket(longest):
     # one kernel instantiation per bucket of "blocks kept in registers": the longest row decides which one runs, the
