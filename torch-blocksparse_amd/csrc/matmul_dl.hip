@@ -50,10 +50,14 @@ constexpr int kStages = 3;
 __device__ __forceinline__ int kc_swz(int row) { return (row >> 2) & 3; }
 __device__ __forceinline__ int kc_offset(int row, int chunk) { return row * 64 + ((chunk ^ kc_swz(row)) << 4); }
 // Reduction strided: [32 reduction indices][R elements], as in memory.  The transposing read of a 16-lane group takes
-// 32 contiguous bytes (a pair of chunks) from each of four consecutive reduction rows; pair p of row k sits at pair slot
-// p ^ (k & 3) (R >= 64: a row is a multiple of 128 bytes, so unswizzled rows would all start in the same bank).
-// R = 32: a row is 64 bytes = 2 pairs, rows k and k + 2 start in the same bank: pair slot p ^ ((k >> 1) & 1).
-template <int R> __device__ __forceinline__ int ks_swz(int k) { return R >= 64 ? (k & 3) : ((k >> 1) & 1); }
+// 32 contiguous bytes (a pair of chunks) from each of four consecutive reduction rows, and two such groups (neighbouring
+// pairs p, p + 1 of the same four rows) are served together: eight pieces of 32 bytes that should cover the 64 banks
+// once.  R >= 128 (a row is a multiple of 256 bytes: every row starts in bank 0): pair p of row k sits at pair slot
+// p ^ 2 (k & 3), so the even pair lands on the four even slots and the odd pair on the four odd ones (with p ^ (k & 3)
+// the two groups met in the same four slots: half of the LDS cycles of the kernels that read both operands this way
+// were bank conflicts).  R = 64 (128-byte rows: two rows per bank period): p ^ (k & 3).  R = 32 (a row is 2 pairs,
+// rows k and k + 2 start in the same bank): p ^ ((k >> 1) & 1).
+template <int R> __device__ __forceinline__ int ks_swz(int k) { return R >= 128 ? ((k & 3) << 1) : R >= 64 ? (k & 3) : ((k >> 1) & 1); }
 template <int R> __device__ __forceinline__ int ks_offset(int k, int col) {   // col in elements, multiple of 4
   const int chunk = col >> 3, pair = (chunk >> 1) ^ ks_swz<R>(k);
   return k * (R * 2) + (((pair << 1) | (chunk & 1)) << 4) + ((col & 7) << 1);
@@ -888,8 +892,8 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
   if (dtype == BSP_F32 || g.NF < 256) return 0;
   if (block == 32) {   // needs the group plan (whole blocks, no split chains)
     // Measured on 2048^3 products at a quarter of the blocks (8 x 16 of them): with the dense operand's reduction
-    // contiguous 1.60-1.83 ms against 1.89-2.05 for the general kernel; with it strided the general kernel's 1.54 ms
-    // stand against 1.71, so those stay where they were.
+    // contiguous 1.60-1.83 ms against 1.89-2.05 for the general kernel; with it strided the general kernel's 1.47-1.58 ms
+    // stand against 1.70-1.73 (also with the conflict-free layout of the strided tiles), so those stay where they were.
     if (!dn_kc) return 0;
     if (!g.gplan || g.n_pgroups <= 0 || g.lines <= 0 || g.n_split != 0) return 0;
     const int rc = dtype == BSP_F16 ? launch_rg_dl<f16>(g, sp_trans, dn_kc, out_nc, st) : launch_rg_dl<bf16>(g, sp_trans, dn_kc, out_nc, st);
@@ -897,7 +901,8 @@ int xsd_dl(int dtype, const XsdArgs &g, int block, bool sp_trans, bool dn_kc, bo
   }
   if (block != 64 && block != 128) return 0;
   // (sparse operand transposed and dense operand with the reduction contiguous, the dX product of a sparse linear layer:
-  // measured 0.064 ms here against 0.059 ms for the general kernel at block 128, equal at block 64: left where it was)
+  // measured 0.064 ms here against 0.059 ms for the general kernel at block 128, 0.0595 against 0.0596 once the strided
+  // tiles were free of bank conflicts, equal at block 64: left where it was)
   if (sp_trans && dn_kc) return 0;
   int rc;
   if (dtype == BSP_F16) rc = block == 128 ? launch_dl<f16, 128>(g, sp_trans, dn_kc, out_nc, st) : launch_dl<f16, 64>(g, sp_trans, dn_kc, out_nc, st);
