@@ -436,7 +436,8 @@ def other_config(config, steps, warmup):
         peak = FP32_PEAK_TFLOPS if dtype == torch.float32 else MFMA_PEAK_TFLOPS
         bits = 32 if dtype == torch.float32 else 16
         if mode == 'sdd':
-            kernel = ('k_sdd_rg_dl' if (block == 32 and K >= 256 and bits == 16) else
+            kernel = ('k_sdd_rg_dl' if (block in (16, 32) and K >= 256 and K % 32 == 0 and bits == 16) else
+                      'k_sdd128_splitk + k_sdd_splitk_sum' if (block == 128 and bits == 16 and K >= 512 and K % 32 == 0 and nnz * Z < 768) else
                       'k_sdd64_rg' if (block in (16, 64) and bits == 16 and K in (64, 128) and not ta and tb_) else
                       'k_sdd_rg_small' if (block == 32 and bits == 16 and K == 64 and not ta and tb_) else 'k_sdd (general)')
         elif mode == 'dsd':      # kernel rows = rows of op(A); dense operand reduction-contiguous when B is read transposed
@@ -576,7 +577,7 @@ def reference_bench_shapes(steps, warmup):
     fl = 2.0 * batch * hidden * nnz * block * block
     nbytes = 2 * (batch * nnz * block * block + 2 * batch * heads * L * hidden)
     out.append({'launch': 'sdd  batch 1, 12 heads, seq 4096, hidden 512, block 16, fixed layout (stride 64, 4 vertical), fp16', 'nnz_blocks': nnz,
-                'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'roofline': launch_roofline('k_sdd (general)', fl, nbytes, ms)})
+                'ms': round(ms, 4), 'TFLOP/s': round(fl / ms * 1e-9, 2), 'roofline': launch_roofline('k_sdd_rg_dl<block 16>', fl, nbytes, ms)})
 
     # softmax: bench_op of tests/test_softmax.py
     def softmax_case(label, Z, lay, block):
