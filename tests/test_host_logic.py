@@ -246,3 +246,22 @@ def test_replace_mha_takes_the_reference_form_with_one_info_argument():
     assert isinstance(model.self_attn, tb.MultiheadAttention)
     with pytest.raises(TypeError):
         tb.replace_mha(model, layout)
+
+
+def test_sdd_in_parts_argument_checks_and_workspace_size():
+    # host-side checks of bsp_sdd_matmul_splitk (nothing is launched: every call below is refused before it touches the GPU)
+    import ctypes
+    lib = _lib.load()
+    assert lib.bsp_sdd_splitk_workspace_bytes(1, 102, 1) == 0
+    assert lib.bsp_sdd_splitk_workspace_bytes(2, 10, 4) == 2 * 10 * 4 * 128 * 128 * 4
+    buf = (ctypes.c_char * 4096)()
+    base = (ctypes.addressof(buf) + 255) // 256 * 256
+    ptr = ctypes.c_void_p(base)
+
+    def call(dtype=_lib.F16, a=ptr, K=1024, block=128, parts=4, ws=ptr, ws_bytes=1 << 40, lda=1024, flags=0):
+        return lib.bsp_sdd_matmul_splitk(dtype, a, ptr, ptr, 1, 0, 1, K, 0, 0, lda, 0, 0, 1024, 0, block, ptr, None, 5, parts, ws, ws_bytes, flags, None)
+    assert call(a=None) == -1 and call(parts=0) == -1 and call(parts=65) == -1 and call(lda=1021) == -1       # BSP_ERR_ARG
+    assert call(block=64) == _lib.ERR_UNSUPPORTED and call(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
+    assert call(K=1000) == _lib.ERR_K_MULTIPLE and call(K=1040) == _lib.ERR_UNSUPPORTED                         # 16 | K, 32 | K
+    assert call(flags=_lib.FLAG_GENERAL_ONLY) == _lib.ERR_UNSUPPORTED and call(flags=_lib.FLAG_NO_WIDE) == _lib.ERR_UNSUPPORTED
+    assert call(ws=None) == -1 and call(ws_bytes=1024) == _lib.ERR_CAPACITY
