@@ -102,3 +102,46 @@ def test_split_chains_captured_then_a_larger_eager_call_between_replays():
         assert torch.equal(out, eager), 'replay %d differs from the eager run' % rep
         assert all(bool((f == float(rep)).all()) for f in filler)
         del big, filler
+
+
+def test_sparse_linear_layer_captured_and_replayed():
+    # A block-128 sparse linear layer, forward and backward: the wide dds kernels and the weight gradient as an sdd
+    # in parts (fp32 partial blocks in a workspace of the operator, allocated by the warm-up step).  Replays must equal
+    # the eager run bit for bit, with eager work and a larger eager call in between.
+    torch.manual_seed(21)
+    block, tokens, feat = 128, 1024, 512
+    lay = (torch.rand(1, feat // block, feat // block) < 0.5).long()
+    lay[0, 0, 0] = 1
+    lin = tb.Linear(feat, feat, block, lay).to(DEV).half()
+    x = torch.randn(tokens, feat, device=DEV, dtype=torch.float16)
+    dy = torch.randn(tokens, feat, device=DEV, dtype=torch.float16)
+
+    def step(x, dy):
+        xg = x.detach().clone().requires_grad_(True)
+        y = lin(xg)
+        dx, dw = torch.autograd.grad(y, (xg, lin.weight), dy)
+        return y.detach(), dx, dw
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(x, dy)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    sx, sdy = x.clone(), dy.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step(sx, sdy)
+    big_x = torch.randn(4 * tokens, feat, device=DEV, dtype=torch.float16)
+    for rep in range(3):
+        step(big_x, torch.randn_like(big_x))                 # a longer reduction: more parts, a larger workspace
+        fx, fdy = torch.randn_like(sx), torch.randn_like(sdy)
+        eager = step(fx, fdy)
+        torch.cuda.synchronize()
+        sx.copy_(fx)
+        sdy.copy_(fdy)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, a, b in zip(('y', 'dx', 'dw'), out, eager):
+            assert torch.equal(a, b), 'replay %d differs from the eager run: %s' % (rep, name)
