@@ -1,0 +1,278 @@
+"""GPU: the fused attention chain (bsp_attention_fwd / bsp_attention_bwd behind attention_chain) against the dense fp32
+oracle, against the three-operator chain it stands for, and at the points where it must hand over to that chain."""
+import ctypes
+
+import pytest
+import torch
+
+import torch_blocksparse as tb
+from torch_blocksparse import _lib, attention_core as ac
+from oracle import dense_oracle as D
+from helpers import assert_close, guard_allocations
+
+pytestmark = pytest.mark.gpu
+DEV = 'cuda'
+
+
+@pytest.fixture(autouse=True)
+def fused_on():
+    old = ac.FUSED
+    ac.FUSED = True
+    yield
+    ac.FUSED = old
+
+
+def _ops(layout):
+    return (tb.MatMul(layout, 64, 'sdd', trans_a=False, trans_b=True), tb.Softmax(layout, 64), tb.MatMul(layout, 64, 'dsd'))
+
+
+def _causal_window_layout(H, R, window=3, stride=4):
+    """causal: `window` blocks before the diagonal plus every stride-th block-column: rows of 1 .. window + R / stride blocks"""
+    lay = torch.zeros(H, R, R, dtype=torch.int64)
+    for h in range(H):
+        for r in range(R):
+            lay[h, r, max(0, r - window + 1):r + 1] = 1
+            lay[h, r, [c for c in range(0, r + 1) if c % stride == (h % stride)]] = 1
+    return lay
+
+
+def _run(ops, q, k, v, do, fused, **kw):
+    ac.FUSED = fused
+    qg, kg, vg = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+    before = ac.fused_calls
+    o = ac.attention_chain(ops[0], ops[1], ops[2], qg, kg, vg, **kw)
+    assert (ac.fused_calls > before) == fused
+    o.backward(do)
+    torch.cuda.synchronize()
+    return o.detach(), qg.grad, kg.grad, vg.grad
+
+
+# differences between the fused kernels and the three operators, relative to the largest value of the tensor: the
+# forward pass computes the same roundings (scores to the storage type, softmax in fp32) and differs by the order of
+# the sums; the backward pass replaces sum(p dp) by sum(do o), equal in exact arithmetic
+CHAIN_TOL = {torch.float16: (1.5e-3, 4e-3), torch.bfloat16: (1.2e-2, 3e-2)}
+
+
+@pytest.mark.parametrize('dtype,dh,masks', [
+    (torch.float16, 64, ()),
+    (torch.float16, 64, ('kpm_add',)),
+    (torch.float16, 64, ('kpm_mul', 'attn_mul')),
+    (torch.float16, 64, ('rpe', 'attn_add')),
+    (torch.bfloat16, 64, ('kpm_add', 'rpe')),
+    (torch.float16, 128, ('kpm_add',)),
+    (torch.bfloat16, 128, ('rpe', 'attn_mul', 'kpm_mul')),
+])
+def test_fused_chain_against_dense_oracle_and_three_operators(dtype, dh, masks):
+    torch.manual_seed(len(masks) * 7 + dh)
+    Z, H, R = 2, 3, 16
+    L = R * 64
+    layout = _causal_window_layout(H, R)
+    assert 4 < int(layout.sum(2).max()) <= 8
+    ops = _ops(layout)
+    q, k, v, do = [torch.randn(Z, H, L, dh, device=DEV).to(dtype) for _ in range(4)]
+    kw = dict(scale=dh ** -0.5)
+    okw = {}
+    if 'kpm_add' in masks:
+        m = torch.zeros(Z, L)
+        m[0, L - 100:] = float('-inf')
+        kw.update(key_padding_mask=m.to(DEV).to(dtype), key_padding_mask_mode='add')
+    if 'kpm_mul' in masks:
+        m = torch.ones(Z, L)
+        m[1, L - 77:] = 0
+        kw.update(key_padding_mask=m.to(DEV).to(dtype), key_padding_mask_mode='mul')
+    if 'attn_mul' in masks:
+        kw.update(attn_mask=torch.tril(torch.ones(L, L)).to(DEV).to(dtype), attn_mask_mode='mul')
+    if 'attn_add' in masks:
+        kw.update(attn_mask=(0.5 * torch.randn(L, L)).to(DEV).to(dtype), attn_mask_mode='add')
+    if 'rpe' in masks:
+        kw.update(rpe=(0.3 * torch.randn(H, L, L)).to(DEV).to(dtype))
+    okw = {n: kw[n] for n in ('rpe', 'key_padding_mask', 'attn_mask', 'key_padding_mask_mode') if n in kw}
+    okw['attn_mask_mode'] = kw.get('attn_mask_mode', 'add')
+    with guard_allocations('fused attention'):
+        got = _run(ops, q, k, v, do, True, **kw)
+    ref = D.attention(q, k, v, layout, 64, kw['scale'], do=do, **okw)
+    chain = _run(ops, q, k, v, do, False, **kw)
+    for name, g, r, c in zip(('o', 'dq', 'dk', 'dv'), got, ref, chain):
+        assert_close(g, r, dtype, 'fused ' + name)
+        tol = CHAIN_TOL[dtype][0 if name in ('o', 'dv') else 1] * float(c.float().abs().max())
+        assert float((g.float() - c.float()).abs().max()) <= tol, name
+
+
+def test_rows_of_zero_one_and_eight_blocks_and_rectangular_layout():
+    # keys longer than queries (C > R), an empty block-row (its rows of o and dq are zero), rows of 1 and of 8 blocks
+    torch.manual_seed(3)
+    Z, H, R, C, dh = 2, 2, 6, 10, 64
+    layout = torch.zeros(H, R, C, dtype=torch.int64)
+    layout[:, 0, 3] = 1
+    layout[:, 1, :8] = 1
+    layout[0, 3, [0, 9]] = 1
+    layout[1, 3, [2, 4, 5]] = 1
+    layout[:, 4, 1:9] = 1
+    layout[:, 5, 9] = 1                     # block-row 2 stays empty
+    ops = _ops(layout)
+    q, do = [torch.randn(Z, H, R * 64, dh, device=DEV).half() for _ in range(2)]
+    k, v = [torch.randn(Z, H, C * 64, dh, device=DEV).half() for _ in range(2)]
+    with guard_allocations('fused attention, ragged layout'):
+        got = _run(ops, q, k, v, do, True, scale=0.125)
+    chain = _run(ops, q, k, v, do, False, scale=0.125)
+    assert not bool(got[0][:, :, 128:192].any()) and not bool(got[1][:, :, 128:192].any())
+    for name, g, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
+        assert float((g.float() - c.float()).abs().max()) <= 4e-3 * float(c.float().abs().max()), name
+    live = torch.ones(R, dtype=torch.bool)
+    live[2] = False
+    rows = live.repeat_interleave(64)
+    ref = D.attention(q[:, :, rows], k, v, layout[:, live], 64, 0.125, do=do[:, :, rows], attn_mask_mode='add')
+    assert_close(got[0][:, :, rows], ref[0], torch.float16, 'o')
+    assert_close(got[1][:, :, rows], ref[1], torch.float16, 'dq')
+    assert_close(got[2], ref[2], torch.float16, 'dk')
+    assert_close(got[3], ref[3], torch.float16, 'dv')
+
+
+def test_strided_operands_and_gradient_subsets():
+    torch.manual_seed(5)
+    Z, H, R, dh = 2, 4, 8, 64
+    L = R * 64
+    layout = _causal_window_layout(H, R, window=2, stride=3)
+    ops = _ops(layout)
+    # [Z, L, H, dh] storage seen as [Z, H, L, dh]: unit stride along the head dimension, the rest strided
+    q, k, v, do = [torch.randn(Z, L, H, dh, device=DEV).half().permute(0, 2, 1, 3) for _ in range(4)]
+    got = _run(ops, q, k, v, do, True, scale=0.125)
+    chain = _run(ops, q.contiguous(), k.contiguous(), v.contiguous(), do.contiguous(), False, scale=0.125)
+    for name, g, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
+        assert g.shape == c.shape
+        assert float((g.float() - c.float()).abs().max()) <= 4e-3 * float(c.float().abs().max()), name
+    # only some inputs need a gradient
+    for need in ((True, False, False), (False, True, False), (False, False, True), (False, True, True)):
+        ts = [t.detach().clone().requires_grad_(n) for t, n in zip((q, k, v), need)]
+        o = ac.attention_chain(ops[0], ops[1], ops[2], ts[0], ts[1], ts[2], scale=0.125)
+        o.backward(do)
+        for t, n, c in zip(ts, need, chain[1:]):
+            assert (t.grad is not None) == n
+            if n:
+                assert float((t.grad.float() - c.float()).abs().max()) <= 4e-3 * float(c.float().abs().max())
+
+
+def test_backward_is_reproducible_at_full_occupancy():
+    """BigBird layout at 16384 positions: 6144 workgroups, four per compute unit.  The kernels' tile ring relies on every
+    LDS read of a stage having returned before the barrier that lets the stage be refilled; with that wait missing, one
+    block in about 150000 came out with another tile's values.  Identical inputs must give identical bits."""
+    torch.manual_seed(0)
+    layout = tb.bigbird_layout(12, 256, 3, 2, 3, seed=0, causal=True)
+    B, H, L, dh = 2, 12, 16384, 64
+    q, k, v, do = [torch.randn(B, H, L, dh, device=DEV, dtype=torch.float16) for _ in range(4)]
+    core = ac.AttentionCore(layout, 64)
+    first = None
+    for rep in range(6):
+        qg, kg = q.clone().requires_grad_(True), k.clone().requires_grad_(True)
+        o = core(qg, kg, v, scale=0.125)
+        o.backward(do)
+        torch.cuda.synchronize()
+        if first is None:
+            first = (o.detach().clone(), qg.grad.clone(), kg.grad.clone())
+        else:
+            assert torch.equal(o, first[0]) and torch.equal(qg.grad, first[1]) and torch.equal(kg.grad, first[2]), rep
+    # and right: one (batch, head) slice against the dense oracle
+    z, h = 1, 3
+    ref = D.attention(q[z:z + 1, h:h + 1], k[z:z + 1, h:h + 1], v[z:z + 1, h:h + 1], layout[h:h + 1], 64, 0.125,
+                      do=do[z:z + 1, h:h + 1], attn_mask_mode='add')
+    assert_close(first[0][z:z + 1, h:h + 1], ref[0], torch.float16, 'o')
+    assert_close(first[1][z:z + 1, h:h + 1], ref[1], torch.float16, 'dq')
+    assert_close(first[2][z:z + 1, h:h + 1], ref[2], torch.float16, 'dk')
+
+
+def test_modules_take_the_fused_kernels_and_agree_with_the_operators():
+    torch.manual_seed(6)
+    cfg = tb.SparsityConfig(mode='fixed', block=64, stride=256, attention='unidirectional')
+    mod = tb.SparseSelfAttention(cfg)
+    B, H, L, dh = 2, 4, 1024, 64
+    q, k, v, do = [torch.randn(B, H, L, dh, device=DEV).half() for _ in range(4)]
+    kpm = torch.zeros(B, L, device=DEV).half()
+    kpm[1, 900:] = float('-inf')
+    res = {}
+    for fused in (True, False):
+        ac.FUSED = fused
+        ts = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        n0 = ac.fused_calls
+        o = mod(ts[0], ts[1], ts[2], key_padding_mask=kpm)
+        assert (ac.fused_calls - n0) == int(fused)
+        o.backward(do)
+        res[fused] = [o.detach()] + [t.grad for t in ts]
+    for g, c in zip(res[True], res[False]):
+        assert float((g.float() - c.float()).abs().max()) <= 4e-3 * float(c.float().abs().max())
+    # nn.MultiheadAttention drop-in: block 64, head dimension 64
+    E, heads, Lm = 256, 4, 512
+    layout = torch.tril(torch.ones(heads, Lm // 64, Lm // 64)).long()
+    torch.manual_seed(0)
+    mha = tb.MultiheadAttention(E, heads, layout, 64).to(DEV).half()
+    x = torch.rand(Lm, 2, E, device=DEV).half()
+    outs = {}
+    for fused in (True, False):
+        ac.FUSED = fused
+        n0 = ac.fused_calls
+        xg = x.clone().requires_grad_(True)
+        y, _ = mha(xg, xg, xg, need_weights=False)
+        assert (ac.fused_calls - n0) == int(fused)
+        y.float().sum().backward()
+        outs[fused] = (y.detach(), xg.grad)
+    for g, c in zip(outs[True], outs[False]):
+        assert float((g.float() - c.float()).abs().max()) <= 6e-3 * float(c.float().abs().max()) + 1e-3
+
+
+def test_cases_left_to_the_three_operators():
+    torch.manual_seed(7)
+    Z, H, dh = 1, 2, 64
+    # a row of nine blocks: longer than the fused kernels hold in registers
+    layout = torch.zeros(H, 10, 10, dtype=torch.int64)
+    layout[:, :, 0] = 1
+    layout[:, 9, :9] = 1
+    ops = _ops(layout)
+    q, k, v = [torch.randn(Z, H, 640, dh, device=DEV).half() for _ in range(3)]
+    n0 = ac.fused_calls
+    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    assert ac.fused_calls == n0
+    assert_close(o, D.attention(q, k, v, layout, 64, 0.125, attn_mask_mode='add'), torch.float16, 'o')
+    # dropout, fp32, another block size, a head dimension the kernels do not have
+    lay = torch.tril(torch.ones(H, 4, 4)).long()
+    ops = _ops(lay)
+    q, k, v = [torch.randn(Z, H, 256, dh, device=DEV).half() for _ in range(3)]
+    for args, kw in (((q, k, v), dict(dropout_p=0.5)), ((q.float(), k.float(), v.float()), {}),
+                     ((q[..., :32].contiguous(), k[..., :32].contiguous(), v[..., :32].contiguous()), {})):
+        n0 = ac.fused_calls
+        ac.attention_chain(ops[0], ops[1], ops[2], *args, scale=0.125, **kw)
+        assert ac.fused_calls == n0
+    ops32 = (tb.MatMul(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32, 'sdd', trans_b=True),
+             tb.Softmax(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32),
+             tb.MatMul(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32, 'dsd'))
+    n0 = ac.fused_calls
+    ac.attention_chain(ops32[0], ops32[1], ops32[2], q, k, v, scale=0.125)
+    assert ac.fused_calls == n0
+    # operators built on different layouts are not a chain the fused kernels can stand for
+    other = lay.clone()
+    other[:, 3, 0] = 0
+    mixed = (tb.MatMul(lay, 64, 'sdd', trans_b=True), tb.Softmax(lay, 64), tb.MatMul(other, 64, 'dsd'))
+    assert ac._core_for(*mixed) is None
+    # the reference's dtype check on the masks (softmax.py:348-353) comes before any launch
+    with pytest.raises(ValueError):
+        ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, key_padding_mask=torch.zeros(Z, 256, device=DEV))
+
+
+def test_c_abi_argument_checks():
+    lib = _lib.load()
+    t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
+    p = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
+    lut, maxlut = tb.Softmax(torch.ones(1, 1, 1, dtype=torch.int64), 64).make_lut(torch.device(DEV))
+    null = ctypes.c_void_p(0)
+    st = (t.stride(0), t.stride(1), t.stride(2))
+
+    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64):
+        return lib.bsp_attention_fwd(dtype, _lib.ptr(q), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(t.clone()), 1, 1, 1, D,
+                                     st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut,
+                                     null, 0, 0, 0, null, 0, 0, null, 0, 0, _lib.stream_ptr(torch.device(DEV)))
+    assert fwd() == _lib.OK
+    assert fwd(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
+    assert fwd(block=32) == _lib.ERR_UNSUPPORTED
+    assert fwd(D=96) == _lib.ERR_UNSUPPORTED
+    assert fwd(maxlut=9) == _lib.ERR_ROW_TOO_LONG
+    assert fwd(ldq=60) != _lib.OK                       # a row stride that is not a multiple of 8 elements
+    assert fwd(q=None) != _lib.OK
+    torch.cuda.synchronize()

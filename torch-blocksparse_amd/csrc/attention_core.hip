@@ -1,0 +1,727 @@
+// The attention chain of one block-row in one kernel, block 64, fp16 / bf16, for gfx950.
+//
+// The reference's attention modules run three operators per call: scores = sdd(q, k^T), softmax in place, context =
+// dsd(p, v) (deepspeedsparseselfattention.py:152-157; attention.py:190-202), and autograd adds five more launches for
+// the backward pass.  Every one of them streams the [Z, nnz, 64, 64] sparse tensor through HBM: at head_dim 64 the
+// chain is bound by that traffic, not by arithmetic.  Here a workgroup owns one block-row of one (batch, head); each
+// of its four wavefronts keeps 16 rows of ALL nonzero blocks of that block-row in MFMA accumulators, so the scores
+// never leave the registers between the three steps:
+//
+//   forward  : s = q . k^T  ->  p = softmax(s * scale + rpe + key-padding mask + attention mask)  ->  o = p . v
+//              p is written once (the backward pass needs it), o once; the scores are never stored.
+//   backward : dp = do . v^T  ->  ds = p * (dp - sum(p * dp)) * scale  ->  dq = ds . k
+//              p is read once, ds written once (dk = ds^T . q and dv = p^T . do remain ordinary dsd products).
+//
+// Arithmetic mirrors the separate operators: the scores (and dp) are rounded to the storage type before the softmax
+// sees them, as they are when sdd stores them; the softmax is computed in fp32 (log2 domain) and rounded before the
+// second product consumes it.
+//
+// Register layout.  The first product is computed transposed, s^T = k_tile . q^T, with the MFMA 16x16x32: its A operand
+// (rows of the result) is a k tile read from LDS, its B operand the wavefront's 16 q rows, loaded once from global
+// memory straight into operand registers.  A lane then holds, for q row lane % 16, four result rows 4 * (lane / 16) + e
+// of each 16-row sub-tile.  The k rows are dealt to the sub-tiles so that these are keys 32s + 8 * (lane / 16) + 0..7
+// of the block (s = 0, 1): eight consecutive keys, which is at once a 16-byte piece of a row of p (stored as it is) and
+// the B-operand fragment of the second product o^T = v^T . p^T (no shuffle, no LDS round trip).  v^T comes from the v
+// tile in LDS through the transposing LDS read.
+#include "matmul_generic.h"
+#include "softmax_common.h"
+#include <type_traits>
+
+namespace bsp {
+namespace {
+
+// LDS stages of the tile ring: loads run (stages - 1) tiles ahead of their use; three at head dimension 128, where a
+// tile is 16 KiB and a launch may ask for 64 KiB of dynamic LDS without further ado
+template <int D> constexpr int ring_stages() { return D == 64 ? 4 : 3; }
+
+#define BSP_GLOBAL_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
+#define BSP_LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
+// Wait until at most n vector-memory operations of this wavefront are outstanding AND all of its LDS reads have returned.
+// The second half matters before the barrier of a ring step: the barrier lets other wavefronts start the direct-to-LDS
+// load that overwrites the stage this wavefront read last, and a read that is still in flight then can return the new
+// tile's bytes (the compiler is free to leave the wait for a read's data behind the barrier, next to its first use;
+// seen as one wrong block in 150000 at full occupancy).
+#define BSP_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0x0 << 8))
+
+// Tiles of 64 rows x D elements travel from global memory straight into LDS (global_load_lds_dwordx4: 16 bytes per
+// lane, 1 KiB of consecutive LDS per wavefront-level load), so their rows lie unpadded, 2 D bytes apart, and the bank
+// conflicts of the reads are avoided by an XOR swizzle of the 16-byte chunks inside a row, applied by choosing which
+// global chunk each lane fetches.  Two swizzles, one per way a tile is read:
+//   tiles of the first product (16-byte reads, sixteen lanes per clock, the lanes' rows differ in bits 0, 1, 3, 4):
+//     D = 64 (rows r, r + 2 start in the same bank): chunk c of row r at slot c ^ (bit 1 | bit 3 << 1 | bit 4 << 2);
+//     D = 128 (every row starts in bank 0): slot c ^ (bits 0, 1 | bits 3, 4 << 2);
+//   tiles of the second product (transposing reads: a 16-lane group takes 32 bytes, a pair of chunks, from each of four
+//     consecutive rows; the group served with it reads rows 8 further on): pair p of row r at pair slot
+//     p ^ (r & 3) ^ (bit 3) for D = 64, p ^ 2 (r & 3) ^ (bit 3) for D = 128.
+template <int D> __device__ __forceinline__ int swz_first(int r) {
+  return D == 64 ? (((r >> 1) & 1) | (((r >> 3) & 3) << 1)) : ((r & 3) | (((r >> 3) & 3) << 2));
+}
+template <int D> __device__ __forceinline__ int swz_second(int r) {
+  return D == 64 ? ((r & 3) ^ ((r >> 3) & 1)) : (((r & 3) << 1) ^ ((r >> 3) & 1));
+}
+// byte offsets inside a tile
+template <int D> __device__ __forceinline__ int first_offset(int r, int chunk) { return r * (2 * D) + ((chunk ^ swz_first<D>(r)) << 4); }
+template <int D> __device__ __forceinline__ int second_offset(int r, int col) {   // col in elements, a multiple of 4
+  const int chunk = col >> 3, pair = (chunk >> 1) ^ swz_second<D>(r);
+  return r * (2 * D) + (((pair << 1) | (chunk & 1)) << 4) + ((col & 7) << 1);
+}
+
+struct AttnArgs {
+  const void *x, *y1, *y2;   // forward: q, k, v; backward: do, v, k
+  const void *p_in;          // backward: the saved softmax
+  void *p_out, *o;           // forward: p, o; backward: ds, dq
+  const void *o_in;          // backward: the forward result o
+  int64_t oin_sz, oin_sh, oin_ld;
+  int64_t x_sz, x_sh, x_ld, y1_sz, y1_sh, y1_ld, y2_sz, y2_sh, y2_ld, o_sz, o_sh, o_ld, pin_sz, pout_sz;
+  float scale;
+  const int32_t *lut;        // the softmax table (softmax.py:201-221): per block-row (size, offset), per block (id, col, row, head)
+  const void *rpe; int64_t rpe_sz, rpe_sh, rpe_sr;
+  const void *kpm; int64_t kpm_sz; int kpm_mul;
+  const void *attn; int64_t attn_sr; int attn_mul;
+  int Z, H, R;
+};
+
+// Four operand fragments of the second product through the transposing LDS read: for each of four LDS addresses, rows
+// 0..3 (reduction indices 0..3 of the lane's column) at the address and rows 4..7 at the address + HI bytes.  Written as
+// one assembly block with its own wait: the compiler would otherwise, before every such read, wait for all direct-to-LDS
+// loads in flight (it cannot tell that they fill other stages of the ring), which would undo the prefetch.
+template <typename T, int HI>
+__device__ __forceinline__ void tr_frags4(typename Mma16<T>::frag_t (&f)[4], uint32_t a0, uint32_t a1, uint32_t a2, uint32_t a3) {
+  s16x4 lo0, hi0, lo1, hi1, lo2, hi2, lo3, hi3;
+  asm volatile(
+      "ds_read_b64_tr_b16 %0, %8\n\t"
+      "ds_read_b64_tr_b16 %1, %8 offset:%12\n\t"
+      "ds_read_b64_tr_b16 %2, %9\n\t"
+      "ds_read_b64_tr_b16 %3, %9 offset:%12\n\t"
+      "ds_read_b64_tr_b16 %4, %10\n\t"
+      "ds_read_b64_tr_b16 %5, %10 offset:%12\n\t"
+      "ds_read_b64_tr_b16 %6, %11\n\t"
+      "ds_read_b64_tr_b16 %7, %11 offset:%12\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(lo0), "=&v"(hi0), "=&v"(lo1), "=&v"(hi1), "=&v"(lo2), "=&v"(hi2), "=&v"(lo3), "=&v"(hi3)
+      : "v"(a0), "v"(a1), "v"(a2), "v"(a3), "n"(HI));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef typename Mma16<T>::frag_t frag_t;
+  f[0] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7));
+  f[1] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7));
+  f[2] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo2, hi2, 0, 1, 2, 3, 4, 5, 6, 7));
+  f[3] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo3, hi3, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// acc[j][e] = out[row lane % 16][column 16j + 4 * (lane / 16) + e] of a 16 x D slice -> the wavefront's piece of LDS ->
+// stores of whole rows (16 bytes per lane, a row = D / 8 consecutive lanes)
+template <typename T, int D> __device__ __forceinline__ void store_rows(T *cs, T *dst, int64_t ld, const f32x4 (&acc)[D / 16], int lane) {
+  constexpr int LDK = D + 8, CPR = D / 8;
+#pragma unroll
+  for (int j = 0; j < D / 16; j++) {
+    union { u32x2 raw; T e[4]; } pk;
+#pragma unroll
+    for (int e = 0; e < 4; e++) pk.e[e] = from_float<T>(acc[j][e]);
+    *reinterpret_cast<u32x2 *>(cs + (lane & 15) * LDK + 16 * j + 4 * (lane >> 4)) = pk.raw;
+  }
+  __builtin_amdgcn_wave_barrier();   // LDS operations of one wavefront complete in order; this only pins the code order
+#pragma unroll
+  for (int i = 0; i < CPR / 4; i++) {
+    const int c = lane + 64 * i;
+    const u32x4 v = *reinterpret_cast<const u32x4 *>(cs + (c / CPR) * LDK + (c % CPR) * 8);
+    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst + (int64_t)(c / CPR) * ld + (c % CPR) * 8));
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// The wavefront's 16 rows of a 64 x 64 block of the sparse tensor (2 KiB of consecutive addresses), a lane holding
+// columns 8 * (lane / 16) .. + 7 (c0) and 32 + 8 * (lane / 16) .. (c1) of row lane % 16: through the wavefront's piece of
+// LDS (rows of 72 elements), then two stores of 1 KiB of consecutive addresses.  (Stored straight from the registers,
+// every store instruction writes sixteen separate 64-byte pieces: measured, the forward kernel then takes 170 us
+// instead of 107 without the stores.)
+template <typename T> __device__ __forceinline__ void store_block_rows(T *cs, T *dst, const u32x4 &c0, const u32x4 &c1, int lane) {
+  T *w = cs + (lane & 15) * 72 + 8 * (lane >> 4);
+  *reinterpret_cast<u32x4 *>(w) = c0;
+  *reinterpret_cast<u32x4 *>(w + 32) = c1;
+  __builtin_amdgcn_wave_barrier();   // LDS operations of one wavefront complete in order; this only pins the code order
+#pragma unroll
+  for (int i = 0; i < 2; i++) {
+    const int c = lane + 64 * i;
+    *reinterpret_cast<u32x4 *>(dst + c * 8) = *reinterpret_cast<const u32x4 *>(cs + (c >> 3) * 72 + (c & 7) * 8);
+  }
+  __builtin_amdgcn_wave_barrier();
+}
+
+// D = head dimension (64 or 128); NB = most blocks a block-row may hold (the host picks the bucket from the table's
+// longest row); EXTRA = a relative position embedding or an attention mask is present.
+template <typename T, int D, int NB, bool EXTRA>
+__global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  typedef Pack<T, 8> P8;
+  constexpr int NK = D / 32;            // MFMA steps along the head dimension in the first product
+  constexpr int ND = D / 16;            // 16-column sub-tiles of the result of the second product
+  constexpr int LDK = D + 8;            // row of the staging slice of the result (16 bytes of padding)
+  constexpr int TB = 64 * D * 2;        // bytes of a tile
+  constexpr int LW = TB / 1024 / 4;     // wavefront-level loads per wavefront and tile
+  constexpr int CPR = D / 8;            // 16-byte chunks per tile row
+  constexpr int kStages = ring_stages<D>();
+  // dynamic LDS: the tile ring (at the end it stages the results: per wavefront a slice of the dense and one of the
+  // sparse result), then the key-padding terms
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char *ring = smem;
+  T *stage_out = reinterpret_cast<T *>(smem);
+  float *kpm_s = reinterpret_cast<float *>(smem + kStages * TB);
+  static_assert(4 * 16 * (LDK + 72) * 2 <= kStages * TB, "the staged results fit into the ring");
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n_wg = (int64_t)a.Z * a.H * a.R;
+  const int64_t wg = xcd_remap(blockIdx.x, n_wg);
+  // block-rows from the last one down (the longest rows of a causal layout first), all rows of a (batch, head) in a
+  // row: its k and v tiles stay in the L2 of the XCD that works on it
+  const int br = a.R - 1 - (int)(wg % a.R);
+  const int zh = (int)(wg / a.R);
+  const int h = zh % a.H, z = zh / a.H;
+  const table_ptr lut = as_table(a.lut);
+  const int size = lut[2 * (h * a.R + br) + 0];   // header (size, offset), softmax.py:30-32
+  const int offset = lut[2 * (h * a.R + br) + 1];
+  const int qrow = lane & 15, q = lane >> 4;
+  const int64_t row = (int64_t)br * 64 + wave * 16 + qrow;   // the lane's row of the dense matrices (first product)
+  T *cs = stage_out + wave * 16 * LDK;
+  T *stage_p = stage_out + 4 * 16 * LDK + wave * (16 * 72);
+  T *po = reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + ((int64_t)br * 64 + wave * 16) * a.o_ld;
+  f32x4 o[ND];
+#pragma unroll
+  for (int j = 0; j < ND; j++) o[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (size <= 0) {   // an empty block-row: its rows of the dense result are zero, as the dsd operator leaves them
+    store_rows<T, D>(cs, po, a.o_ld, o, lane);
+    return;
+  }
+  const table_ptr core = lut + offset;
+  int32_t bid[NB], bcol[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) {
+    const int bb = b < size ? b : 0;    // blocks past the end repeat the first one (valid to read, never used)
+    bid[b] = core[4 * bb + 0];
+    bcol[b] = core[4 * bb + 1];
+  }
+  const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
+  frag_t xq[NK];
+#pragma unroll
+  for (int s2 = 0; s2 < NK; s2++) xq[s2] = *reinterpret_cast<const frag_t *>(px + 32 * s2);
+  const T *py1 = reinterpret_cast<const T *>(a.y1) + z * a.y1_sz + h * a.y1_sh;
+  const T *py2 = reinterpret_cast<const T *>(a.y2) + z * a.y2_sz + h * a.y2_sh;
+  // The unified tile sequence of the workgroup: y1 tiles of blocks 0 .. size - 1, then y2 tiles of the same blocks.
+  // Tile n lives in ring stage n % kStages.  Per-lane part of the addresses: load i of this wavefront covers rows
+  // (wave * LW + i) * (64 / CPR) .. of the tile, lane l its row l / CPR and the chunk that belongs into slot l % CPR.
+  int64_t off1[LW], off2[LW];
+#pragma unroll
+  for (int i = 0; i < LW; i++) {
+    const int r = (wave * LW + i) * (64 / CPR) + lane / CPR, slot = lane % CPR;
+    off1[i] = (int64_t)r * a.y1_ld + ((slot ^ swz_first<D>(r)) << 3);
+    off2[i] = (int64_t)r * a.y2_ld + (((((slot >> 1) ^ swz_second<D>(r)) << 1) | (slot & 1)) << 3);
+  }
+  const int total = 2 * size;
+  int next_col;
+  // the block-column of tile n, from the table (a scalar load; clamped past the end)
+  auto tile_col = [&](int n) {
+    const int m = n < size ? n : n - size;
+    return core[4 * (m < size ? m : size - 1) + 1];
+  };
+  auto issue = [&](int n, int col) {
+    unsigned char *st = ring + (n % kStages) * TB + wave * LW * 1024;
+    if (n < size) {
+      const T *base = py1 + (int64_t)col * 64 * a.y1_ld;
+#pragma unroll
+      for (int i = 0; i < LW; i++) __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + i * 1024), 16, 0, 0);
+    } else {
+      const T *base = py2 + (int64_t)col * 64 * a.y2_ld;
+#pragma unroll
+      for (int i = 0; i < LW; i++) __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + i * 1024), 16, 0, 0);
+    }
+  };
+  // Before tile n is read: this wavefront's loads of it have landed (all but those of the tiles issued after it,
+  // kStages - 2 of them or fewer near the end), then the barrier (everybody's have, and everybody is done reading tile n - 1), then the
+  // load of tile n + kStages - 1 into the stage that tile n - 1 used.
+  auto step = [&](int n) {
+    const int rem = total - 1 - n;
+    if (rem >= kStages - 2) BSP_WAIT_VM(LW * (kStages - 2));
+    else if (kStages > 3 && rem == 1) BSP_WAIT_VM(LW);
+    else BSP_WAIT_VM(0);
+    asm volatile("" ::: "memory");                     // (the compiler must not move LDS accesses across the barrier)
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (n + kStages - 1 < total) issue(n + kStages - 1, next_col);
+    next_col = tile_col(n + kStages);                  // the table runs one step ahead of the load that uses it
+  };
+  // The key-padding term of every column of the block-row (softmax.py:104-106, 122-124), fetched once per workgroup
+  // and kept in LDS as the value that is added to the logits; the first barrier below orders it before its readers.
+  P8 kp;
+  const bool kpm_lane = a.kpm && tid < NB * 8;
+  {
+    if (kpm_lane) {
+      const int b = tid >> 3;
+      int col = bcol[0];
+#pragma unroll
+      for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
+      kp.load(reinterpret_cast<const T *>(a.kpm) + z * a.kpm_sz + (int64_t)col * 64 + (tid & 7) * 8);
+    }
+  }
+  // the first two tiles always exist (a row has at least one block); in a straight line, so that the wait for the
+  // key-padding values counts exactly the loads issued after them
+  issue(0, tile_col(0));
+  issue(1, tile_col(1));
+  {
+    if (kpm_lane) {
+      const float unit = logit_unit<T>();
+#pragma unroll
+      for (int e4 = 0; e4 < 8; e4 += 4) {
+        f32x4 add;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const float m = to_float(kp.e[e4 + e]);
+          add[e] = a.kpm_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+        }
+        *reinterpret_cast<f32x4 *>(&kpm_s[tid * 8 + e4]) = add;
+      }
+    }
+  }
+#pragma unroll
+  for (int n = 2; n < kStages - 1; n++)
+    if (n < total) issue(n, tile_col(n));
+  next_col = tile_col(kStages - 1);
+
+  // ---- first product: acc[b][jt][e] = (x . y1_b^T)[row lane % 16][key 32 * (jt / 2) + 8 * (lane / 16) + 4 * (jt % 2) + e]
+  f32x4 acc[NB][4];
+  // the k row that supplies result row m of sub-tile jt (see the file comment)
+  const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size) {
+      step(b);
+      const unsigned char *tile = ring + (b % kStages) * TB;
+      frag_t kf[4][NK];
+#pragma unroll
+      for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+        for (int s2 = 0; s2 < NK; s2++)
+          kf[jt][s2] = *reinterpret_cast<const frag_t *>(tile + first_offset<D>(32 * (jt >> 1) + 4 * (jt & 1) + krow0, 4 * s2 + q));
+#pragma unroll
+      for (int jt = 0; jt < 4; jt++) {
+        acc[b][jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < NK; s2++) acc[b][jt] = M::run(kf[jt][s2], xq[s2], acc[b][jt]);
+      }
+    }
+
+  // ---- between the products: the softmax on the wavefront's 16 rows.  A lane's
+  // values of block b: two chunks (s = 0, 1) of eight consecutive columns 32s + 8 * (lane / 16) + i, i = 4t + e in
+  // acc[b][2s + t][e].  The reductions over a row run over the lane's values, then over the four lanes that share it.
+  frag_t pf[NB][2];
+  T *pout = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz + wave * 1024;   // the wavefront's 16 rows of block 0
+  {
+    const float unit = logit_unit<T>(), sc = a.scale * unit;
+    const bool has_kpm = a.kpm != nullptr;
+    float mx = -INFINITY;
+    constexpr int GS = EXTRA ? (NB < 4 ? NB : 4) : NB;   // blocks whose mask values are in flight together
+#pragma unroll
+    for (int g = 0; g < NB; g += GS) {
+      P8 pr[EXTRA ? GS : 1][2], pa[EXTRA ? GS : 1][2];
+      if constexpr (EXTRA) {
+#pragma unroll
+        for (int b = g; b < g + GS; b++)
+          if (b < size) {
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+              const int64_t gcol = (int64_t)bcol[b] * 64 + 32 * s + 8 * q;
+              if (a.rpe)                                                // address: softmax.py:50-55
+                pr[b - g][s].load(reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol);
+              if (a.attn) pa[b - g][s].load(reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol);   // :67-70
+            }
+          }
+      }
+#pragma unroll
+      for (int b = g; b < g + GS; b++)
+        if (b < size) {
+#pragma unroll
+          for (int s = 0; s < 2; s++) {
+            float add[8];
+            if (has_kpm) {
+#pragma unroll
+              for (int e4 = 0; e4 < 8; e4 += 4)
+                *reinterpret_cast<f32x4 *>(&add[e4]) = *reinterpret_cast<const f32x4 *>(&kpm_s[b * 64 + 32 * s + 8 * q + e4]);
+            } else {
+#pragma unroll
+              for (int i = 0; i < 8; i++) add[i] = 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+              float fx = fmaf(to_float(from_float<T>(acc[b][2 * s + (i >> 2)][i & 3])), sc, add[i]);   // softmax.py:112-116, 122-124
+              if constexpr (EXTRA) {
+                if (a.rpe) fx = fmaf(to_float(pr[b - g][s].e[i]), unit, fx);   // :118-120
+                if (a.attn) {                                                  // :126-128, 'mul' mode :108-110
+                  const float m = to_float(pa[b - g][s].e[i]);
+                  fx += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+                }
+              }
+              acc[b][2 * s + (i >> 2)][i & 3] = fx;
+              mx = fmaxf(mx, fx);
+            }
+          }
+        }
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16));                                  // :130
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    float sum = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+          for (int e = 0; e < 4; e++) { acc[b][jt][e] = exp_sub<T>(acc[b][jt][e], mx); sum += acc[b][jt][e]; }   // :131-132
+      }
+    sum += __shfl_xor(sum, 16);
+    sum += __shfl_xor(sum, 32);
+    const float inv = 1.f / sum;
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+      if (b < size) {
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          P8 y;
+#pragma unroll
+          for (int i = 0; i < 8; i++) y.e[i] = from_float<T>(acc[b][2 * s + (i >> 2)][i & 3] * inv);   // :137
+          pf[b][s] = __builtin_bit_cast(frag_t, y.raw);
+        }
+      }
+  }
+
+  // ---- second product: o^T[d][row] += y2_b^T[d][key] . pf_b[key][row]; the y2 tiles continue the ring
+  // a lane's part of the LDS addresses of its transposing reads: rows 8 * (lane / 16) + (lane % 16) / 4 (+ 4, + 32 as
+  // immediate offsets: neither changes the swizzle), columns 16j + 4 * (lane % 4)
+  const int tr_row = q * 8 + (qrow >> 2), tr_col = (qrow & 3) * 4;
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)BSP_LDS_PTR(ring);
+  uint32_t tr_off[ND];
+#pragma unroll
+  for (int j = 0; j < ND; j++) tr_off[j] = second_offset<D>(tr_row, 16 * j + tr_col);
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size) {
+      step(size + b);
+      const uint32_t tile_lds = ring_lds + ((size + b) % kStages) * TB;
+#pragma unroll
+      for (int s = 0; s < 2; s++)
+#pragma unroll
+        for (int j4 = 0; j4 < ND; j4 += 4) {
+          frag_t vf[4];
+          const uint32_t t0 = tile_lds + s * (32 * 2 * D);
+          tr_frags4<T, 4 * 2 * D>(vf, t0 + tr_off[j4], t0 + tr_off[j4 + 1], t0 + tr_off[j4 + 2], t0 + tr_off[j4 + 3]);
+#pragma unroll
+          for (int j = 0; j < 4; j++) o[j4 + j] = M::run(vf[j], pf[b][s], o[j4 + j]);
+        }
+    }
+  // The sparse result leaves only now, although it has been ready since the softmax: on this architecture loads and
+  // stores share one counter of outstanding operations, so stores issued before the second product would have to be
+  // acknowledged by memory before the wait for its next tile could end (measured: the stores then cost their full
+  // 50 us on top of the rest instead of overlapping with other workgroups).  The values are the operand registers pf.
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();                        // the ring is free: everybody is done reading the last tile
+  asm volatile("" ::: "memory");
+  store_rows<T, D>(cs, po, a.o_ld, o, lane);
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size)
+      store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+}
+
+// wait until at most c (0, 2, 4, 6 or 8) vector-memory operations are outstanding; the instruction takes an immediate
+__device__ __forceinline__ void wait_vm(int c) {
+  if (c >= 8) BSP_WAIT_VM(8);
+  else if (c >= 6) BSP_WAIT_VM(6);
+  else if (c >= 4) BSP_WAIT_VM(4);
+  else if (c >= 2) BSP_WAIT_VM(2);
+  else BSP_WAIT_VM(0);
+}
+
+// The backward chain.  x = do, y1 = v, y2 = k.  Unlike the forward chain it needs no second look at a row before its
+// values can be finished: the sum over the row in the softmax gradient, sum_j p_j dp_j, equals sum_d do_d o_d (o = p . v,
+// dp = do . v^T), which the wavefront computes up front from its 16 rows of do and of the forward result.  So block
+// after block goes through dp = do . v_b^T -> ds_b = p_b * (dp - delta) * scale at once: the tile sequence is
+// v_0, p_0, v_1, p_1, ... (the block of p is one more 8 KiB tile of the ring: no register-staged loads inside the
+// loop, whose waits the compiler would place after all direct-to-LDS loads in flight), then k_0, k_1, ... for
+// dq = ds . k.  Only the packed ds (the operand of the second product) stays in registers.
+template <typename T, int D, int NB>
+__global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
+  typedef Mma16<T> M;
+  typedef typename M::frag_t frag_t;
+  typedef Pack<T, 8> P8;
+  constexpr int NK = D / 32, ND = D / 16, LDK = D + 8;
+  constexpr int TB = 64 * D * 2;        // bytes of a ring stage (a v or k tile; a block of p fills the first 8 KiB)
+  constexpr int LW = TB / 1024 / 4;     // wavefront-level loads per wavefront and v / k tile
+  constexpr int LWP = 2;                // ... and block of p
+  constexpr int CPR = D / 8;
+  constexpr int kStages = ring_stages<D>();
+  extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
+  unsigned char *ring = smem;
+  T *stage_out = reinterpret_cast<T *>(smem);
+  static_assert(4 * 16 * (LDK + 72) * 2 <= kStages * TB, "the staged results fit into the ring");
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t n_wg = (int64_t)a.Z * a.H * a.R;
+  const int64_t wg = xcd_remap(blockIdx.x, n_wg);
+  const int br = a.R - 1 - (int)(wg % a.R);          // as in the forward kernel
+  const int zh = (int)(wg / a.R);
+  const int h = zh % a.H, z = zh / a.H;
+  const table_ptr lut = as_table(a.lut);
+  const int size = lut[2 * (h * a.R + br) + 0];
+  const int offset = lut[2 * (h * a.R + br) + 1];
+  const int qrow = lane & 15, q = lane >> 4;
+  const int64_t row = (int64_t)br * 64 + wave * 16 + qrow;
+  T *cs = stage_out + wave * 16 * LDK;
+  T *stage_p = stage_out + 4 * 16 * LDK + wave * (16 * 72);
+  T *po = reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + ((int64_t)br * 64 + wave * 16) * a.o_ld;
+  f32x4 o[ND];
+#pragma unroll
+  for (int j = 0; j < ND; j++) o[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  if (size <= 0) {   // an empty block-row: zero rows of dq
+    store_rows<T, D>(cs, po, a.o_ld, o, lane);
+    return;
+  }
+  const table_ptr core = lut + offset;
+  int32_t bid[NB];
+#pragma unroll
+  for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
+  const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
+  const T *pof = reinterpret_cast<const T *>(a.o_in) + z * a.oin_sz + h * a.oin_sh + row * a.oin_ld + 8 * q;
+  frag_t xq[NK], oq[NK];
+#pragma unroll
+  for (int s2 = 0; s2 < NK; s2++) {
+    xq[s2] = *reinterpret_cast<const frag_t *>(px + 32 * s2);
+    oq[s2] = *reinterpret_cast<const frag_t *>(pof + 32 * s2);
+  }
+  const T *py1 = reinterpret_cast<const T *>(a.y1) + z * a.y1_sz + h * a.y1_sh;
+  const T *py2 = reinterpret_cast<const T *>(a.y2) + z * a.y2_sz + h * a.y2_sh;
+  const T *pin = reinterpret_cast<const T *>(a.p_in) + z * a.pin_sz;
+  // Tile n < 2 size: block n / 2, its v tile (n even) or its block of p (n odd); then the k tiles.  Stage n % kStages.
+  int64_t off1[LW], off2[LW];
+  int offp[LWP];
+#pragma unroll
+  for (int i = 0; i < LW; i++) {
+    const int r = (wave * LW + i) * (64 / CPR) + lane / CPR, slot = lane % CPR;
+    off1[i] = (int64_t)r * a.y1_ld + ((slot ^ swz_first<D>(r)) << 3);
+    off2[i] = (int64_t)r * a.y2_ld + (((((slot >> 1) ^ swz_second<D>(r)) << 1) | (slot & 1)) << 3);
+  }
+  // a block of p: rows of 128 bytes; a lane reads 16 bytes of row 16 * wave + lane % 16, sixteen consecutive rows per
+  // clock: chunk c of row r at slot c ^ ((r >> 1) & 7)
+#pragma unroll
+  for (int i = 0; i < LWP; i++) {
+    const int r = (wave * LWP + i) * 8 + (lane >> 3), slot = lane & 7;
+    offp[i] = r * 64 + ((slot ^ ((r >> 1) & 7)) << 3);
+  }
+  const int total = 3 * size;
+  auto loads_of = [&](int n) { return n >= total ? 0 : (n < 2 * size && (n & 1)) ? LWP : LW; };
+  // block-column (v and k tiles) or block id (p) of tile n, from the table (a scalar load; clamped past the end)
+  auto tile_key = [&](int n) {
+    const int m = n < 2 * size ? (n >> 1) : n - 2 * size;
+    return core[4 * (m < size ? m : size - 1) + ((n < 2 * size && (n & 1)) ? 0 : 1)];
+  };
+  int next_key;
+  auto issue = [&](int n, int key) {
+    unsigned char *st = ring + (n % kStages) * TB;
+    if (n < 2 * size && (n & 1)) {
+      const T *base = pin + (int64_t)key * 4096;
+#pragma unroll
+      for (int i = 0; i < LWP; i++)
+        __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+    } else if (n < 2 * size) {
+      const T *base = py1 + (int64_t)key * 64 * a.y1_ld;
+#pragma unroll
+      for (int i = 0; i < LW; i++)
+        __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
+    } else {
+      const T *base = py2 + (int64_t)key * 64 * a.y2_ld;
+#pragma unroll
+      for (int i = 0; i < LW; i++)
+        __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
+    }
+  };
+  // as in the forward kernel; the tiles issued after tile n differ in their number of loads
+  auto step = [&](int n) {
+    wait_vm(loads_of(n + 1) + (kStages > 3 ? loads_of(n + 2) : 0));
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (n + kStages - 1 < total) issue(n + kStages - 1, next_key);
+    next_key = tile_key(n + kStages);
+  };
+#pragma unroll
+  for (int n = 0; n < kStages - 1; n++) issue(n, tile_key(n));   // (a row has at least one block: three tiles)
+  next_key = tile_key(kStages - 1);
+  // delta = sum_d do[row][d] * o[row][d]: sixteen products per lane, then over the four lanes of the row
+  float delta = 0.f;
+#pragma unroll
+  for (int s2 = 0; s2 < NK; s2++)
+#pragma unroll
+    for (int i = 0; i < 8; i++) delta = fmaf(to_float(xq[s2][i]), to_float(oq[s2][i]), delta);
+  delta += __shfl_xor(delta, 16);
+  delta += __shfl_xor(delta, 32);
+
+  frag_t pf[NB][2];
+  const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
+  const int prow = wave * 16 + qrow, pswz = (prow >> 1) & 7;
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size) {
+      step(2 * b);
+      const unsigned char *tile = ring + ((2 * b) % kStages) * TB;
+      frag_t kf[4][NK];
+#pragma unroll
+      for (int jt = 0; jt < 4; jt++)
+#pragma unroll
+        for (int s2 = 0; s2 < NK; s2++)
+          kf[jt][s2] = *reinterpret_cast<const frag_t *>(tile + first_offset<D>(32 * (jt >> 1) + 4 * (jt & 1) + krow0, 4 * s2 + q));
+      f32x4 acc[4];
+#pragma unroll
+      for (int jt = 0; jt < 4; jt++) {
+        acc[jt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s2 = 0; s2 < NK; s2++) acc[jt] = M::run(kf[jt][s2], xq[s2], acc[jt]);
+      }
+      step(2 * b + 1);
+      const unsigned char *pt = ring + ((2 * b + 1) % kStages) * TB + prow * 128;
+#pragma unroll
+      for (int s = 0; s < 2; s++) {
+        P8 y, d;
+        y.raw = *reinterpret_cast<const u32x4 *>(pt + (((q + 4 * s) ^ pswz) << 4));
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+          const float dp = to_float(from_float<T>(acc[2 * s + (i >> 2)][i & 3]));   // dp as the sdd operator would have stored it
+          d.e[i] = from_float<T>(to_float(y.e[i]) * (dp - delta) * a.scale);          // softmax.py:189
+        }
+        pf[b][s] = __builtin_bit_cast(frag_t, d.raw);
+      }
+    }
+
+  // ---- second product: dq^T[d][row] += k_b^T[d][key] . ds_b[key][row]
+  const int tr_row = q * 8 + (qrow >> 2), tr_col = (qrow & 3) * 4;
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)BSP_LDS_PTR(ring);
+  uint32_t tr_off[ND];
+#pragma unroll
+  for (int j = 0; j < ND; j++) tr_off[j] = second_offset<D>(tr_row, 16 * j + tr_col);
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size) {
+      step(2 * size + b);
+      const uint32_t tile_lds = ring_lds + ((2 * size + b) % kStages) * TB;
+#pragma unroll
+      for (int s = 0; s < 2; s++)
+#pragma unroll
+        for (int j4 = 0; j4 < ND; j4 += 4) {
+          frag_t vf[4];
+          const uint32_t t0 = tile_lds + s * (32 * 2 * D);
+          tr_frags4<T, 4 * 2 * D>(vf, t0 + tr_off[j4], t0 + tr_off[j4 + 1], t0 + tr_off[j4 + 2], t0 + tr_off[j4 + 3]);
+#pragma unroll
+          for (int j = 0; j < 4; j++) o[j4 + j] = M::run(vf[j], pf[b][s], o[j4 + j]);
+        }
+    }
+  // ds leaves at the end, for the reason given in the forward kernel
+  T *pout = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz + wave * 1024;
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  store_rows<T, D>(cs, po, a.o_ld, o, lane);
+#pragma unroll
+  for (int b = 0; b < NB; b++)
+    if (b < size)
+      store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+}
+
+
+template <int D, int NB> constexpr int lds_bytes(bool bwd) { return ring_stages<D>() * 64 * D * 2 + (bwd ? 0 : NB * 64 * 4); }
+
+template <typename T, int D, int NB> void launch_nb(const AttnArgs &a, bool bwd, hipStream_t st) {
+  const dim3 grid((unsigned)((int64_t)a.Z * a.H * a.R)), wg(256);
+  constexpr int LDS = lds_bytes<D, NB>(false), LDS_BWD = lds_bytes<D, NB>(true);
+  static_assert(LDS <= 64 * 1024, "within what a launch may ask for without raising the kernel's limit");
+  if (bwd) hipLaunchKernelGGL((k_attn64_bwd<T, D, NB>), grid, wg, LDS_BWD, st, a);
+  else if (a.rpe || a.attn) hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, true>), grid, wg, LDS, st, a);
+  else hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, false>), grid, wg, LDS, st, a);
+}
+
+template <typename T, int D> int launch_d(const AttnArgs &a, int maxlut, bool bwd, hipStream_t st) {
+  if (maxlut <= 4) launch_nb<T, D, 4>(a, bwd, st);
+  else if (maxlut <= 8) launch_nb<T, D, 8>(a, bwd, st);
+  else return BSP_ERR_ROW_TOO_LONG;
+  return BSP_OK;
+}
+
+template <typename T> int launch_t(const AttnArgs &a, int D, int maxlut, bool bwd, hipStream_t st) {
+  if (D == 64) return launch_d<T, 64>(a, maxlut, bwd, st);
+  if (D == 128) return launch_d<T, 128>(a, maxlut, bwd, st);
+  return BSP_ERR_UNSUPPORTED;
+}
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *stream) {
+  if (!a.x || !a.y1 || !a.y2 || !a.p_out || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
+    return BSP_ERR_ARG;
+  if (block != 64 || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
+  if (maxlut > BSP_ATTENTION_MAX_ROW_BLOCKS) return BSP_ERR_ROW_TOO_LONG;
+  // 16-byte vector accesses everywhere: every pointer and every stride a multiple of 8 elements
+  const void *ptrs[] = {a.x, a.y1, a.y2, a.p_in, a.o_in, a.p_out, a.o, a.rpe, a.kpm, a.attn};
+  for (const void *p : ptrs)
+    if (!aligned16(p)) return BSP_ERR_ARG;
+  const int64_t strides[] = {a.x_sz, a.x_sh, a.x_ld, a.y1_sz, a.y1_sh, a.y1_ld, a.y2_sz, a.y2_sh, a.y2_ld, a.o_sz, a.o_sh, a.o_ld,
+                             a.pin_sz, a.pout_sz, a.rpe_sz, a.rpe_sh, a.rpe_sr, a.kpm_sz, a.attn_sr, a.oin_sz, a.oin_sh, a.oin_ld};
+  for (int64_t s : strides)
+    if (s % 8) return BSP_ERR_ARG;
+  if (a.x_ld < D || a.y1_ld < D || a.y2_ld < D || a.o_ld < D || (bwd && a.oin_ld < D)) return BSP_ERR_ARG;
+  if ((int64_t)a.Z * a.H * a.R >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  int rc;
+  if (dtype == BSP_F16) rc = launch_t<f16>(a, D, maxlut, bwd, as_stream(stream));
+  else rc = launch_t<bf16>(a, D, maxlut, bwd, as_stream(stream));
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
+}
+
+}  // namespace
+}  // namespace bsp
+
+using namespace bsp;
+
+extern "C" int bsp_attention_fwd(int dtype, const void *q, const void *k, const void *v, void *p, void *o, int Z, int H, int R,
+                                 int D, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t k_stride_z, int64_t k_stride_h,
+                                 int64_t ldk, int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t o_stride_z,
+                                 int64_t o_stride_h, int64_t ldo, int64_t p_stride_z, int block, float scale, const int32_t *d_lut,
+                                 int maxlut, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
+                                 const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r,
+                                 int attn_mul, void *stream) {
+  AttnArgs a{};
+  a.x = q; a.y1 = k; a.y2 = v; a.p_in = nullptr; a.p_out = p; a.o = o;
+  a.x_sz = q_stride_z; a.x_sh = q_stride_h; a.x_ld = ldq;
+  a.y1_sz = k_stride_z; a.y1_sh = k_stride_h; a.y1_ld = ldk;
+  a.y2_sz = v_stride_z; a.y2_sh = v_stride_h; a.y2_ld = ldv;
+  a.o_sz = o_stride_z; a.o_sh = o_stride_h; a.o_ld = ldo;
+  a.pin_sz = 0; a.pout_sz = p_stride_z;
+  a.scale = scale; a.lut = d_lut;
+  a.rpe = rpe; a.rpe_sz = rpe_stride_z; a.rpe_sh = rpe_stride_h; a.rpe_sr = rpe_stride_r;
+  a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
+  a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
+  a.Z = Z; a.H = H; a.R = R;
+  return run(dtype, a, D, block, maxlut, false, stream);
+}
+
+extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, const void *p, const void *o, void *ds,
+                                 void *dq, int Z, int H, int R, int D, int64_t do_stride_z, int64_t do_stride_h, int64_t lddo,
+                                 int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
+                                 int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
+                                 int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
+                                 const int32_t *d_lut, int maxlut, void *stream) {
+  AttnArgs a{};
+  a.x = d_o; a.y1 = v; a.y2 = k; a.p_in = p; a.p_out = ds; a.o = dq;
+  a.o_in = o; a.oin_sz = o_stride_z; a.oin_sh = o_stride_h; a.oin_ld = ldo;
+  a.x_sz = do_stride_z; a.x_sh = do_stride_h; a.x_ld = lddo;
+  a.y1_sz = v_stride_z; a.y1_sh = v_stride_h; a.y1_ld = ldv;
+  a.y2_sz = k_stride_z; a.y2_sh = k_stride_h; a.y2_ld = ldk;
+  a.o_sz = dq_stride_z; a.o_sh = dq_stride_h; a.o_ld = lddq;
+  a.pin_sz = p_stride_z; a.pout_sz = ds_stride_z;
+  a.scale = scale; a.lut = d_lut;
+  a.Z = Z; a.H = H; a.R = R;
+  return run(dtype, a, D, block, maxlut, true, stream);
+}

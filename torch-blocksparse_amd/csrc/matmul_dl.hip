@@ -35,8 +35,12 @@ inline bool raise_lds_limit(const void *kernel, int bytes, std::atomic<uint64_t>
 
 #define BSP_GLOBAL_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
 #define BSP_LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
-// wait until at most n vector-memory operations of this wavefront are outstanding (nothing else is waited for)
-#define BSP_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0xF << 8))
+// Wait until at most n vector-memory operations of this wavefront are outstanding and all of its LDS reads have
+// returned.  It stands before the barrier of a reduction step, behind which other wavefronts start the direct-to-LDS
+// loads that overwrite the stage read last: a read still in flight then could return the new bytes.  (In these
+// kernels the matrix instructions that consume a step's reads come before the barrier in the compiled code, so the
+// reads have returned anyway; the explicit wait does not leave that to the instruction scheduler.)
+#define BSP_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 0xF) | (((n) >> 4) << 14) | (0x7 << 4) | (0x0 << 8))
 
 constexpr int kTK = 32;          // reduction step (elements)
 constexpr int kTN = 256;         // tile of the dense free dimension

@@ -10,6 +10,7 @@ import torch
 import torch.nn as nn
 from torch.nn.functional import linear
 
+from .attention_core import attention_chain
 from .layouts import make_layout  # noqa: F401  (re-exported like the reference's attention.make_layout)
 from .matmul import MatMul
 from .softmax import Softmax
@@ -104,13 +105,12 @@ def multi_head_attention_forward(query, key, value, embed_dim_to_check, num_head
     q = q.reshape(bsz, num_heads, q.shape[1], q.shape[2]).contiguous()
     k = k.reshape(bsz, num_heads, k.shape[1], k.shape[2]).contiguous()
     v = v.reshape(bsz, num_heads, v.shape[1], v.shape[2]).contiguous()
-    w = sparse_dot_sdd_nt(q, k)
-    # dropout on the attention weights (nn.functional.multi_head_attention_forward applies it after the softmax; the
-    # reference raises NotImplementedError for dropout != 0): fused into the softmax kernel
-    w = sparse_softmax(w, key_padding_mask=key_padding_mask, attn_mask=attn_mask,
-                       key_padding_mask_mode=key_padding_mask_mode, attn_mask_mode=attn_mask_mode,
-                       dropout_p=float(dropout_p) if training else 0.)
-    out = sparse_dot_dsd_nn(w, v)
+    # The reference's three calls (attention.py:190-202), in one launch where the kernels allow it.  Dropout on the
+    # attention weights (nn.functional.multi_head_attention_forward applies it after the softmax; the reference raises
+    # NotImplementedError for dropout != 0) is fused into the softmax kernel of the three-operator path.
+    out = attention_chain(sparse_dot_sdd_nt, sparse_softmax, sparse_dot_dsd_nn, q, k, v, key_padding_mask=key_padding_mask,
+                          attn_mask=attn_mask, key_padding_mask_mode=key_padding_mask_mode, attn_mask_mode=attn_mask_mode,
+                          dropout_p=float(dropout_p) if training else 0.)
     out = out.reshape(bsz * num_heads, out.shape[2], out.shape[3])
     out = out.transpose(0, 1).contiguous().view(tgt_len, bsz, embed_dim)
     out = linear(out, out_proj_weight, out_proj_bias)

@@ -1,0 +1,169 @@
+"""The chain scores -> softmax -> context of the attention modules, in one launch per direction where that is possible.
+
+The reference's modules call three operators, sparse_dot_sdd_nt(q, k), sparse_softmax(...), sparse_dot_dsd_nn(p, v)
+(deepspeedsparseselfattention.py:152-157; attention.py:190-202).  `attention_chain` takes the same three operator
+objects and the same arguments and returns the same context tensor; when the operators are this package's, built on
+one layout with blocks of 64, and the tensors are fp16 / bf16 with a head dimension of 64 or 128, it runs the fused
+kernels (bsp_attention_fwd / bsp_attention_bwd) instead: the scores stay in registers between the three steps.
+In every other case, and with FUSED = False, it calls the three operators one after the other.
+"""
+import ctypes
+import os
+
+import torch
+
+from . import _lib
+from .matmul import MatMul
+from .softmax import Softmax, _sparse_softmax
+
+FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
+MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS
+fused_calls = 0             # forward calls that took the fused kernels; tests read it
+
+
+def _vec_ok(t):
+    """16-byte vector accesses: unit inner stride, every other stride a multiple of 8 elements, aligned base."""
+    return t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1])
+
+
+def _vec(t):
+    return t if _vec_ok(t) else t.contiguous()
+
+
+class AttentionCore:
+    """What the fused kernels need beside the tensors: the softmax table of the layout and the two products that stay
+    ordinary operators in the backward pass (dv = p^T . do and dk = ds^T . q)."""
+
+    def __init__(self, layout, block, softmax=None):
+        self.layout = layout
+        self.block = block
+        self.spdims = tuple(layout.shape)
+        self.softmax = softmax if softmax is not None else Softmax(layout, block)
+        self.dsd_tn = MatMul(layout, block, 'dsd', trans_a=True, trans_b=False)
+        self.nnz = None
+
+    def blocks(self):
+        if self.nnz is None:
+            self.nnz = int((self.layout != 0).sum())
+        return self.nnz
+
+    def usable(self, q, k, v, dropout_p=0.):
+        """Can this call take the fused kernels?  (Shapes that do not fit the layout are left to the operators, which
+        raise the reference's errors.)"""
+        if not FUSED or self.block != 64 or dropout_p:
+            return False
+        if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
+            return False
+        if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.size(3) not in (64, 128):
+            return False
+        H, R, C = self.spdims
+        Z, D = q.size(0), q.size(3)
+        if tuple(q.shape) != (Z, H, R * 64, D) or tuple(k.shape) != (Z, H, C * 64, D) or tuple(v.shape) != (Z, H, C * 64, D):
+            return False
+        _, maxlut = self.softmax.make_lut(q.device)
+        return 0 < maxlut <= MAX_ROW_BLOCKS
+
+    def __call__(self, q, k, v, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
+                 key_padding_mask_mode='add', attn_mask_mode='add'):
+        for name, m in (('relative position embedding', rpe), ('Attention mask', attn_mask), ('Key padding mask', key_padding_mask)):
+            if m is not None and m.dtype != q.dtype:      # softmax.py:348-353
+                raise ValueError('%s must be %s' % (name, q.dtype))
+        lut, maxlut = self.softmax.make_lut(q.device)
+        return _attention_core.apply(q, k, v, float(scale), rpe, key_padding_mask, attn_mask, key_padding_mask_mode,
+                                     attn_mask_mode, self, lut, maxlut)
+
+
+class _attention_core(torch.autograd.Function):
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode, core, lut, maxlut):
+        global fused_calls
+        H, R, C = core.spdims
+        Z, D = q.size(0), q.size(3)
+        nnz = core.blocks()
+        # the masks against the layout, exactly as the softmax operator checks them (it takes every address from the table)
+        _sparse_softmax._check_shapes(torch.empty((Z, nnz, 64, 64), device='meta'), rpe, key_padding_mask, attn_mask, core.spdims, 64, nnz)
+        q, k, v = _vec(q), _vec(k), _vec(v)
+        null = ctypes.c_void_p(0)
+        rpe_args = (null, 0, 0, 0)
+        if rpe is not None:                                # element (z, h, r, c), softmax.py:50-55, 265
+            while rpe.dim() < 4:
+                rpe = rpe.unsqueeze(0)
+            rpe = _sparse_softmax._strided16(rpe.expand(Z, H, rpe.size(2), rpe.size(3)), 'rpe')
+            rpe_args = (_lib.ptr(rpe), rpe.stride(0), rpe.stride(1), rpe.stride(2))
+        kpm_args = (null, 0)
+        if key_padding_mask is not None:                   # element (z, c), softmax.py:60-62, 274
+            key_padding_mask = _sparse_softmax._strided16(key_padding_mask, 'key_padding_mask')
+            kpm_args = (_lib.ptr(key_padding_mask), key_padding_mask.stride(0) if key_padding_mask.size(0) > 1 else 0)
+        attn_args = (null, 0)
+        if attn_mask is not None:                          # element (r, c), softmax.py:67-70, 283
+            attn_mask = _sparse_softmax._strided16(attn_mask, 'attn_mask')
+            attn_args = (_lib.ptr(attn_mask), attn_mask.stride(0))
+        p = torch.empty((Z, nnz, 64, 64), dtype=q.dtype, device=q.device)
+        o = torch.empty((Z, H, R * 64, D), dtype=q.dtype, device=q.device)
+        rc = _lib.load().bsp_attention_fwd(
+            _lib.DTYPES[q.dtype], _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(p), _lib.ptr(o), Z, H, R, D,
+            q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
+            o.stride(0), o.stride(1), o.stride(2), p.stride(0), 64, scale, _lib.ptr(lut), maxlut,
+            rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3], kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
+            attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'), _lib.stream_ptr(q.device))
+        _lib.check(rc, 'bsp_attention_fwd')
+        fused_calls += 1
+        ctx.save_for_backward(q, k, v, p, o, lut)
+        ctx.core, ctx.scale, ctx.maxlut = core, scale, maxlut
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, p, o, lut = ctx.saved_tensors
+        core = ctx.core
+        H, R, C = core.spdims
+        Z, D = q.size(0), q.size(3)
+        do = _vec(do)
+        dq = dk = dv = None
+        if ctx.needs_input_grad[2]:
+            dv = core.dsd_tn(p, do)                        # p^T . do, as the dsd operator's backward does (matmul.py:598-601)
+        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
+            ds = torch.empty_like(p)
+            dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+            rc = _lib.load().bsp_attention_bwd(
+                _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, R, D,
+                do.stride(0), do.stride(1), do.stride(2), v.stride(0), v.stride(1), v.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0), 64, ctx.scale, _lib.ptr(lut), ctx.maxlut,
+                _lib.stream_ptr(q.device))
+            _lib.check(rc, 'bsp_attention_bwd')
+            if ctx.needs_input_grad[1]:
+                dk = core.dsd_tn(ds, q)                    # ds^T . q (matmul.py:598-601 of the sdd operator)
+            if not ctx.needs_input_grad[0]:
+                dq = None
+        return (dq, dk, dv) + (None,) * 9
+
+
+def _core_for(sdd_nt, softmax, dsd_nn):
+    """The fused core that stands for this triple of operators, or None when they are not such a triple."""
+    if not (isinstance(sdd_nt, MatMul) and isinstance(dsd_nn, MatMul) and isinstance(softmax, Softmax)):
+        return None
+    core = getattr(softmax, '_attention_core', None)
+    if core is not None and core[0] is sdd_nt and core[1] is dsd_nn:
+        return core[2]
+    ok = (sdd_nt.mode == 'sdd' and not sdd_nt.trans_a and sdd_nt.trans_b and dsd_nn.mode == 'dsd' and not dsd_nn.trans_a
+          and not dsd_nn.trans_b and sdd_nt.block == softmax.block == dsd_nn.block == 64)
+    if ok:
+        for other in (sdd_nt.layout, dsd_nn.layout):
+            ok = ok and (other is softmax.layout or (other.shape == softmax.layout.shape and bool((other == softmax.layout).all())))
+    made = AttentionCore(softmax.layout, softmax.block, softmax) if ok else None
+    softmax._attention_core = (sdd_nt, dsd_nn, made)
+    return made
+
+
+def attention_chain(sdd_nt, softmax, dsd_nn, q, k, v, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
+                    key_padding_mask_mode='add', attn_mask_mode='add', dropout_p=0.):
+    """dsd_nn(softmax(sdd_nt(q, k), ...), v): fused when the operators and tensors allow it, else the three calls."""
+    core = _core_for(sdd_nt, softmax, dsd_nn)
+    if core is not None and core.usable(q, k, v, dropout_p):
+        return core(q, k, v, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode)
+    w = sdd_nt(q, k)
+    kwargs = dict(dropout_p=dropout_p) if dropout_p else {}
+    w = softmax(w, scale=scale, rpe=rpe, key_padding_mask=key_padding_mask, attn_mask=attn_mask,
+                key_padding_mask_mode=key_padding_mask_mode, attn_mask_mode=attn_mask_mode, **kwargs)
+    return dsd_nn(w, v)
