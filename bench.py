@@ -85,6 +85,15 @@ def recorded_traffic():
     return rec.get('bytes_per_launch', {}) if rec.get('kernel_sources_sha256') == kernel_sources_sha() else {}
 
 
+def recorded_kernel_traffic(kernel):
+    """HBM bytes per launch of one kernel from the same record (None when absent or stale)."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return None
+    return rec.get('bytes_per_kernel_launch', {}).get(kernel) if rec.get('kernel_sources_sha256') == kernel_sources_sha() else None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -236,6 +245,30 @@ def main():
         'roofline': roofline, 'kernels': kernels, 'calibration_copy': calib,
         'traffic_source': os.path.relpath(TRAFFIC_FILE, ROOT) if traffic else None,
     }
+    if block == 64:
+        # not the headline: the same workload through the call the attention modules make, which takes the fused kernels
+        ms_fused = fused_chain_step(w, args.steps, args.warmup)
+        if ms_fused is not None:
+            def timeit(f, reps=max(20, min(args.steps, 100))):
+                for _ in range(5):
+                    f()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                for _ in range(reps):
+                    f()
+                e1.record()
+                e1.synchronize()
+                return e0.elapsed_time(e1) / reps
+            out['fused_attention_chain'] = {
+                'what': 'attention_chain(sdd, softmax, dsd, q, k, v): bsp_attention_fwd, then in the backward pass dsd (p^T.do), '
+                        'bsp_attention_bwd, dsd (ds^T.q); same workload, same flop count',
+                'ms_per_step': round(ms_fused, 4), 'TFLOP/s': round(6 * w.flops_mm / ms_fused * 1e-9, 3),
+                'vs_three_operators': round(ms_per_step / ms_fused, 3),
+                'launches': fused_chain_launches(w.lay, w.q.detach(), w.k.detach(), w.v.detach(), w.do, w.scale, timeit,
+                                                 [('additive key-padding mask', dict(key_padding_mask=w.kpm))])}
+            if traffic:
+                for ent in out['fused_attention_chain']['launches']:
+                    ent['roofline']['traffic'] = recorded_kernel_traffic(ent['roofline']['kernel'])
     lay, dh, scale = w.lay, w.dh, w.scale
     del w
     torch.cuda.empty_cache()
@@ -369,6 +402,75 @@ def xsd_kernel_name(block, dtype_bits, free_dim, sp_trans, dn_kc):
         if block == 32 and free_dim <= 128:
             return 'k_xsd_rg_small'
     return 'k_xsd (general)'
+
+
+def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants):
+    """The fused attention kernels (bsp_attention_fwd / bsp_attention_bwd: what the attention modules launch instead of
+    sdd -> softmax -> dsd when block, dtype and head dimension allow), each timed on its own through the C ABI.
+    variants: [(label, softmax keyword arguments)] for the forward kernel.  Algorithmic bytes: forward q, k, v, o and
+    the sparse p once each; backward do, o, v, k, dq and the sparse p and ds once each (masks: what the layout touches
+    is counted by the caller's softmax figures, not here)."""
+    import torch
+    from torch_blocksparse import attention_core as ac
+    core = ac.AttentionCore(lay, 64)
+    B, H, L, dh = q.shape
+    nnz = core.blocks()
+    dense = q.numel() * q.element_size()
+    xb = B * nnz * 64 * 64 * q.element_size()
+    out = []
+    state = {}
+    for label, kw in variants:
+        def fwd():
+            with torch.no_grad():
+                state['o'] = ac._attention_core.forward(state.setdefault('ctx', _Ctx()), q, k, v, float(scale), kw.get('rpe'), kw.get('key_padding_mask'),
+                                                        kw.get('attn_mask'), kw.get('key_padding_mask_mode', 'add'), kw.get('attn_mask_mode', 'add'),
+                                                        core, *core.softmax.make_lut(q.device))
+        ms = timeit(fwd)
+        nbytes = 4 * dense + xb
+        out.append({'launch': 'fused forward: q.k^T, softmax, p.v (%s)' % label, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
+                    'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_fwd', 0, nbytes, ms)})
+    ctx = state['ctx']
+    ctx.needs_input_grad = (True, False, False)      # the kernel alone: dk and dv are the two dsd launches listed with the operators
+
+    def bwd():
+        with torch.no_grad():
+            ac._attention_core.backward(ctx, do)
+    ms = timeit(bwd)
+    nbytes = 5 * dense + 2 * xb
+    out.append({'launch': 'fused backward: do.v^T, softmax gradient, ds.k', 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
+                'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_bwd', 0, nbytes, ms)})
+    return out
+
+
+class _Ctx:
+    """Stand-in for the autograd context when the fused kernels are called outside autograd (timing only)."""
+    needs_input_grad = (True, True, True)
+
+    def save_for_backward(self, *t):
+        self.saved_tensors = t
+
+
+def fused_chain_step(w, steps, warmup):
+    """The headline workload through attention_chain (the call the attention modules make): forward and backward with the
+    fused kernels, timed like the headline step."""
+    import torch
+    from torch_blocksparse import attention_core as ac
+
+    def step():
+        w.q.grad = w.k.grad = w.v.grad = None
+        o = ac.attention_chain(w.sdd, w.sm, w.dsd, w.q, w.k, w.v, scale=w.scale, key_padding_mask=w.kpm)
+        o.backward(w.do)
+    before = ac.fused_calls
+    for _ in range(SETTLE_STEPS + warmup):
+        step()
+    torch.cuda.synchronize()
+    if ac.fused_calls == before:
+        return None
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
 
 
 def other_config(config, steps, warmup):
@@ -519,6 +621,8 @@ def other_config(config, steps, warmup):
                           else 'k_xsd64_rg<sparse operand %s>' % ('transposed' if '^T.' in name else 'as stored'))
                 ent['roofline'] = launch_roofline(kernel, flops, nbytes, ms)
                 out.append(ent)
+        out.extend(fused_chain_launches(lay, q, k, v, do, 0.125, timeit,
+                                        [('scale only', {}), ('rpe + causal mask', dict(rpe=rpe, attn_mask=causal, attn_mask_mode='mul'))]))
         workload = ('BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, '
                     'forward and backward launches; bound: HBM (softmax bytes: 2|x| + the mask and rpe bytes the layout touches)')
     torch.cuda.empty_cache()
@@ -737,6 +841,9 @@ def record_traffic(fetch_dir, write_dir):
         ('k_sdd64_rg', ('k_sdd64_rg',)), ('k_xsd64_rg<sparse operand as stored>', ('k_xsd64_rg', 'Lb0E')),
         ('k_xsd64_rg<sparse operand transposed>', ('k_xsd64_rg', 'Lb1E')), ('k_softmax_fwd', ('k_softmax_fwd',)),
         ('k_softmax_bwd', ('k_softmax_bwd',)))}
+    for name in ('k_attn64_fwd', 'k_attn64_bwd'):          # the fused chain of the attention modules, run after the headline step
+        if any(name in k for k in fetch) and any(name in k for k in write):
+            per_kernel[name] = kernel_bytes(name, name)
     rec = {'kernel_sources_sha256': kernel_sources_sha(), 'bytes_per_counted_KiB': {'FETCH_SIZE': round(fs, 1), 'WRITE_SIZE': round(ws, 1)},
            'bytes_per_kernel_launch': per_kernel, 'counters_per_kernel_launch': split,
            'bytes_per_launch': {name: per_kernel[k] for name, k in KERNEL_OF.items()},
