@@ -56,6 +56,59 @@ def test_attention_chain_captured_and_replayed(block, dtype):
             assert torch.equal(a, b), 'replay %d differs from the eager run: %s (block %d)' % (rep, name, block)
 
 
+@pytest.mark.parametrize('masked', [False, True])
+def test_fused_attention_chain_captured_and_replayed(masked):
+    # the call the attention modules make: one fused launch per direction plus the two transposed products
+    from torch_blocksparse import attention_core as ac
+    torch.manual_seed(6)
+    B, H, L, dh = 2, 3, 1024, 64
+    lay = tb.sparse_transformer_layout(H, L // 64, 4, 8, True)
+    sdd = tb.MatMul(lay, 64, 'sdd', trans_a=False, trans_b=True)
+    dsd = tb.MatMul(lay, 64, 'dsd')
+    sm = tb.Softmax(lay, 64)
+    q, k, v, do = [torch.randn(B, H, L, dh, device=DEV, dtype=torch.float16) for _ in range(4)]
+    kpm = torch.zeros(B, L, device=DEV, dtype=torch.float16)
+    kpm[1, L - 100:] = float('-inf')
+    kw = dict(scale=0.125, key_padding_mask=kpm)
+    if masked:
+        kw.update(attn_mask=torch.tril(torch.ones(L, L, device=DEV, dtype=torch.float16)), attn_mask_mode='mul',
+                  rpe=(0.2 * torch.randn(L, L, device=DEV)).half())
+    old = ac.FUSED
+    ac.FUSED = True
+    try:
+        def chain(q, k, v, do):
+            qg, kg, vg = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+            n0 = ac.fused_calls
+            o = ac.attention_chain(sdd, sm, dsd, qg, kg, vg, **kw)
+            assert ac.fused_calls == n0 + 1
+            dq, dk, dv = torch.autograd.grad(o, (qg, kg, vg), do)
+            return o.detach(), dq, dk, dv
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                chain(q, k, v, do)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        static_in = [t.clone() for t in (q, k, v, do)]
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            static_out = chain(*static_in)
+        for rep in range(4):
+            fresh = [torch.randn_like(t) for t in static_in]
+            eager = chain(*fresh)
+            torch.cuda.synchronize()
+            for s_, f in zip(static_in, fresh):
+                s_.copy_(f)
+            graph.replay()
+            torch.cuda.synchronize()
+            for name, a, b in zip(('out', 'dq', 'dk', 'dv'), static_out, eager):
+                assert torch.equal(a, b), 'replay %d differs from the eager run: %s' % (rep, name)
+    finally:
+        ac.FUSED = old
+
+
 def test_split_chains_captured_then_a_larger_eager_call_between_replays():
     # A layout with a line of more than 128 blocks: the chain is cut into parts whose fp32 partial tiles live in the
     # plan's workspace, and a captured launch carries that buffer's address.  An eager call with a larger batch between
