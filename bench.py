@@ -245,7 +245,7 @@ def main():
         'roofline': roofline, 'kernels': kernels, 'calibration_copy': calib,
         'traffic_source': os.path.relpath(TRAFFIC_FILE, ROOT) if traffic else None,
     }
-    if block == 64:
+    if True:
         # not the headline: the same workload through the call the attention modules make, which takes the fused kernels
         ms_fused = fused_chain_step(w, args.steps, args.warmup)
         if ms_fused is not None:
@@ -265,7 +265,7 @@ def main():
                 'ms_per_step': round(ms_fused, 4), 'TFLOP/s': round(6 * w.flops_mm / ms_fused * 1e-9, 3),
                 'vs_three_operators': round(ms_per_step / ms_fused, 3),
                 'launches': fused_chain_launches(w.lay, w.q.detach(), w.k.detach(), w.v.detach(), w.do, w.scale, timeit,
-                                                 [('additive key-padding mask', dict(key_padding_mask=w.kpm))])}
+                                                 [('additive key-padding mask', dict(key_padding_mask=w.kpm))], block)}
             if traffic:
                 for ent in out['fused_attention_chain']['launches']:
                     ent['roofline']['traffic'] = recorded_kernel_traffic(ent['roofline']['kernel'])
@@ -404,7 +404,7 @@ def xsd_kernel_name(block, dtype_bits, free_dim, sp_trans, dn_kc):
     return 'k_xsd (general)'
 
 
-def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants):
+def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants, block=64):
     """The fused attention kernels (bsp_attention_fwd / bsp_attention_bwd: what the attention modules launch instead of
     sdd -> softmax -> dsd when block, dtype and head dimension allow), each timed on its own through the C ABI.
     variants: [(label, softmax keyword arguments)] for the forward kernel.  Algorithmic bytes: forward q, k, v, o and
@@ -412,11 +412,11 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants):
     is counted by the caller's softmax figures, not here)."""
     import torch
     from torch_blocksparse import attention_core as ac
-    core = ac.AttentionCore(lay, 64)
+    core = ac.AttentionCore(lay, block)
     B, H, L, dh = q.shape
     nnz = core.blocks()
     dense = q.numel() * q.element_size()
-    xb = B * nnz * 64 * 64 * q.element_size()
+    xb = B * nnz * block * block * q.element_size()
     out = []
     state = {}
     for label, kw in variants:
@@ -424,7 +424,7 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants):
             with torch.no_grad():
                 state['o'] = ac._attention_core.forward(state.setdefault('ctx', _Ctx()), q, k, v, float(scale), kw.get('rpe'), kw.get('key_padding_mask'),
                                                         kw.get('attn_mask'), kw.get('key_padding_mask_mode', 'add'), kw.get('attn_mask_mode', 'add'),
-                                                        core, *core.softmax.make_lut(q.device))
+                                                        core, *core.tables(q.device))
         ms = timeit(fwd)
         nbytes = 4 * dense + xb
         out.append({'launch': 'fused forward: q.k^T, softmax, p.v (%s)' % label, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),

@@ -269,35 +269,43 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  * The attention chain of the reference's modules in one launch per direction: replaces the sequence
  * sparse_dot_sdd_nt -> sparse_softmax -> sparse_dot_dsd_nn of DeepSpeedSparseSelfAttention.forward
  * (deepspeedsparseselfattention.py:152-157) and of multi_head_attention_forward (attention.py:190-202), and the
- * matching part of their autograd graph (matmul.py:587-606, softmax.py:315-326).  Block 64, fp16 / bf16, head
- * dimension D = 64 or 128, rows of at most BSP_ATTENTION_MAX_ROW_BLOCKS nonzero blocks (maxlut of the softmax
- * table); BSP_ERR_UNSUPPORTED / BSP_ERR_ROW_TOO_LONG otherwise, and the caller runs the three operators.
+ * matching part of their autograd graph (matmul.py:587-606, softmax.py:315-326).  fp16 / bf16, head dimension
+ * D = 64 or 128, blocks of 64, 32 or 16; BSP_ERR_UNSUPPORTED / BSP_ERR_ROW_TOO_LONG otherwise, and the caller runs
+ * the three operators.
+ *   block 64: d_lut / maxlut from bsp_softmax_lut_build on the layout, R = its block-rows, d_tiles = NULL; rows of at
+ *             most BSP_ATTENTION_MAX_ROW_BLOCKS blocks.
+ *   blocks 16 and 32 (S = 64 / block, layout sides divisible by S): the kernels work on 64 x 64 tiles.  d_lut / maxlut
+ *             from bsp_softmax_lut_build on the layout coarsened to tiles ([H, R_blocks / S, C_blocks / S], a tile
+ *             present if any of its S x S blocks is), R = its rows, at most BSP_ATTENTION_MAX_ROW_BLOCKS tiles per
+ *             row; d_tiles: per present tile, in the order of that table's block ids (row-major over head, tile-row,
+ *             tile-column), S * S ints: the ids of its blocks in the [Z, nnz, block, block] tensor, row by row, -1
+ *             where absent.
  *   forward : p = softmax(round(q . k^T) * scale + rpe + kpm + attn) over each row's nonzero blocks, o = p . v.
- *             q, o: [Z, H, 64 R, D]; k, v: [Z, H, 64 C, D], unit stride along D; p: [Z, nnz, 64, 64] (every block is
- *             written); rows of o in an empty block-row are set to zero.  Masks as for bsp_softmax_fwd.
+ *             q, o: [Z, H, rows, D]; k, v: [Z, H, columns, D], unit stride along D; p: [Z, nnz, block, block] (every
+ *             block is written); rows of o without any block are set to zero.  Masks as for bsp_softmax_fwd.
  *   backward: ds = p * (round(do . v^T) - delta) * scale, dq = ds . k, with delta = sum_d do[row][d] * o[row][d], o
  *             the result of the forward call: in exact arithmetic this is the sum over the row of p * (do . v^T) that
  *             the softmax gradient subtracts (softmax.py:187-189), and it is known before the row's blocks are, so
- *             each block is finished as soon as its product is.  ds: [Z, nnz, 64, 64], a tensor of its own.  The two
- *             remaining gradients are ordinary products of the caller: dk = ds^T . q and dv = p^T . do
+ *             each block is finished as soon as its product is.  ds: [Z, nnz, block, block], a tensor of its own.
+ *             The two remaining gradients are ordinary products of the caller: dk = ds^T . q and dv = p^T . do
  *             (bsp_dsd_matmul with trans_a).
  * round() is the rounding to the storage type that the scores undergo when the sdd operator stores them, kept so
- * that the result matches the three-operator chain.  d_lut / maxlut from bsp_softmax_lut_build.  Every pointer
- * 16-byte aligned, every stride a multiple of 8 elements. */
+ * that the result matches the three-operator chain.  Every pointer 16-byte aligned, every stride a multiple of 8
+ * elements. */
 #define BSP_ATTENTION_MAX_ROW_BLOCKS 8
 int bsp_attention_fwd(int dtype, const void *q, const void *k, const void *v, void *p, void *o, int Z, int H, int R,
                       int D, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t k_stride_z, int64_t k_stride_h,
                       int64_t ldk, int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t o_stride_z,
                       int64_t o_stride_h, int64_t ldo, int64_t p_stride_z, int block, float scale, const int32_t *d_lut,
-                      int maxlut, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
-                      const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r,
-                      int attn_mul, void *stream);
+                      int maxlut, const int32_t *d_tiles, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h,
+                      int64_t rpe_stride_r, const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn,
+                      int64_t attn_stride_r, int attn_mul, void *stream);
 int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, const void *p, const void *o, void *ds,
                       void *dq, int Z, int H, int R, int D, int64_t do_stride_z, int64_t do_stride_h, int64_t lddo,
                       int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                       int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                       int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                      const int32_t *d_lut, int maxlut, void *stream);
+                      const int32_t *d_lut, int maxlut, const int32_t *d_tiles, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Dense utility ops of the reference package.

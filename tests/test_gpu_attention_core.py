@@ -231,7 +231,7 @@ def test_cases_left_to_the_three_operators():
     o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0
     assert_close(o, D.attention(q, k, v, layout, 64, 0.125, attn_mask_mode='add'), torch.float16, 'o')
-    # dropout, fp32, another block size, a head dimension the kernels do not have
+    # dropout, fp32, a head dimension the kernels do not have, blocks of 128
     lay = torch.tril(torch.ones(H, 4, 4)).long()
     ops = _ops(lay)
     q, k, v = [torch.randn(Z, H, 256, dh, device=DEV).half() for _ in range(3)]
@@ -240,11 +240,10 @@ def test_cases_left_to_the_three_operators():
         n0 = ac.fused_calls
         ac.attention_chain(ops[0], ops[1], ops[2], *args, scale=0.125, **kw)
         assert ac.fused_calls == n0
-    ops32 = (tb.MatMul(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32, 'sdd', trans_b=True),
-             tb.Softmax(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32),
-             tb.MatMul(lay.repeat_interleave(2, 1).repeat_interleave(2, 2), 32, 'dsd'))
+    lay128 = torch.ones(H, 2, 2).long()                        # blocks of 128 have no fused kernel
+    ops128 = (tb.MatMul(lay128, 128, 'sdd', trans_b=True), tb.Softmax(lay128, 128), tb.MatMul(lay128, 128, 'dsd'))
     n0 = ac.fused_calls
-    ac.attention_chain(ops32[0], ops32[1], ops32[2], q, k, v, scale=0.125)
+    ac.attention_chain(ops128[0], ops128[1], ops128[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0
     # operators built on different layouts are not a chain the fused kernels can stand for
     other = lay.clone()
@@ -256,6 +255,90 @@ def test_cases_left_to_the_three_operators():
         ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, key_padding_mask=torch.zeros(Z, 256, device=DEV))
 
 
+@pytest.mark.parametrize('block,dtype,dh,R,C,density,masks', [
+    (32, torch.float16, 64, 8, 8, 0.5, ()),
+    (16, torch.float16, 64, 16, 16, 0.4, ('kpm',)),
+    (16, torch.float16, 64, 32, 32, 0.3, ('kpm', 'attn')),
+    (32, torch.bfloat16, 128, 16, 12, 0.4, ('kpm', 'rpe')),
+    (16, torch.float16, 128, 24, 32, 0.25, ('rpe',)),
+    (16, torch.bfloat16, 64, 12, 20, 0.15, ()),
+])
+def test_blocks_of_16_and_32_on_gathered_tiles(block, dtype, dh, R, C, density, masks):
+    """Small blocks: the kernels work on 64 x 64 tiles of the layout; blocks absent from a present tile take no part in
+    the softmax and are not stored, a row of small blocks without any block (inside a tile-row that its neighbours
+    keep alive) gives zero rows of o and dq, rectangular layouts, every mask."""
+    torch.manual_seed(R * C + block)
+    Z, H = 2, 2
+    lay = (torch.rand(H, R, C) < density).long()
+    lay[:, :, 0] = 1
+    lay[:, 4:8, :] = 0                # rows of small blocks without any block ...
+    lay[:, 5, 3] = 1                  # ... one of which is kept (so at block 16 its tile-row exists)
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.Softmax(lay, block), tb.MatMul(lay, block, 'dsd'))
+    q, do = [torch.randn(Z, H, R * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    k, v = [torch.randn(Z, H, C * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    kw = dict(scale=dh ** -0.5)
+    if 'kpm' in masks:
+        m = torch.zeros(Z, C * block)
+        m[0, -37:] = float('-inf')
+        kw['key_padding_mask'] = m.to(DEV).to(dtype)
+    if 'rpe' in masks:
+        kw['rpe'] = (0.3 * torch.randn(R * block, C * block)).to(DEV).to(dtype)
+    if 'attn' in masks:
+        kw.update(attn_mask=(torch.rand(R * block, C * block) < 0.8).to(DEV).to(dtype), attn_mask_mode='mul')
+        kw['attn_mask'][:, 0] = 1      # (no row loses all its columns)
+    with guard_allocations('fused attention, block %d' % block):
+        got = _run(ops, q, k, v, do, True, **kw)
+    chain = _run(ops, q, k, v, do, False, **kw)
+    live = lay.sum(2).ne(0).all(0)                    # rows of small blocks that hold a block in every head
+    rows = live.repeat_interleave(block)
+    dead = ~lay.sum(2).ne(0).any(0).repeat_interleave(block)
+    assert not bool(got[0][:, :, dead.to(DEV)].any()) and not bool(got[1][:, :, dead.to(DEV)].any())
+    tol = CHAIN_TOL[dtype][1]
+    for name, g, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
+        assert not bool(torch.isnan(g).any()), name
+        assert float((g.float() - c.float()).abs().max()) <= tol * float(c.float().abs().max()), name
+    okw = {n: kw[n] for n in ('key_padding_mask', 'attn_mask') if n in kw}
+    if 'rpe' in kw:
+        okw['rpe'] = kw['rpe'][rows.to(DEV)]
+    if 'attn_mask' in okw:
+        okw['attn_mask'] = okw['attn_mask'][rows.to(DEV)]
+    ref = D.attention(q[:, :, rows.to(DEV)], k, v, lay[:, live], block, kw['scale'], do=do[:, :, rows.to(DEV)],
+                      attn_mask_mode=kw.get('attn_mask_mode', 'add'), **okw)
+    assert_close(got[0][:, :, rows.to(DEV)], ref[0], dtype, 'o')
+    assert_close(got[1][:, :, rows.to(DEV)], ref[1], dtype, 'dq')
+    # dk and dv collect contributions from every row: against the oracle when the rows left out above (empty in some
+    # head) are empty in every head, against the three operators (above) in any case
+    if bool((lay.sum(2).ne(0).all(0) | ~lay.sum(2).ne(0).any(0)).all()):
+        assert_close(got[2], ref[2], dtype, 'dk')
+        assert_close(got[3], ref[3], dtype, 'dv')
+
+
+def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
+    torch.manual_seed(9)
+    Z, H, dh = 1, 2, 64
+    q, k, v = [torch.randn(Z, H, 18 * 16, dh, device=DEV).half() for _ in range(3)]
+    lay = torch.tril(torch.ones(H, 18, 18)).long()            # 18 rows of blocks of 16: not a whole number of tiles
+    ops = (tb.MatMul(lay, 16, 'sdd', trans_b=True), tb.Softmax(lay, 16), tb.MatMul(lay, 16, 'dsd'))
+    n0 = ac.fused_calls
+    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    assert ac.fused_calls == n0
+    assert_close(o, D.attention(q, k, v, lay, 16, 0.125, attn_mask_mode='add'), torch.float16, 'o')
+    # a tile-row of nine tiles
+    lay = torch.ones(H, 4, 36).long()
+    ops = (tb.MatMul(lay, 16, 'sdd', trans_b=True), tb.Softmax(lay, 16), tb.MatMul(lay, 16, 'dsd'))
+    q = torch.randn(Z, H, 64, dh, device=DEV).half()
+    k, v = [torch.randn(Z, H, 36 * 16, dh, device=DEV).half() for _ in range(2)]
+    n0 = ac.fused_calls
+    ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    assert ac.fused_calls == n0
+    # the default block of the sparse self-attention module is 16: it takes the fused kernels
+    mod = tb.SparseSelfAttention(tb.SparsityConfig(mode='fixed', block=16, stride=64, attention='unidirectional'))
+    q, k, v = [torch.randn(2, 4, 512, dh, device=DEV).half() for _ in range(3)]
+    n0 = ac.fused_calls
+    mod(q, k, v)
+    assert ac.fused_calls == n0 + 1
+
+
 def test_c_abi_argument_checks():
     lib = _lib.load()
     t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
@@ -264,13 +347,15 @@ def test_c_abi_argument_checks():
     null = ctypes.c_void_p(0)
     st = (t.stride(0), t.stride(1), t.stride(2))
 
-    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64):
+    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64, tiles=null):
         return lib.bsp_attention_fwd(dtype, _lib.ptr(q), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(t.clone()), 1, 1, 1, D,
-                                     st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut,
+                                     st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut, tiles,
                                      null, 0, 0, 0, null, 0, 0, null, 0, 0, _lib.stream_ptr(torch.device(DEV)))
     assert fwd() == _lib.OK
     assert fwd(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
-    assert fwd(block=32) == _lib.ERR_UNSUPPORTED
+    assert fwd(block=128) == _lib.ERR_UNSUPPORTED
+    assert fwd(block=32) != _lib.OK                     # small blocks need the tile table
+    assert fwd(tiles=_lib.ptr(lut)) != _lib.OK          # ... and blocks of 64 take none
     assert fwd(D=96) == _lib.ERR_UNSUPPORTED
     assert fwd(maxlut=9) == _lib.ERR_ROW_TOO_LONG
     assert fwd(ldq=60) != _lib.OK                       # a row stride that is not a multiple of 8 elements

@@ -71,6 +71,7 @@ struct AttnArgs {
   const void *p_in;          // backward: the saved softmax
   void *p_out, *o;           // forward: p, o; backward: ds, dq
   const void *o_in;          // backward: the forward result o
+  const int32_t *tiles;      // blocks of 16 / 32: per 64 x 64 tile of the layout the ids of its blocks (-1: absent), see bsp_attention_fwd
   int64_t oin_sz, oin_sh, oin_ld;
   int64_t x_sz, x_sh, x_ld, y1_sz, y1_sh, y1_ld, y2_sz, y2_sh, y2_ld, o_sz, o_sh, o_ld, pin_sz, pout_sz;
   float scale;
@@ -147,10 +148,38 @@ template <typename T> __device__ __forceinline__ void store_block_rows(T *cs, T 
   __builtin_amdgcn_wave_barrier();
 }
 
+// Blocks of 16 and 32 (SUBS = 64 / block > 1): the kernels work on 64 x 64 tiles of the layout (a tile is present if any
+// of its SUBS x SUBS blocks is); the table is the softmax table of the layout coarsened to tiles and `tiles` holds, per
+// tile in that table's order, the ids of its blocks row by row, -1 where absent.  A wavefront's 16 rows lie in one row
+// of small blocks (rs) and a lane's chunk of 8 columns in one small block: its id, or -1.
+// t = the ids of the wavefront's row of small blocks in the tile (scalars, fetched once per block of the row; kept as a
+// vector type: an array indexed in a select chain ends up in scratch memory, whose loads count as vector-memory
+// operations and stall every wait of the tile ring)
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+template <int SUBS> __device__ __forceinline__ int chunk_block_id(const i32x4 &t, int s, int q) {
+  if constexpr (SUBS == 2) return s ? t[1] : t[0];           // columns 32s + 8q .. of the tile: small block column s
+  else if constexpr (SUBS == 4) return s ? ((q >> 1) ? t[3] : t[2]) : ((q >> 1) ? t[1] : t[0]);   // small block column 2s + q / 2
+  else return 0;
+}
+template <int SUBS> __device__ __forceinline__ i32x4 load_block_ids(table_ptr tiles, int tile, int rs) {
+  i32x4 t = {0, 0, 0, 0};
+  if constexpr (SUBS > 1) {
+    const table_ptr src = tiles + (int64_t)tile * (SUBS * SUBS) + rs * SUBS;
+#pragma unroll
+    for (int c = 0; c < SUBS; c++) t[c] = src[c];
+  }
+  return t;
+}
+// the lane's chunk (row 16 * wave + lane % 16 of the tile, columns 32s + 8q ..) inside its small block, in elements
+template <int SUBS> __device__ __forceinline__ int chunk_in_block(int wave, int qrow, int s, int q) {
+  constexpr int B = 64 / SUBS;
+  return ((16 * wave + qrow) % B) * B + (32 * s + 8 * q) % B;
+}
+
 // D = head dimension (64 or 128); NB = most blocks a block-row may hold (the host picks the bucket from the table's
 // longest row); EXTRA = a relative position embedding or an attention mask is present.
-template <typename T, int D, int NB, bool EXTRA>
-__global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
+template <typename T, int D, int NB, bool EXTRA, int SUBS = 1>
+__global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(AttnArgs a) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
   typedef Pack<T, 8> P8;
@@ -199,6 +228,9 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
     bid[b] = core[4 * bb + 0];
     bcol[b] = core[4 * bb + 1];
   }
+  i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
+#pragma unroll
+  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], (16 * wave) / (64 / SUBS));
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   frag_t xq[NK];
 #pragma unroll
@@ -317,6 +349,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
     const float unit = logit_unit<T>(), sc = a.scale * unit;
     const bool has_kpm = a.kpm != nullptr;
     float mx = -INFINITY;
+    int any_block = SUBS == 1;                           // small blocks: does the lane's row of small blocks hold any block?
     constexpr int GS = EXTRA ? (NB < 4 ? NB : 4) : NB;   // blocks whose mask values are in flight together
 #pragma unroll
     for (int g = 0; g < NB; g += GS) {
@@ -348,6 +381,14 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
 #pragma unroll
               for (int i = 0; i < 8; i++) add[i] = 0.f;
             }
+            if constexpr (SUBS > 1) {                    // a chunk in an absent small block takes no part in the row
+              const bool here = chunk_block_id<SUBS>(tid_[b], s, q) >= 0;
+              any_block |= here;
+              if (!here) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) add[i] = -INFINITY;
+              }
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
               float fx = fmaf(to_float(from_float<T>(acc[b][2 * s + (i >> 2)][i & 3])), sc, add[i]);   // softmax.py:112-116, 122-124
@@ -378,6 +419,10 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
     sum += __shfl_xor(sum, 16);
     sum += __shfl_xor(sum, 32);
     const float inv = 1.f / sum;
+    if constexpr (SUBS > 1) {   // rows of a small block-row without blocks (inside a tile-row that others keep alive): zeros for p . v
+      any_block |= __shfl_xor(any_block, 16);
+      any_block |= __shfl_xor(any_block, 32);
+    }
 #pragma unroll
     for (int b = 0; b < NB; b++)
       if (b < size) {
@@ -385,7 +430,10 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
         for (int s = 0; s < 2; s++) {
           P8 y;
 #pragma unroll
-          for (int i = 0; i < 8; i++) y.e[i] = from_float<T>(acc[b][2 * s + (i >> 2)][i & 3] * inv);   // :137
+          for (int i = 0; i < 8; i++) {
+            const float v = acc[b][2 * s + (i >> 2)][i & 3] * inv;                                    // :137
+            y.e[i] = from_float<T>(SUBS > 1 && !any_block ? 0.f : v);
+          }
           pf[b][s] = __builtin_bit_cast(frag_t, y.raw);
         }
       }
@@ -425,8 +473,21 @@ __global__ void __launch_bounds__(256, 2) k_attn64_fwd(AttnArgs a) {
   store_rows<T, D>(cs, po, a.o_ld, o, lane);
 #pragma unroll
   for (int b = 0; b < NB; b++)
-    if (b < size)
-      store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+    if (b < size) {
+      if constexpr (SUBS == 1) {
+        store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+      } else {
+        // small blocks: a wavefront's rows of a block are contiguous (512 bytes at block 16, 1 KiB at block 32), so its
+        // lanes store their chunks directly, block by block; nothing is stored for an absent block
+        T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const int id = chunk_block_id<SUBS>(tid_[b], s, q);
+          if (id >= 0)
+            *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[b][s]);
+        }
+      }
+    }
 }
 
 // wait until at most c (0, 2, 4, 6 or 8) vector-memory operations are outstanding; the instruction takes an immediate
@@ -445,7 +506,7 @@ __device__ __forceinline__ void wait_vm(int c) {
 // v_0, p_0, v_1, p_1, ... (the block of p is one more 8 KiB tile of the ring: no register-staged loads inside the
 // loop, whose waits the compiler would place after all direct-to-LDS loads in flight), then k_0, k_1, ... for
 // dq = ds . k.  Only the packed ds (the operand of the second product) stays in registers.
-template <typename T, int D, int NB>
+template <typename T, int D, int NB, int SUBS = 1>
 __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
@@ -485,6 +546,9 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   int32_t bid[NB];
 #pragma unroll
   for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
+  i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
+#pragma unroll
+  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], (16 * wave) / (64 / SUBS));
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   const T *pof = reinterpret_cast<const T *>(a.o_in) + z * a.oin_sz + h * a.oin_sh + row * a.oin_ld + 8 * q;
   frag_t xq[NK], oq[NK];
@@ -507,11 +571,21 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   }
   // a block of p: rows of 128 bytes; a lane reads 16 bytes of row 16 * wave + lane % 16, sixteen consecutive rows per
   // clock: chunk c of row r at slot c ^ ((r >> 1) & 7)
+  // (small blocks: the chunk's offset inside its small block, and which small block column it lies in)
+  int colp[LWP];
 #pragma unroll
   for (int i = 0; i < LWP; i++) {
-    const int r = (wave * LWP + i) * 8 + (lane >> 3), slot = lane & 7;
-    offp[i] = r * 64 + ((slot ^ ((r >> 1) & 7)) << 3);
+    const int r = (wave * LWP + i) * 8 + (lane >> 3), slot = lane & 7, chunk = slot ^ ((r >> 1) & 7);
+    if constexpr (SUBS == 1) {
+      offp[i] = r * 64 + (chunk << 3);
+      colp[i] = 0;
+    } else {
+      constexpr int B = 64 / SUBS;
+      offp[i] = (r % B) * B + (chunk * 8) % B;
+      colp[i] = (chunk * 8) / B;
+    }
   }
+  const int rs = (16 * wave) / (64 / SUBS);              // the wavefront's row of small blocks inside a tile
   const int total = 3 * size;
   auto loads_of = [&](int n) { return n >= total ? 0 : (n < 2 * size && (n & 1)) ? LWP : LW; };
   // block-column (v and k tiles) or block id (p) of tile n, from the table (a scalar load; clamped past the end)
@@ -523,10 +597,27 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   auto issue = [&](int n, int key) {
     unsigned char *st = ring + (n % kStages) * TB;
     if (n < 2 * size && (n & 1)) {
-      const T *base = pin + (int64_t)key * 4096;
+      if constexpr (SUBS == 1) {
+        const T *base = pin + (int64_t)key * 4096;
 #pragma unroll
-      for (int i = 0; i < LWP; i++)
-        __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+        for (int i = 0; i < LWP; i++)
+          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+      } else {
+        // the tile of p gathered from its small blocks; chunks of absent blocks fetch the start of the tensor instead
+        // (every load is issued: the waits count them) and are replaced by zeros when they are read
+        const int m = n >> 1;
+        i32x4 ids = tid_[0];
+#pragma unroll
+        for (int b2 = 1; b2 < NB; b2++) ids = (m == b2) ? tid_[b2] : ids;
+#pragma unroll
+        for (int i = 0; i < LWP; i++) {
+          int id = ids[0];
+#pragma unroll
+          for (int c = 1; c < SUBS; c++) id = (colp[i] == c) ? ids[c] : id;
+          const T *src = id >= 0 ? pin + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + offp[i] : pin;
+          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(src), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+        }
+      }
     } else if (n < 2 * size) {
       const T *base = py1 + (int64_t)key * 64 * a.y1_ld;
 #pragma unroll
@@ -587,10 +678,13 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
       for (int s = 0; s < 2; s++) {
         P8 y, d;
         y.raw = *reinterpret_cast<const u32x4 *>(pt + (((q + 4 * s) ^ pswz) << 4));
+        bool here = true;
+        if constexpr (SUBS > 1) here = chunk_block_id<SUBS>(tid_[b], s, q) >= 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
           const float dp = to_float(from_float<T>(acc[2 * s + (i >> 2)][i & 3]));   // dp as the sdd operator would have stored it
-          d.e[i] = from_float<T>(to_float(y.e[i]) * (dp - delta) * a.scale);          // softmax.py:189
+          const float v = to_float(y.e[i]) * (dp - delta) * a.scale;                  // softmax.py:189
+          d.e[i] = from_float<T>(here ? v : 0.f);
         }
         pf[b][s] = __builtin_bit_cast(frag_t, d.raw);
       }
@@ -626,32 +720,49 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   store_rows<T, D>(cs, po, a.o_ld, o, lane);
 #pragma unroll
   for (int b = 0; b < NB; b++)
-    if (b < size)
-      store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+    if (b < size) {
+      if constexpr (SUBS == 1) {
+        store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
+      } else {
+        T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          const int id = chunk_block_id<SUBS>(tid_[b], s, q);
+          if (id >= 0)
+            *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[b][s]);
+        }
+      }
+    }
 }
-
 
 template <int D, int NB> constexpr int lds_bytes(bool bwd) { return ring_stages<D>() * 64 * D * 2 + (bwd ? 0 : NB * 64 * 4); }
 
-template <typename T, int D, int NB> void launch_nb(const AttnArgs &a, bool bwd, hipStream_t st) {
+template <typename T, int D, int NB, int SUBS> void launch_nb(const AttnArgs &a, bool bwd, hipStream_t st) {
   const dim3 grid((unsigned)((int64_t)a.Z * a.H * a.R)), wg(256);
   constexpr int LDS = lds_bytes<D, NB>(false), LDS_BWD = lds_bytes<D, NB>(true);
   static_assert(LDS <= 64 * 1024, "within what a launch may ask for without raising the kernel's limit");
-  if (bwd) hipLaunchKernelGGL((k_attn64_bwd<T, D, NB>), grid, wg, LDS_BWD, st, a);
-  else if (a.rpe || a.attn) hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, true>), grid, wg, LDS, st, a);
-  else hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, false>), grid, wg, LDS, st, a);
+  if (bwd) hipLaunchKernelGGL((k_attn64_bwd<T, D, NB, SUBS>), grid, wg, LDS_BWD, st, a);
+  else if (a.rpe || a.attn) hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, true, SUBS>), grid, wg, LDS, st, a);
+  else hipLaunchKernelGGL((k_attn64_fwd<T, D, NB, false, SUBS>), grid, wg, LDS, st, a);
 }
 
-template <typename T, int D> int launch_d(const AttnArgs &a, int maxlut, bool bwd, hipStream_t st) {
-  if (maxlut <= 4) launch_nb<T, D, 4>(a, bwd, st);
-  else if (maxlut <= 8) launch_nb<T, D, 8>(a, bwd, st);
+template <typename T, int D, int SUBS> int launch_d(const AttnArgs &a, int maxlut, bool bwd, hipStream_t st) {
+  if (maxlut <= 4) launch_nb<T, D, 4, SUBS>(a, bwd, st);
+  else if (maxlut <= 8) launch_nb<T, D, 8, SUBS>(a, bwd, st);
   else return BSP_ERR_ROW_TOO_LONG;
   return BSP_OK;
 }
 
-template <typename T> int launch_t(const AttnArgs &a, int D, int maxlut, bool bwd, hipStream_t st) {
-  if (D == 64) return launch_d<T, 64>(a, maxlut, bwd, st);
-  if (D == 128) return launch_d<T, 128>(a, maxlut, bwd, st);
+template <typename T, int SUBS> int launch_s(const AttnArgs &a, int D, int maxlut, bool bwd, hipStream_t st) {
+  if (D == 64) return launch_d<T, 64, SUBS>(a, maxlut, bwd, st);
+  if (D == 128) return launch_d<T, 128, SUBS>(a, maxlut, bwd, st);
+  return BSP_ERR_UNSUPPORTED;
+}
+
+template <typename T> int launch_t(const AttnArgs &a, int D, int block, int maxlut, bool bwd, hipStream_t st) {
+  if (block == 64) return launch_s<T, 1>(a, D, maxlut, bwd, st);
+  if (block == 32) return launch_s<T, 2>(a, D, maxlut, bwd, st);
+  if (block == 16) return launch_s<T, 4>(a, D, maxlut, bwd, st);
   return BSP_ERR_UNSUPPORTED;
 }
 
@@ -660,7 +771,8 @@ bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 
 int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *stream) {
   if (!a.x || !a.y1 || !a.y2 || !a.p_out || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
     return BSP_ERR_ARG;
-  if (block != 64 || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
+  if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
+  if ((block != 64) != (a.tiles != nullptr)) return BSP_ERR_ARG;   // the tile table goes with the small blocks, and only with them
   if (maxlut > BSP_ATTENTION_MAX_ROW_BLOCKS) return BSP_ERR_ROW_TOO_LONG;
   // 16-byte vector accesses everywhere: every pointer and every stride a multiple of 8 elements
   const void *ptrs[] = {a.x, a.y1, a.y2, a.p_in, a.o_in, a.p_out, a.o, a.rpe, a.kpm, a.attn};
@@ -673,8 +785,8 @@ int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *st
   if (a.x_ld < D || a.y1_ld < D || a.y2_ld < D || a.o_ld < D || (bwd && a.oin_ld < D)) return BSP_ERR_ARG;
   if ((int64_t)a.Z * a.H * a.R >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   int rc;
-  if (dtype == BSP_F16) rc = launch_t<f16>(a, D, maxlut, bwd, as_stream(stream));
-  else rc = launch_t<bf16>(a, D, maxlut, bwd, as_stream(stream));
+  if (dtype == BSP_F16) rc = launch_t<f16>(a, D, block, maxlut, bwd, as_stream(stream));
+  else rc = launch_t<bf16>(a, D, block, maxlut, bwd, as_stream(stream));
   if (rc != BSP_OK) return rc;
   BSP_LAUNCH_CHECK();
   return BSP_OK;
@@ -689,7 +801,7 @@ extern "C" int bsp_attention_fwd(int dtype, const void *q, const void *k, const 
                                  int D, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t k_stride_z, int64_t k_stride_h,
                                  int64_t ldk, int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t o_stride_z,
                                  int64_t o_stride_h, int64_t ldo, int64_t p_stride_z, int block, float scale, const int32_t *d_lut,
-                                 int maxlut, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
+                                 int maxlut, const int32_t *d_tiles, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
                                  const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r,
                                  int attn_mul, void *stream) {
   AttnArgs a{};
@@ -699,7 +811,7 @@ extern "C" int bsp_attention_fwd(int dtype, const void *q, const void *k, const 
   a.y2_sz = v_stride_z; a.y2_sh = v_stride_h; a.y2_ld = ldv;
   a.o_sz = o_stride_z; a.o_sh = o_stride_h; a.o_ld = ldo;
   a.pin_sz = 0; a.pout_sz = p_stride_z;
-  a.scale = scale; a.lut = d_lut;
+  a.scale = scale; a.lut = d_lut; a.tiles = d_tiles;
   a.rpe = rpe; a.rpe_sz = rpe_stride_z; a.rpe_sh = rpe_stride_h; a.rpe_sr = rpe_stride_r;
   a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
@@ -712,7 +824,7 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
                                  int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                                  int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                                  int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                                 const int32_t *d_lut, int maxlut, void *stream) {
+                                 const int32_t *d_lut, int maxlut, const int32_t *d_tiles, void *stream) {
   AttnArgs a{};
   a.x = d_o; a.y1 = v; a.y2 = k; a.p_in = p; a.p_out = ds; a.o = dq;
   a.o_in = o; a.oin_sz = o_stride_z; a.oin_sh = o_stride_h; a.oin_ld = ldo;
@@ -721,7 +833,7 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
   a.y2_sz = k_stride_z; a.y2_sh = k_stride_h; a.y2_ld = ldk;
   a.o_sz = dq_stride_z; a.o_sh = dq_stride_h; a.o_ld = lddq;
   a.pin_sz = p_stride_z; a.pout_sz = ds_stride_z;
-  a.scale = scale; a.lut = d_lut;
+  a.scale = scale; a.lut = d_lut; a.tiles = d_tiles;
   a.Z = Z; a.H = H; a.R = R;
   return run(dtype, a, D, block, maxlut, true, stream);
 }

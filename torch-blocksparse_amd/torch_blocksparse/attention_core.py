@@ -3,7 +3,7 @@
 The reference's modules call three operators, sparse_dot_sdd_nt(q, k), sparse_softmax(...), sparse_dot_dsd_nn(p, v)
 (deepspeedsparseselfattention.py:152-157; attention.py:190-202).  `attention_chain` takes the same three operator
 objects and the same arguments and returns the same context tensor; when the operators are this package's, built on
-one layout with blocks of 64, and the tensors are fp16 / bf16 with a head dimension of 64 or 128, it runs the fused
+one layout with blocks of 16, 32 or 64, and the tensors are fp16 / bf16 with a head dimension of 64 or 128, it runs the fused
 kernels (bsp_attention_fwd / bsp_attention_bwd) instead: the scores stay in registers between the three steps.
 In every other case, and with FUSED = False, it calls the three operators one after the other.
 """
@@ -13,7 +13,7 @@ import os
 import torch
 
 from . import _lib
-from .matmul import MatMul
+from .matmul import MatMul, _LayoutOnDevice
 from .softmax import Softmax, _sparse_softmax
 
 FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
@@ -31,8 +31,9 @@ def _vec(t):
 
 
 class AttentionCore:
-    """What the fused kernels need beside the tensors: the softmax table of the layout and the two products that stay
-    ordinary operators in the backward pass (dv = p^T . do and dk = ds^T . q)."""
+    """What the fused kernels need beside the tensors: the softmax table of the layout (of the layout coarsened to 64 x 64
+    tiles, plus the ids of each tile's blocks, when the blocks are 16 or 32) and the two products that stay ordinary
+    operators in the backward pass (dv = p^T . do and dk = ds^T . q)."""
 
     def __init__(self, layout, block, softmax=None):
         self.layout = layout
@@ -41,48 +42,67 @@ class AttentionCore:
         self.softmax = softmax if softmax is not None else Softmax(layout, block)
         self.dsd_tn = MatMul(layout, block, 'dsd', trans_a=True, trans_b=False)
         self.nnz = None
+        self._tables = dict()
 
     def blocks(self):
         if self.nnz is None:
             self.nnz = int((self.layout != 0).sum())
         return self.nnz
 
+    def tables(self, device):
+        """(table, longest row, tile table or None, rows of the table's layout) on `device`, or None when the layout does
+        not divide into 64 x 64 tiles."""
+        key = str(device)
+        if key not in self._tables:
+            S = 64 // self.block
+            H, R, C = self.spdims
+            if S == 1:
+                lut, maxlut = self.softmax.make_lut(device)
+                self._tables[key] = (lut, maxlut, None, R)
+            elif R % S or C % S:
+                self._tables[key] = None
+            else:
+                cctx, ids = _LayoutOnDevice(self.layout, device).coarse(S)
+                lut, maxlut = _sparse_softmax.make_lut(cctx.lay, 64, device)
+                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S)
+        return self._tables[key]
+
     def usable(self, q, k, v, dropout_p=0.):
         """Can this call take the fused kernels?  (Shapes that do not fit the layout are left to the operators, which
         raise the reference's errors.)"""
-        if not FUSED or self.block != 64 or dropout_p:
+        if not FUSED or self.block not in (16, 32, 64) or dropout_p:
             return False
         if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
             return False
         if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.size(3) not in (64, 128):
             return False
         H, R, C = self.spdims
-        Z, D = q.size(0), q.size(3)
-        if tuple(q.shape) != (Z, H, R * 64, D) or tuple(k.shape) != (Z, H, C * 64, D) or tuple(v.shape) != (Z, H, C * 64, D):
+        Z, D, b = q.size(0), q.size(3), self.block
+        if tuple(q.shape) != (Z, H, R * b, D) or tuple(k.shape) != (Z, H, C * b, D) or tuple(v.shape) != (Z, H, C * b, D):
             return False
-        _, maxlut = self.softmax.make_lut(q.device)
-        return 0 < maxlut <= MAX_ROW_BLOCKS
+        t = self.tables(q.device)
+        return t is not None and 0 < t[1] <= MAX_ROW_BLOCKS
 
     def __call__(self, q, k, v, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
                  key_padding_mask_mode='add', attn_mask_mode='add'):
         for name, m in (('relative position embedding', rpe), ('Attention mask', attn_mask), ('Key padding mask', key_padding_mask)):
             if m is not None and m.dtype != q.dtype:      # softmax.py:348-353
                 raise ValueError('%s must be %s' % (name, q.dtype))
-        lut, maxlut = self.softmax.make_lut(q.device)
+        lut, maxlut, tiles, rows = self.tables(q.device)
         return _attention_core.apply(q, k, v, float(scale), rpe, key_padding_mask, attn_mask, key_padding_mask_mode,
-                                     attn_mask_mode, self, lut, maxlut)
+                                     attn_mask_mode, self, lut, maxlut, tiles, rows)
 
 
 class _attention_core(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, q, k, v, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode, core, lut, maxlut):
+    def forward(ctx, q, k, v, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode, core, lut, maxlut, tiles, rows):
         global fused_calls
         H, R, C = core.spdims
-        Z, D = q.size(0), q.size(3)
+        Z, D, block = q.size(0), q.size(3), core.block
         nnz = core.blocks()
         # the masks against the layout, exactly as the softmax operator checks them (it takes every address from the table)
-        _sparse_softmax._check_shapes(torch.empty((Z, nnz, 64, 64), device='meta'), rpe, key_padding_mask, attn_mask, core.spdims, 64, nnz)
+        _sparse_softmax._check_shapes(torch.empty((Z, nnz, block, block), device='meta'), rpe, key_padding_mask, attn_mask, core.spdims, block, nnz)
         q, k, v = _vec(q), _vec(k), _vec(v)
         null = ctypes.c_void_p(0)
         rpe_args = (null, 0, 0, 0)
@@ -99,18 +119,18 @@ class _attention_core(torch.autograd.Function):
         if attn_mask is not None:                          # element (r, c), softmax.py:67-70, 283
             attn_mask = _sparse_softmax._strided16(attn_mask, 'attn_mask')
             attn_args = (_lib.ptr(attn_mask), attn_mask.stride(0))
-        p = torch.empty((Z, nnz, 64, 64), dtype=q.dtype, device=q.device)
-        o = torch.empty((Z, H, R * 64, D), dtype=q.dtype, device=q.device)
+        p = torch.empty((Z, nnz, block, block), dtype=q.dtype, device=q.device)
+        o = torch.empty((Z, H, R * block, D), dtype=q.dtype, device=q.device)
         rc = _lib.load().bsp_attention_fwd(
-            _lib.DTYPES[q.dtype], _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(p), _lib.ptr(o), Z, H, R, D,
+            _lib.DTYPES[q.dtype], _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(p), _lib.ptr(o), Z, H, rows, D,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
-            o.stride(0), o.stride(1), o.stride(2), p.stride(0), 64, scale, _lib.ptr(lut), maxlut,
+            o.stride(0), o.stride(1), o.stride(2), p.stride(0), block, scale, _lib.ptr(lut), maxlut, _lib.ptr(tiles),
             rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3], kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
             attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'), _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_fwd')
         fused_calls += 1
         ctx.save_for_backward(q, k, v, p, o, lut)
-        ctx.core, ctx.scale, ctx.maxlut = core, scale, maxlut
+        ctx.core, ctx.scale, ctx.maxlut, ctx.tiles, ctx.rows = core, scale, maxlut, tiles, rows
         return o
 
     @staticmethod
@@ -127,16 +147,16 @@ class _attention_core(torch.autograd.Function):
             ds = torch.empty_like(p)
             dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
             rc = _lib.load().bsp_attention_bwd(
-                _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, R, D,
+                _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, ctx.rows, D,
                 do.stride(0), do.stride(1), do.stride(2), v.stride(0), v.stride(1), v.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0), 64, ctx.scale, _lib.ptr(lut), ctx.maxlut,
-                _lib.stream_ptr(q.device))
+                o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0), core.block, ctx.scale, _lib.ptr(lut), ctx.maxlut,
+                _lib.ptr(ctx.tiles), _lib.stream_ptr(q.device))
             _lib.check(rc, 'bsp_attention_bwd')
             if ctx.needs_input_grad[1]:
                 dk = core.dsd_tn(ds, q)                    # ds^T . q (matmul.py:598-601 of the sdd operator)
             if not ctx.needs_input_grad[0]:
                 dq = None
-        return (dq, dk, dv) + (None,) * 9
+        return (dq, dk, dv) + (None,) * 11
 
 
 def _core_for(sdd_nt, softmax, dsd_nn):
@@ -147,7 +167,7 @@ def _core_for(sdd_nt, softmax, dsd_nn):
     if core is not None and core[0] is sdd_nt and core[1] is dsd_nn:
         return core[2]
     ok = (sdd_nt.mode == 'sdd' and not sdd_nt.trans_a and sdd_nt.trans_b and dsd_nn.mode == 'dsd' and not dsd_nn.trans_a
-          and not dsd_nn.trans_b and sdd_nt.block == softmax.block == dsd_nn.block == 64)
+          and not dsd_nn.trans_b and sdd_nt.block == softmax.block == dsd_nn.block and softmax.block in (16, 32, 64))
     if ok:
         for other in (sdd_nt.layout, dsd_nn.layout):
             ok = ok and (other is softmax.layout or (other.shape == softmax.layout.shape and bool((other == softmax.layout).all())))
