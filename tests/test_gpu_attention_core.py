@@ -16,10 +16,12 @@ DEV = 'cuda'
 
 @pytest.fixture(autouse=True)
 def fused_on():
-    old = ac.FUSED
+    old, fill = ac.FUSED, dict(ac.MIN_TILE_FILL)
     ac.FUSED = True
+    ac.MIN_TILE_FILL.clear()               # the kernels are tested on every layout, also where the operators would be chosen
     yield
     ac.FUSED = old
+    ac.MIN_TILE_FILL.update(fill)
 
 
 def _ops(layout):
@@ -221,16 +223,27 @@ def test_modules_take_the_fused_kernels_and_agree_with_the_operators():
 def test_cases_left_to_the_three_operators():
     torch.manual_seed(7)
     Z, H, dh = 1, 2, 64
-    # a row of nine blocks: longer than the fused kernels hold in registers
+    # a row of nine blocks is streamed by the fused kernels, which then take no per-element mask: with an attention mask
+    # or a relative position embedding such a layout goes to the operators
     layout = torch.zeros(H, 10, 10, dtype=torch.int64)
     layout[:, :, 0] = 1
     layout[:, 9, :9] = 1
     ops = _ops(layout)
     q, k, v = [torch.randn(Z, H, 640, dh, device=DEV).half() for _ in range(3)]
+    am = (0.5 * torch.randn(640, 640, device=DEV)).half()
     n0 = ac.fused_calls
-    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, attn_mask=am)
     assert ac.fused_calls == n0
-    assert_close(o, D.attention(q, k, v, layout, 64, 0.125, attn_mask_mode='add'), torch.float16, 'o')
+    assert_close(o, D.attention(q, k, v, layout, 64, 0.125, attn_mask=am, attn_mask_mode='add'), torch.float16, 'o')
+    ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, rpe=am)
+    assert ac.fused_calls == n0
+    # a row of 32768 elements: the softmax operator's own bound (softmax.py:225-227)
+    layout = torch.ones(1, 1, 512, dtype=torch.int64)
+    ops = _ops(layout)
+    k = torch.randn(1, 1, 32768, dh, device=DEV).half()
+    with pytest.raises(NotImplementedError):
+        ac.attention_chain(ops[0], ops[1], ops[2], q[:, :1, :64], k, k, scale=0.125)
+    assert ac.fused_calls == n0
     # dropout, fp32, a head dimension the kernels do not have, blocks of 128
     lay = torch.tril(torch.ones(H, 4, 4)).long()
     ops = _ops(lay)
@@ -323,20 +336,112 @@ def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
     o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0
     assert_close(o, D.attention(q, k, v, lay, 16, 0.125, attn_mask_mode='add'), torch.float16, 'o')
-    # a tile-row of nine tiles
-    lay = torch.ones(H, 4, 36).long()
+    # tiles that are mostly holes: the kernels would compute them whole, the operators are chosen
+    lay = torch.zeros(H, 16, 16, dtype=torch.int64)
+    lay[:, torch.arange(16), torch.arange(16)] = 1            # one block of 16 per tile of 4 x 4
     ops = (tb.MatMul(lay, 16, 'sdd', trans_b=True), tb.Softmax(lay, 16), tb.MatMul(lay, 16, 'dsd'))
-    q = torch.randn(Z, H, 64, dh, device=DEV).half()
-    k, v = [torch.randn(Z, H, 36 * 16, dh, device=DEV).half() for _ in range(2)]
+    q, k, v = [torch.randn(Z, H, 256, dh, device=DEV).half() for _ in range(3)]
+    ac.MIN_TILE_FILL.update({16: 0.3, 32: 0.5})
     n0 = ac.fused_calls
-    ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0
+    ac.MIN_TILE_FILL.clear()
+    o2 = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
+    assert ac.fused_calls == n0 + 1
+    assert float((o.float() - o2.float()).abs().max()) <= 4e-3 * float(o.float().abs().max())
+    ac.MIN_TILE_FILL.update({16: 0.3, 32: 0.5})
     # the default block of the sparse self-attention module is 16: it takes the fused kernels
     mod = tb.SparseSelfAttention(tb.SparsityConfig(mode='fixed', block=16, stride=64, attention='unidirectional'))
     q, k, v = [torch.randn(2, 4, 512, dh, device=DEV).half() for _ in range(3)]
     n0 = ac.fused_calls
     mod(q, k, v)
     assert ac.fused_calls == n0 + 1
+
+
+@pytest.mark.parametrize('block,dtype,dh,R,C,kpm', [
+    (64, torch.float16, 64, 12, 20, None),
+    (64, torch.float16, 64, 16, 16, 'add'),
+    (64, torch.bfloat16, 128, 10, 24, 'mul'),
+    (64, torch.float16, 128, 9, 9, None),
+    (32, torch.float16, 64, 16, 40, 'add'),
+    (16, torch.bfloat16, 64, 24, 80, 'mul'),
+    (16, torch.float16, 128, 16, 48, None),
+])
+def test_rows_longer_than_eight_tiles_are_streamed(block, dtype, dh, R, C, kpm):
+    """Rows of 9 .. 24 tiles beside short and empty ones: two-sweep forward, block-by-block backward; key-padding masks
+    in both modes, among them a whole masked tile in the middle of a row (its maximum so far stays where it was) and
+    one at the start (the running maximum starts at -inf)."""
+    torch.manual_seed(R + C + block)
+    Z, H = 2, 2
+    lay = (torch.rand(H, R, C) < 0.7).long()
+    lay[:, 0, :] = 1                       # the longest row the layout allows
+    lay[:, 1, :] = 0
+    lay[:, 1, C - 1] = 1                   # a row of one block (which the masks below leave alone)
+    lay[0, 2, :] = 0                       # an empty row in one head
+    S = 64 // block
+    assert int(lay.view(H, R // S, S, C // S, S).sum((2, 4)).ne(0).sum(2).max()) > 8
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.Softmax(lay, block), tb.MatMul(lay, block, 'dsd'))
+    q, do = [torch.randn(Z, H, R * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    k, v = [torch.randn(Z, H, C * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    kw = dict(scale=dh ** -0.5)
+    if kpm == 'add':
+        m = 0.5 * torch.randn(Z, C * block)
+        m[0, 128:200] = float('-inf')
+        m[1, :70] = float('-inf')
+        kw.update(key_padding_mask=m.to(DEV).to(dtype), key_padding_mask_mode='add')
+    if kpm == 'mul':
+        m = torch.ones(Z, C * block)
+        m[0, :64] = 0
+        m[1, 190:330] = 0
+        kw.update(key_padding_mask=m.to(DEV).to(dtype), key_padding_mask_mode='mul')
+    with guard_allocations('fused attention, long rows'):
+        got = _run(ops, q, k, v, do, True, **kw)
+    chain = _run(ops, q, k, v, do, False, **kw)
+    tol = CHAIN_TOL[dtype]
+    for name, g, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
+        assert not bool(torch.isnan(g).any()), name
+        assert float((g.float() - c.float()).abs().max()) <= tol[0 if name in ('o', 'dv') else 1] * float(c.float().abs().max()), name
+    live = lay.sum(2).ne(0).all(0)
+    rows = live.repeat_interleave(block).to(DEV)
+    okw = {n: kw[n] for n in ('key_padding_mask', 'key_padding_mask_mode') if n in kw}
+    ref = D.attention(q[:, :, rows], k, v, lay[:, live], block, kw['scale'], do=do[:, :, rows], attn_mask_mode='add', **okw)
+    assert_close(got[0][:, :, rows], ref[0], dtype, 'o')
+    assert_close(got[1][:, :, rows], ref[1], dtype, 'dq')
+
+
+def test_streamed_rows_that_are_masked_everywhere_give_nan_like_the_operators():
+    torch.manual_seed(11)
+    Z, H, R, C, dh = 1, 1, 2, 12, 64
+    lay = torch.ones(H, R, C, dtype=torch.int64)
+    ops = _ops(lay)
+    q = torch.randn(Z, H, R * 64, dh, device=DEV).half()
+    k, v = [torch.randn(Z, H, C * 64, dh, device=DEV).half() for _ in range(2)]
+    m = torch.full((Z, C * 64), float('-inf'), device=DEV).half()
+    ac.FUSED = True
+    n0 = ac.fused_calls
+    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, key_padding_mask=m)
+    assert ac.fused_calls == n0 + 1
+    ac.FUSED = False
+    c = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, key_padding_mask=m)
+    assert bool(torch.isnan(o).all()) and bool(torch.isnan(c).all())
+
+
+def test_streamed_backward_is_reproducible_at_full_occupancy():
+    """Dense attention over 2048 keys (32 tiles a row), enough workgroups to fill every compute unit several times: the
+    tile ring is reused under load; the same inputs give the same bits."""
+    torch.manual_seed(13)
+    Z, H, R, dh = 4, 8, 32, 64
+    lay = torch.ones(H, R, R, dtype=torch.int64)
+    ops = _ops(lay)
+    q, k, v, do = [torch.randn(Z, H, R * 64, dh, device=DEV).half() for _ in range(4)]
+    first = _run(ops, q, k, v, do, True, scale=0.125)
+    for _ in range(4):
+        again = _run(ops, q, k, v, do, True, scale=0.125)
+        for a, b in zip(first, again):
+            assert torch.equal(a, b)
+    chain = _run(ops, q, k, v, do, False, scale=0.125)
+    for name, g, c in zip(('o', 'dq', 'dk', 'dv'), first, chain):
+        assert float((g.float() - c.float()).abs().max()) <= CHAIN_TOL[torch.float16][1] * float(c.float().abs().max()), name
 
 
 def test_c_abi_argument_checks():
@@ -347,17 +452,19 @@ def test_c_abi_argument_checks():
     null = ctypes.c_void_p(0)
     st = (t.stride(0), t.stride(1), t.stride(2))
 
-    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64, tiles=null):
+    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64, tiles=null, rpe=null):
         return lib.bsp_attention_fwd(dtype, _lib.ptr(q), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(t.clone()), 1, 1, 1, D,
                                      st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut, tiles,
-                                     null, 0, 0, 0, null, 0, 0, null, 0, 0, _lib.stream_ptr(torch.device(DEV)))
+                                     rpe, 0, 0, 64, null, 0, 0, null, 0, 0, _lib.stream_ptr(torch.device(DEV)))
     assert fwd() == _lib.OK
     assert fwd(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
     assert fwd(block=128) == _lib.ERR_UNSUPPORTED
     assert fwd(block=32) != _lib.OK                     # small blocks need the tile table
     assert fwd(tiles=_lib.ptr(lut)) != _lib.OK          # ... and blocks of 64 take none
     assert fwd(D=96) == _lib.ERR_UNSUPPORTED
-    assert fwd(maxlut=9) == _lib.ERR_ROW_TOO_LONG
+    assert fwd(maxlut=9) == _lib.OK                     # (the streaming kernels; the table's rows hold one block)
+    assert fwd(maxlut=9, rpe=_lib.ptr(t)) == _lib.ERR_ROW_TOO_LONG
+    assert fwd(maxlut=512) == _lib.ERR_ROW_TOO_LONG
     assert fwd(ldq=60) != _lib.OK                       # a row stride that is not a multiple of 8 elements
     assert fwd(q=None) != _lib.OK
     torch.cuda.synchronize()

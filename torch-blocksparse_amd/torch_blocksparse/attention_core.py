@@ -17,8 +17,12 @@ from .matmul import MatMul, _LayoutOnDevice
 from .softmax import Softmax, _sparse_softmax
 
 FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
-MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS
+MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS: longer rows are streamed
 fused_calls = 0             # forward calls that took the fused kernels; tests read it
+# Blocks of 16 and 32 are computed as whole 64 x 64 tiles: a tile costs the same however few of its blocks exist, so
+# below this share of present blocks per present tile the three operators (whose work follows the blocks) are faster.
+# Measured break-even points on MI355X, fwd + bwd, head dimension 64, rows of 8 tiles and of 30+ tiles.
+MIN_TILE_FILL = {16: 0.3, 32: 0.5}
 
 
 def _vec_ok(t):
@@ -50,26 +54,27 @@ class AttentionCore:
         return self.nnz
 
     def tables(self, device):
-        """(table, longest row, tile table or None, rows of the table's layout) on `device`, or None when the layout does
-        not divide into 64 x 64 tiles."""
+        """(table, longest row, tile table or None, rows of the table's layout, present blocks per present tile as a share)
+        on `device`, or None when the layout does not divide into 64 x 64 tiles."""
         key = str(device)
         if key not in self._tables:
             S = 64 // self.block
             H, R, C = self.spdims
             if S == 1:
                 lut, maxlut = self.softmax.make_lut(device)
-                self._tables[key] = (lut, maxlut, None, R)
+                self._tables[key] = (lut, maxlut, None, R, 1.)
             elif R % S or C % S:
                 self._tables[key] = None
             else:
                 cctx, ids = _LayoutOnDevice(self.layout, device).coarse(S)
                 lut, maxlut = _sparse_softmax.make_lut(cctx.lay, 64, device)
-                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S)
+                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S, self.blocks() / max(1, ids.numel()))
         return self._tables[key]
 
-    def usable(self, q, k, v, dropout_p=0.):
+    def usable(self, q, k, v, dropout_p=0., per_element_masks=False):
         """Can this call take the fused kernels?  (Shapes that do not fit the layout are left to the operators, which
-        raise the reference's errors.)"""
+        raise the reference's errors.)  Rows of more than MAX_ROW_BLOCKS tiles go to the streaming kernels, which take
+        neither a relative position embedding nor an attention mask (`per_element_masks`)."""
         if not FUSED or self.block not in (16, 32, 64) or dropout_p:
             return False
         if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
@@ -81,14 +86,16 @@ class AttentionCore:
         if tuple(q.shape) != (Z, H, R * b, D) or tuple(k.shape) != (Z, H, C * b, D) or tuple(v.shape) != (Z, H, C * b, D):
             return False
         t = self.tables(q.device)
-        return t is not None and 0 < t[1] <= MAX_ROW_BLOCKS
+        if t is None or t[1] <= 0 or t[4] < MIN_TILE_FILL.get(b, 0.):
+            return False
+        return t[1] <= MAX_ROW_BLOCKS or (not per_element_masks and t[1] * 64 < 32768)
 
     def __call__(self, q, k, v, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
                  key_padding_mask_mode='add', attn_mask_mode='add'):
         for name, m in (('relative position embedding', rpe), ('Attention mask', attn_mask), ('Key padding mask', key_padding_mask)):
             if m is not None and m.dtype != q.dtype:      # softmax.py:348-353
                 raise ValueError('%s must be %s' % (name, q.dtype))
-        lut, maxlut, tiles, rows = self.tables(q.device)
+        lut, maxlut, tiles, rows = self.tables(q.device)[:4]
         return _attention_core.apply(q, k, v, float(scale), rpe, key_padding_mask, attn_mask, key_padding_mask_mode,
                                      attn_mask_mode, self, lut, maxlut, tiles, rows)
 
@@ -180,7 +187,7 @@ def attention_chain(sdd_nt, softmax, dsd_nn, q, k, v, scale=1., rpe=None, key_pa
                     key_padding_mask_mode='add', attn_mask_mode='add', dropout_p=0.):
     """dsd_nn(softmax(sdd_nt(q, k), ...), v): fused when the operators and tensors allow it, else the three calls."""
     core = _core_for(sdd_nt, softmax, dsd_nn)
-    if core is not None and core.usable(q, k, v, dropout_p):
+    if core is not None and core.usable(q, k, v, dropout_p, rpe is not None or attn_mask is not None):
         return core(q, k, v, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode)
     w = sdd_nt(q, k)
     kwargs = dict(dropout_p=dropout_p) if dropout_p else {}
