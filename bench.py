@@ -260,8 +260,9 @@ def main():
                 e1.synchronize()
                 return e0.elapsed_time(e1) / reps
             out['fused_attention_chain'] = {
-                'what': 'attention_chain(sdd, softmax, dsd, q, k, v): bsp_attention_fwd, then in the backward pass dsd (p^T.do), '
-                        'bsp_attention_bwd, dsd (ds^T.q); same workload, same flop count',
+                'what': 'attention_chain(sdd, softmax, dsd, q, k, v): bsp_attention_fwd, then in the backward pass bsp_attention_bwd (dq) '
+                        'and bsp_attention_bwd_kv (dk, dv; the softmax gradient is computed twice and never stored); same workload, '
+                        'flop count of the six products of the three-operator chain',
                 'ms_per_step': round(ms_fused, 4), 'TFLOP/s': round(6 * w.flops_mm / ms_fused * 1e-9, 3),
                 'vs_three_operators': round(ms_per_step / ms_fused, 3),
                 'launches': fused_chain_launches(w.lay, w.q.detach(), w.k.detach(), w.v.detach(), w.do, w.scale, timeit,
@@ -408,7 +409,7 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants, block=64):
     """The fused attention kernels (bsp_attention_fwd / bsp_attention_bwd: what the attention modules launch instead of
     sdd -> softmax -> dsd when block, dtype and head dimension allow), each timed on its own through the C ABI.
     variants: [(label, softmax keyword arguments)] for the forward kernel.  Algorithmic bytes: forward q, k, v, o and
-    the sparse p once each; backward do, o, v, k, dq and the sparse p and ds once each (masks: what the layout touches
+    the sparse p once each; backward rows do, o, v, k, dq and the sparse p once each, backward columns do, q, v, dk, dv and p (masks: what the layout touches
     is counted by the caller's softmax figures, not here)."""
     import torch
     from torch_blocksparse import attention_core as ac
@@ -430,15 +431,25 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants, block=64):
         out.append({'launch': 'fused forward: q.k^T, softmax, p.v (%s)' % label, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
                     'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_fwd', 0, nbytes, ms)})
     ctx = state['ctx']
-    ctx.needs_input_grad = (True, False, False)      # the kernel alone: dk and dv are the two dsd launches listed with the operators
+    delta = torch.empty((B, H, ctx.rows * 64), dtype=torch.float32, device=q.device)
 
-    def bwd():
+    def rows():
         with torch.no_grad():
-            ac._attention_core.backward(ctx, do)
-    ms = timeit(bwd)
-    nbytes = 5 * dense + 2 * xb
-    out.append({'launch': 'fused backward: do.v^T, softmax gradient, ds.k', 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
+            ac._attention_core.rows_kernel(ctx, do, None, delta)
+    ms = timeit(rows)
+    nbytes = 5 * dense + xb
+    out.append({'launch': 'fused backward, rows: do.v^T, softmax gradient, ds.k -> dq', 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
                 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_bwd', 0, nbytes, ms)})
+
+    def columns():
+        with torch.no_grad():
+            ac._attention_core.columns_kernel(ctx, do, delta)
+    ms = timeit(columns)
+    ct = ctx.columns
+    nbytes = 5 * dense + xb + 2 * B * ct.n_slots * 2 * 64 * dh * 4      # (the partial sums of the long columns' parts: written, read)
+    out.append({'launch': 'fused backward, columns: softmax gradient again, p^T.do -> dv, ds^T.q -> dk (%d of %d columns in parts)' % (ct.n_split, H * ct.columns),
+                'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
+                'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_bwd_kv', 0, nbytes, ms)})
     return out
 
 
@@ -841,9 +852,10 @@ def record_traffic(fetch_dir, write_dir):
         ('k_sdd64_rg', ('k_sdd64_rg',)), ('k_xsd64_rg<sparse operand as stored>', ('k_xsd64_rg', 'Lb0E')),
         ('k_xsd64_rg<sparse operand transposed>', ('k_xsd64_rg', 'Lb1E')), ('k_softmax_fwd', ('k_softmax_fwd',)),
         ('k_softmax_bwd', ('k_softmax_bwd',)))}
-    for name in ('k_attn64_fwd', 'k_attn64_bwd'):          # the fused chain of the attention modules, run after the headline step
-        if any(name in k for k in fetch) and any(name in k for k in write):
-            per_kernel[name] = kernel_bytes(name, name)
+    for name in ('k_attn64_fwd', 'k_attn64_bwd', 'k_attn64_bwd_kv'):   # the fused chain of the attention modules, run after the headline step
+        for sub in (name + 'I', name + '<'):               # (the template's name as mangled or as written: k_attn64_bwd is not k_attn64_bwd_kv)
+            if any(sub in k for k in fetch) and any(sub in k for k in write):
+                per_kernel[name] = kernel_bytes(name, sub)
     rec = {'kernel_sources_sha256': kernel_sources_sha(), 'bytes_per_counted_KiB': {'FETCH_SIZE': round(fs, 1), 'WRITE_SIZE': round(ws, 1)},
            'bytes_per_kernel_launch': per_kernel, 'counters_per_kernel_launch': split,
            'bytes_per_launch': {name: per_kernel[k] for name, k in KERNEL_OF.items()},

@@ -287,7 +287,9 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  *   backward: ds = p * (round(do . v^T) - delta) * scale, dq = ds . k, with delta = sum_d do[row][d] * o[row][d], o
  *             the result of the forward call: in exact arithmetic this is the sum over the row of p * (do . v^T) that
  *             the softmax gradient subtracts (softmax.py:187-189), and it is known before the row's blocks are, so
- *             each block is finished as soon as its product is.  ds: [Z, nnz, block, block], a tensor of its own.
+ *             each block is finished as soon as its product is.  ds: [Z, nnz, block, block], a tensor of its own, or
+ *             NULL (not stored); delta: NULL, or [Z][H][delta_stride_h >= 64 R] fp32 that receives delta of every row
+ *             that has a block.
  *             The two remaining gradients are ordinary products of the caller: dk = ds^T . q and dv = p^T . do
  *             (bsp_dsd_matmul with trans_a).
  * round() is the rounding to the storage type that the scores undergo when the sdd operator stores them, kept so
@@ -306,7 +308,27 @@ int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, 
                       int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                       int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                       int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                      const int32_t *d_lut, int maxlut, const int32_t *d_tiles, void *stream);
+                      const int32_t *d_lut, int maxlut, const int32_t *d_tiles, float *delta, int64_t delta_stride_h,
+                      void *stream);
+/* dk and dv of the same chain in one launch, one workgroup per column of 64 x 64 tiles: dv = p^T . do and
+ * dk = ds^T . q with ds computed again from p (the formula above), delta = the row sums that bsp_attention_bwd wrote
+ * ([Z][H][delta_stride_h], fp32).  Call bsp_attention_bwd with ds = NULL and delta given first: the sparse gradient
+ * is then neither written nor read.  Replaces the two transposed dsd products of the operators' backward pass
+ * (matmul.py:598-601).  d_col_lut: the layout (coarsened to tiles for blocks of 16 / 32, as d_lut) read along columns:
+ * n_items work items of eight ints (number of blocks, offset of the first entry in ints from the start, head, column,
+ * slot, 0, 0, 0), then per block four ints (id, row, column, head), the blocks of a column by row.  A work item is a
+ * whole column (slot -1; also every column without blocks, whose rows of dk and dv are set to zero) or one part of a
+ * long column: columns differ in length far more than rows do, so the caller cuts the long ones into parts, whose
+ * partial sums go to fp32 slots (partial: [Z][n_slots][2][64][D] floats, slot = the item's) and are added in order by a
+ * second kernel of the same call, per d_split_lut: n_split entries of four ints (head, column, first slot, parts; a
+ * column's slots are consecutive).  No atomics.  C = columns; dk, dv: [Z, H, columns, D]. */
+int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, const void *v, const void *p, const float *delta, void *dk,
+                         void *dv, int Z, int H, int C, int D, int64_t do_stride_z, int64_t do_stride_h, int64_t lddo,
+                         int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t v_stride_z, int64_t v_stride_h,
+                         int64_t ldv, int64_t dk_stride_z, int64_t dk_stride_h, int64_t lddk, int64_t dv_stride_z,
+                         int64_t dv_stride_h, int64_t lddv, int64_t p_stride_z, int64_t delta_stride_h, int block,
+                         float scale, const int32_t *d_col_lut, int n_items, const int32_t *d_tiles, float *partial,
+                         int n_slots, const int32_t *d_split_lut, int n_split, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Dense utility ops of the reference package.

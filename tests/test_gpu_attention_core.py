@@ -444,6 +444,61 @@ def test_streamed_backward_is_reproducible_at_full_occupancy():
         assert float((g.float() - c.float()).abs().max()) <= CHAIN_TOL[torch.float16][1] * float(c.float().abs().max()), name
 
 
+@pytest.mark.parametrize('block,dh,dtype', [(64, 64, torch.float16), (64, 128, torch.bfloat16), (16, 64, torch.float16), (32, 128, torch.float16)])
+def test_backward_through_the_column_kernel_and_through_the_two_operators(block, dh, dtype):
+    """dk and dv from the column kernel (the default) against the stored softmax gradient and the two transposed dsd
+    operators; a layout whose global columns are cut into parts (every size of part from 1 block on) beside short and
+    empty columns, keys longer than queries."""
+    torch.manual_seed(block + dh)
+    Z, H = 2, 3
+    S = 64 // block
+    R, C = 40 * S, 44 * S
+    lay = torch.zeros(H, R, C, dtype=torch.int64)
+    for r in range(R):
+        lay[:, r, max(0, r - 2 * S):r + 1] = 1            # a band
+    lay[:, :, 0] = 1                                     # a global column: 40 tiles
+    lay[1, 3 * S:, 5 * S] = 1                            # 37 tiles in one head
+    lay[:, :, C - 2 * S:] = 0                            # columns without blocks
+    lay[2, 17 * S:, :] = 0                               # a head whose later rows are empty
+    if S > 1:
+        lay[:, 1::2, 1::3] = 0                           # holes inside the tiles
+        lay[:, :, 0] = 1
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.Softmax(lay, block), tb.MatMul(lay, block, 'dsd'))
+    core = ac._core_for(*ops)
+    ct = core.tables(torch.device(DEV))[5]
+    assert ct.n_split >= H and ct.n_slots > ct.n_split
+    q, do = [torch.randn(Z, H, R * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    k, v = [torch.randn(Z, H, C * block, dh, device=DEV).to(dtype) for _ in range(2)]
+    kpm = torch.zeros(Z, C * block)
+    kpm[1, 100:180] = float('-inf')
+    kw = dict(scale=dh ** -0.5, key_padding_mask=kpm.to(DEV).to(dtype))
+    old = ac.FUSED_KV
+    try:
+        ac.FUSED_KV = True
+        with guard_allocations('fused attention, column kernel'):
+            got = _run(ops, q, k, v, do, True, **kw)
+        again = _run(ops, q, k, v, do, True, **kw)
+        ac.FUSED_KV = False
+        stored = _run(ops, q, k, v, do, True, **kw)
+    finally:
+        ac.FUSED_KV = old
+    chain = _run(ops, q, k, v, do, False, **kw)
+    tol = CHAIN_TOL[dtype]
+    for name, g, a2, s2, c in zip(('o', 'dq', 'dk', 'dv'), got, again, stored, chain):
+        assert torch.equal(g, a2), name                  # parts are summed in a fixed order
+        assert not bool(torch.isnan(g).any()), name
+        ref = float(c.float().abs().max())
+        assert float((g.float() - s2.float()).abs().max()) <= tol[0] * ref, name
+        assert float((g.float() - c.float()).abs().max()) <= tol[0 if name in ('o', 'dv') else 1] * ref, name
+    assert torch.equal(got[0], stored[0]) and torch.equal(got[1], stored[1])      # o and dq do not depend on the choice
+    assert not bool(got[2][:, :, (C - 2 * S) * block:].any()) and not bool(got[3][:, :, (C - 2 * S) * block:].any())
+    live = lay.sum(2).ne(0).all(0)
+    if bool(live.all()):
+        ref = D.attention(q, k, v, lay, block, kw['scale'], do=do, key_padding_mask=kw['key_padding_mask'], attn_mask_mode='add')
+        for name, g, r in zip(('o', 'dq', 'dk', 'dv'), got, ref):
+            assert_close(g, r, dtype, name)
+
+
 def test_c_abi_argument_checks():
     lib = _lib.load()
     t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
@@ -467,4 +522,22 @@ def test_c_abi_argument_checks():
     assert fwd(maxlut=512) == _lib.ERR_ROW_TOO_LONG
     assert fwd(ldq=60) != _lib.OK                       # a row stride that is not a multiple of 8 elements
     assert fwd(q=None) != _lib.OK
+    # the column kernel of the backward pass
+    ct = ac._ColumnTable(torch.ones(1, 1, 1, dtype=torch.int64), torch.device(DEV))
+    delta = torch.zeros(1, 1, 64, device=DEV)
+    dk, dv = t.clone(), t.clone()
+
+    def kv(dtype=0, D=64, block=64, n_items=ct.n_items, lddk=64, delta=delta, n_slots=0, partial=null, tiles=null):
+        return lib.bsp_attention_bwd_kv(dtype, _lib.ptr(t), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(delta), _lib.ptr(dk), _lib.ptr(dv),
+                                        1, 1, 1, D, *st, *st, *st, st[0], st[1], lddk, *st, p.stride(0), 64, block, 1.0, _lib.ptr(ct.items), n_items,
+                                        tiles, partial, n_slots, null, 0, _lib.stream_ptr(torch.device(DEV)))
+    assert kv() == _lib.OK
+    assert kv(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
+    assert kv(D=96) == _lib.ERR_UNSUPPORTED
+    assert kv(block=128) == _lib.ERR_UNSUPPORTED
+    assert kv(block=16) != _lib.OK                      # small blocks need the tile table
+    assert kv(n_items=0) != _lib.OK                     # fewer work items than columns
+    assert kv(lddk=60) != _lib.OK
+    assert kv(delta=None) != _lib.OK
+    assert kv(n_slots=2) != _lib.OK                     # slots without a place for them and without the list of their columns
     torch.cuda.synchronize()

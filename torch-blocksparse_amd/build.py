@@ -14,7 +14,7 @@ LIBDIR = os.path.join(HERE, 'lib')
 OBJDIR = os.path.join(HERE, 'build')
 LIBNAME = 'libbsp_hip.so'
 PROBE_LIBNAME = 'libbsp_probe.so'
-SOURCES = ['lut.hip', 'layout.hip', 'softmax.hip', 'softmax_row.hip', 'attention_core.hip', 'attention_long.hip', 'matmul_f16.hip', 'matmul_bf16.hip', 'matmul_f32.hip', 'matmul_fast64.hip', 'matmul_dl.hip', 'elementwise.hip', 'capi.hip']
+SOURCES = ['lut.hip', 'layout.hip', 'softmax.hip', 'softmax_row.hip', 'attention_core.hip', 'attention_long.hip', 'attention_kv.hip', 'matmul_f16.hip', 'matmul_bf16.hip', 'matmul_f32.hip', 'matmul_fast64.hip', 'matmul_dl.hip', 'elementwise.hip', 'capi.hip']
 FLAGS = ['--offload-arch=gfx950', '-O3', '-std=c++17', '-fPIC', '-fno-gpu-rdc', '-Wall', '-Wno-unused-function',
          # packed-fp32 instruction selection is switched off on purpose
          '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops']

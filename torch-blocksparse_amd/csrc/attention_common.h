@@ -14,6 +14,13 @@ struct AttnArgs {
   const void *p_in;          // backward: the saved softmax
   void *p_out, *o;           // forward: p, o; backward: ds, dq
   const void *o_in;          // backward: the forward result o
+  float *delta;              // backward: sum_d do . o of every row, [Z][H] rows delta_sh apart (row kernels write it when given, the column kernel reads it)
+  int64_t delta_sh;
+  void *o2;                  // column kernel of the backward pass: dv (o is dk)
+  int64_t o2_sz, o2_sh, o2_ld;
+  float *partial;            // ... the slots of the long columns' parts, [Z][n_slots][dk, dv][64][D]
+  const int32_t *split_lut;  // ... per long column (head, column, first slot, parts)
+  int n_slots, n_split;
   const int32_t *tiles;      // blocks of 16 / 32: per 64 x 64 tile of the layout the ids of its blocks (-1: absent), see bsp_attention_fwd
   int64_t oin_sz, oin_sh, oin_ld;
   int64_t x_sz, x_sh, x_ld, y1_sz, y1_sh, y1_ld, y2_sz, y2_sh, y2_ld, o_sz, o_sh, o_ld, pin_sz, pout_sz;
@@ -169,8 +176,39 @@ __device__ __forceinline__ void wait_vm(int c) {
 }
 
 
-// rows of more than BSP_ATTENTION_MAX_ROW_BLOCKS tiles (attention_long.hip); no relative position embedding, no attention mask
+// Two fragments of the same kind (see tr_frags4).
+template <typename T, int HI>
+__device__ __forceinline__ void tr_frags2(typename Mma16<T>::frag_t (&f)[2], uint32_t a0, uint32_t a1) {
+  s16x4 lo0, hi0, lo1, hi1;
+  asm volatile(
+      "ds_read_b64_tr_b16 %0, %4\n\t"
+      "ds_read_b64_tr_b16 %1, %4 offset:%6\n\t"
+      "ds_read_b64_tr_b16 %2, %5\n\t"
+      "ds_read_b64_tr_b16 %3, %5 offset:%6\n\t"
+      "s_waitcnt lgkmcnt(0)"
+      : "=&v"(lo0), "=&v"(hi0), "=&v"(lo1), "=&v"(hi1)
+      : "v"(a0), "v"(a1), "n"(HI));
+  typedef short s16x8 __attribute__((ext_vector_type(8)));
+  typedef typename Mma16<T>::frag_t frag_t;
+  f[0] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo0, hi0, 0, 1, 2, 3, 4, 5, 6, 7));
+  f[1] = __builtin_bit_cast(frag_t, (s16x8)__builtin_shufflevector(lo1, hi1, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// A tile that is read both ways (16-byte reads along a row and transposing reads): the swizzle of the second product
+// with the two halves of a pair exchanged in rows with bit 4 set.  The transposing reads take whole pairs and do not
+// notice; of the sixteen rows of a 16-byte read (bits 0, 1, 3, 4 differ) the pair swizzle separates four and the
+// exchanged halves the other two, so that these are free of bank conflicts as well.
+template <int D> __device__ __forceinline__ int dual_slot(int r, int chunk) {
+  return ((((chunk >> 1) ^ swz_second<D>(r)) << 1) | ((chunk & 1) ^ ((r >> 4) & 1)));
+}
+template <int D> __device__ __forceinline__ int dual_offset(int r, int col) {   // col in elements
+  return r * (2 * D) + (dual_slot<D>(r, col >> 3) << 4) + ((col & 7) << 1);
+}
+
 }  // namespace
+// rows of more than BSP_ATTENTION_MAX_ROW_BLOCKS tiles (attention_long.hip); no relative position embedding, no attention mask
 int attention_long(int dtype, const AttnArgs &a, int D, int block, bool bwd, hipStream_t st);
+// dk and dv, one workgroup per column of tiles (attention_kv.hip)
+int attention_kv(int dtype, const AttnArgs &a, int D, int block, hipStream_t st);
 }  // namespace bsp
 #endif

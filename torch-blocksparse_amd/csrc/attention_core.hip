@@ -492,6 +492,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
     for (int i = 0; i < 8; i++) delta = fmaf(to_float(xq[s2][i]), to_float(oq[s2][i]), delta);
   delta += __shfl_xor(delta, 16);
   delta += __shfl_xor(delta, 32);
+  if (a.delta != nullptr && q == 0) a.delta[((int64_t)z * a.H + h) * a.delta_sh + row] = delta;   // for the column kernel
 
   frag_t pf[NB][2];
   const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
@@ -560,6 +561,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
   store_rows<T, D>(cs, po, a.o_ld, o, lane);
+  if (a.p_out == nullptr) return;   // ds is not asked for (the column kernel computes it again)
 #pragma unroll
   for (int b = 0; b < NB; b++)
     if (b < size) {
@@ -611,7 +613,7 @@ template <typename T> int launch_t(const AttnArgs &a, int D, int block, int maxl
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *stream) {
-  if (!a.x || !a.y1 || !a.y2 || !a.p_out || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
+  if (!a.x || !a.y1 || !a.y2 || (!bwd && !a.p_out) || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
     return BSP_ERR_ARG;
   if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
   if ((block != 64) != (a.tiles != nullptr)) return BSP_ERR_ARG;   // the tile table goes with the small blocks, and only with them
@@ -627,6 +629,7 @@ int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *st
   for (int64_t s : strides)
     if (s % 8) return BSP_ERR_ARG;
   if (a.x_ld < D || a.y1_ld < D || a.y2_ld < D || a.o_ld < D || (bwd && a.oin_ld < D)) return BSP_ERR_ARG;
+  if (a.delta != nullptr && ((reinterpret_cast<uintptr_t>(a.delta) & 3) || a.delta_sh < (int64_t)a.R * 64)) return BSP_ERR_ARG;
   if ((int64_t)a.Z * a.H * a.R >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
   int rc;
   if (is_long) rc = attention_long(dtype, a, D, block, bwd, as_stream(stream));
@@ -669,9 +672,11 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
                                  int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                                  int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                                  int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                                 const int32_t *d_lut, int maxlut, const int32_t *d_tiles, void *stream) {
+                                 const int32_t *d_lut, int maxlut, const int32_t *d_tiles, float *delta, int64_t delta_stride_h,
+                                 void *stream) {
   AttnArgs a{};
   a.x = d_o; a.y1 = v; a.y2 = k; a.p_in = p; a.p_out = ds; a.o = dq;
+  a.delta = delta; a.delta_sh = delta_stride_h;
   a.o_in = o; a.oin_sz = o_stride_z; a.oin_sh = o_stride_h; a.oin_ld = ldo;
   a.x_sz = do_stride_z; a.x_sh = do_stride_h; a.x_ld = lddo;
   a.y1_sz = v_stride_z; a.y1_sh = v_stride_h; a.y1_ld = ldv;
@@ -681,4 +686,47 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
   a.scale = scale; a.lut = d_lut; a.tiles = d_tiles;
   a.Z = Z; a.H = H; a.R = R;
   return run(dtype, a, D, block, maxlut, true, stream);
+}
+
+extern "C" int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, const void *v, const void *p, const float *delta,
+                                    void *dk, void *dv, int Z, int H, int C, int D, int64_t do_stride_z, int64_t do_stride_h,
+                                    int64_t lddo, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t v_stride_z,
+                                    int64_t v_stride_h, int64_t ldv, int64_t dk_stride_z, int64_t dk_stride_h, int64_t lddk,
+                                    int64_t dv_stride_z, int64_t dv_stride_h, int64_t lddv, int64_t p_stride_z,
+                                    int64_t delta_stride_h, int block, float scale, const int32_t *d_col_lut, int n_items,
+                                    const int32_t *d_tiles, float *partial, int n_slots, const int32_t *d_split_lut,
+                                    int n_split, void *stream) {
+  if (!d_o || !q || !v || !p || !delta || !dk || !dv || !d_col_lut || Z <= 0 || H <= 0 || C <= 0 || delta_stride_h < 0 || n_items < H * C)
+    return BSP_ERR_ARG;
+  if (n_slots < 0 || n_split < 0 || (n_slots > 0) != (n_split > 0) || (n_slots > 0 && (!partial || !d_split_lut)) || n_items > H * C + n_slots)
+    return BSP_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(partial) & 15) return BSP_ERR_ARG;
+  if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
+  if ((block != 64) != (d_tiles != nullptr)) return BSP_ERR_ARG;
+  const void *ptrs[] = {d_o, q, v, p, dk, dv};
+  for (const void *ptr : ptrs)
+    if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0) return BSP_ERR_ARG;
+  if (reinterpret_cast<uintptr_t>(delta) & 3) return BSP_ERR_ARG;
+  const int64_t strides[] = {do_stride_z, do_stride_h, lddo, q_stride_z, q_stride_h, ldq, v_stride_z, v_stride_h, ldv,
+                             dk_stride_z, dk_stride_h, lddk, dv_stride_z, dv_stride_h, lddv, p_stride_z};
+  for (int64_t s : strides)
+    if (s % 8) return BSP_ERR_ARG;
+  if (lddo < D || ldq < D || ldv < D || lddk < D || lddv < D) return BSP_ERR_ARG;
+  if ((int64_t)Z * n_items >= ((int64_t)1 << 31) || (int64_t)Z * n_split * 4 >= ((int64_t)1 << 31)) return BSP_ERR_UNSUPPORTED;
+  AttnArgs a{};
+  a.x = v; a.y1 = d_o; a.y2 = q; a.p_in = p; a.o = dk; a.o2 = dv;
+  a.partial = partial; a.n_slots = n_slots; a.split_lut = d_split_lut; a.n_split = n_split;
+  a.delta = const_cast<float *>(delta); a.delta_sh = delta_stride_h;
+  a.x_sz = v_stride_z; a.x_sh = v_stride_h; a.x_ld = ldv;
+  a.y1_sz = do_stride_z; a.y1_sh = do_stride_h; a.y1_ld = lddo;
+  a.y2_sz = q_stride_z; a.y2_sh = q_stride_h; a.y2_ld = ldq;
+  a.o_sz = dk_stride_z; a.o_sh = dk_stride_h; a.o_ld = lddk;
+  a.o2_sz = dv_stride_z; a.o2_sh = dv_stride_h; a.o2_ld = lddv;
+  a.pin_sz = p_stride_z;
+  a.scale = scale; a.lut = d_col_lut; a.tiles = d_tiles;
+  a.Z = Z; a.H = H; a.R = n_items;
+  const int rc = attention_kv(dtype, a, D, block, as_stream(stream));
+  if (rc != BSP_OK) return rc;
+  BSP_LAUNCH_CHECK();
+  return BSP_OK;
 }

@@ -142,6 +142,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
     for (int i = 0; i < 8; i++) delta = fmaf(to_float(xq[s2][i]), to_float(oq[s2][i]), delta);
   delta += __shfl_xor(delta, 16);
   delta += __shfl_xor(delta, 32);
+  if (a.delta != nullptr && q == 0) a.delta[((int64_t)z * a.H + h) * a.delta_sh + row] = delta;   // for the column kernel
 
   const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
   const int prow = wave * 16 + qrow, pswz = (prow >> 1) & 7;
@@ -198,7 +199,8 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) o[j4 + j] = M::run(vf[j], pf[s], o[j4 + j]);
       }
-    if constexpr (SUBS == 1) {
+if (a.p_out == nullptr) continue;   // ds is not asked for
+        if constexpr (SUBS == 1) {
       store_block_rows<T>(stage_p, pz + (int64_t)tile_id * 4096 + wave * 1024, __builtin_bit_cast(u32x4, pf[0]), __builtin_bit_cast(u32x4, pf[1]), lane);
     } else {
 #pragma unroll

@@ -23,6 +23,55 @@ fused_calls = 0             # forward calls that took the fused kernels; tests r
 # below this share of present blocks per present tile the three operators (whose work follows the blocks) are faster.
 # Measured break-even points on MI355X, fwd + bwd, head dimension 64, rows of 8 tiles and of 30+ tiles.
 MIN_TILE_FILL = {16: 0.3, 32: 0.5}
+# dk and dv from the column kernel (bsp_attention_bwd_kv), which computes the softmax gradient again instead of reading it;
+# False: the row kernel stores the gradient and the two products are ordinary dsd operators
+FUSED_KV = os.environ.get('BSP_FUSED_ATTENTION_KV', '1') != '0'
+
+
+KV_PART_BLOCKS = 16         # columns of more blocks than this (and than twice the average column) are computed in parts of about this size
+
+
+class _ColumnTable:
+    """The tables of the column kernel: the layout read along columns, cut into work items.
+    items: per item (blocks, offset of its entries, head, column, slot of its partial sums or -1, 0, 0, 0), then per block
+    (id, row, column, head), a column's blocks by row; the ids are the positions in the row-major order of the nonzero
+    blocks, as everywhere.  A column of more than `part` blocks is cut into parts of near-equal size, each with
+    a slot; split: per such column (head, column, first slot, parts)."""
+
+    def __init__(self, layout, device, part=None):
+        lay = (layout != 0).cpu()
+        H, R, C = lay.shape
+        h, r, c = lay.nonzero().unbind(1)
+        col = h * C + c
+        order = torch.argsort(col * R + r)
+        sizes = torch.bincount(col, minlength=H * C)
+        if part is None:
+            # only columns that stand out are cut (every part costs a slot written and read): those of more than twice the
+            # average length
+            part = max(KV_PART_BLOCKS, -(-2 * int(sizes.sum()) // max(1, H * C)))
+        starts = torch.cumsum(sizes, 0) - sizes
+        parts = torch.clamp((sizes + part - 1) // part, min=1)
+        first_item = torch.cumsum(parts, 0) - parts
+        item_col = torch.repeat_interleave(torch.arange(H * C), parts)
+        n_items = int(item_col.numel())
+        k = torch.arange(n_items) - first_item[item_col]
+        base, rem = sizes[item_col] // parts[item_col], sizes[item_col] % parts[item_col]
+        count = base + (k < rem).long()
+        begin = starts[item_col] + k * base + torch.minimum(k, rem)
+        is_part = parts[item_col] > 1
+        slot = torch.where(is_part, torch.cumsum(is_part.long(), 0) - 1, torch.full_like(count, -1))
+        zero = torch.zeros_like(count)
+        header = torch.stack((count, 8 * n_items + 4 * begin, item_col // C, item_col % C, slot, zero, zero, zero), 1).reshape(-1)
+        entries = torch.stack((order, r[order], c[order], h[order]), 1).reshape(-1)
+        self.items = torch.cat((header, entries)).to(torch.int32).to(device)
+        self.n_items = n_items
+        self.columns = C
+        self.n_slots = int(is_part.sum())
+        long_cols = (parts > 1).nonzero().flatten()
+        self.n_split = int(long_cols.numel())
+        self.split = None
+        if self.n_split:
+            self.split = torch.stack((long_cols // C, long_cols % C, slot[first_item[long_cols]], parts[long_cols]), 1).reshape(-1).to(torch.int32).to(device)
 
 
 def _vec_ok(t):
@@ -54,21 +103,22 @@ class AttentionCore:
         return self.nnz
 
     def tables(self, device):
-        """(table, longest row, tile table or None, rows of the table's layout, present blocks per present tile as a share)
-        on `device`, or None when the layout does not divide into 64 x 64 tiles."""
+        """(table, longest row, tile table or None, rows of the table's layout, present blocks per present tile as a share,
+        tables of the column kernel) on `device`, or None when the layout does not divide into 64 x 64 tiles."""
         key = str(device)
         if key not in self._tables:
             S = 64 // self.block
             H, R, C = self.spdims
             if S == 1:
                 lut, maxlut = self.softmax.make_lut(device)
-                self._tables[key] = (lut, maxlut, None, R, 1.)
+                self._tables[key] = (lut, maxlut, None, R, 1., _ColumnTable(self.layout, device))
             elif R % S or C % S:
                 self._tables[key] = None
             else:
                 cctx, ids = _LayoutOnDevice(self.layout, device).coarse(S)
                 lut, maxlut = _sparse_softmax.make_lut(cctx.lay, 64, device)
-                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S, self.blocks() / max(1, ids.numel()))
+                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S, self.blocks() / max(1, ids.numel()),
+                                     _ColumnTable(cctx.lay, device))
         return self._tables[key]
 
     def usable(self, q, k, v, dropout_p=0., per_element_masks=False):
@@ -138,32 +188,65 @@ class _attention_core(torch.autograd.Function):
         fused_calls += 1
         ctx.save_for_backward(q, k, v, p, o, lut)
         ctx.core, ctx.scale, ctx.maxlut, ctx.tiles, ctx.rows = core, scale, maxlut, tiles, rows
+        ctx.columns = core.tables(q.device)[5]
         return o
+
+    @staticmethod
+    def rows_kernel(ctx, do, ds, delta):
+        """dq; with it the softmax gradient ds (if a tensor is given) and / or the rows' sums delta = sum_d do . o"""
+        q, k, v, p, o, lut = ctx.saved_tensors
+        core = ctx.core
+        Z, H, D = q.size(0), q.size(1), q.size(3)
+        dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        rc = _lib.load().bsp_attention_bwd(
+            _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, ctx.rows, D,
+            do.stride(0), do.stride(1), do.stride(2), v.stride(0), v.stride(1), v.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0) if ds is not None else 0,
+            core.block, ctx.scale, _lib.ptr(lut), ctx.maxlut, _lib.ptr(ctx.tiles), _lib.ptr(delta), delta.stride(1) if delta is not None else 0,
+            _lib.stream_ptr(q.device))
+        _lib.check(rc, 'bsp_attention_bwd')
+        return dq
+
+    @staticmethod
+    def columns_kernel(ctx, do, delta):
+        """dk and dv, the softmax gradient computed again from p and delta"""
+        q, k, v, p, o, lut = ctx.saved_tensors
+        Z, H, D = q.size(0), q.size(1), q.size(3)
+        ct = ctx.columns
+        dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+        dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+        partial = torch.empty((Z, ct.n_slots, 2, 64, D), dtype=torch.float32, device=q.device) if ct.n_slots else None
+        rc = _lib.load().bsp_attention_bwd_kv(
+            _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(q), _lib.ptr(v), _lib.ptr(p), _lib.ptr(delta), _lib.ptr(dk), _lib.ptr(dv), Z, H, ct.columns, D,
+            do.stride(0), do.stride(1), do.stride(2), q.stride(0), q.stride(1), q.stride(2), v.stride(0), v.stride(1), v.stride(2),
+            dk.stride(0), dk.stride(1), dk.stride(2), dv.stride(0), dv.stride(1), dv.stride(2), p.stride(0), delta.stride(1),
+            ctx.core.block, ctx.scale, _lib.ptr(ct.items), ct.n_items, _lib.ptr(ctx.tiles), _lib.ptr(partial), ct.n_slots, _lib.ptr(ct.split), ct.n_split,
+            _lib.stream_ptr(q.device))
+        _lib.check(rc, 'bsp_attention_bwd_kv')
+        return dk, dv
 
     @staticmethod
     def backward(ctx, do):
         q, k, v, p, o, lut = ctx.saved_tensors
         core = ctx.core
-        H, R, C = core.spdims
-        Z, D = q.size(0), q.size(3)
         do = _vec(do)
+        need_q, need_k, need_v = ctx.needs_input_grad[:3]
         dq = dk = dv = None
-        if ctx.needs_input_grad[2]:
-            dv = core.dsd_tn(p, do)                        # p^T . do, as the dsd operator's backward does (matmul.py:598-601)
-        if ctx.needs_input_grad[0] or ctx.needs_input_grad[1]:
-            ds = torch.empty_like(p)
-            dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
-            rc = _lib.load().bsp_attention_bwd(
-                _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, ctx.rows, D,
-                do.stride(0), do.stride(1), do.stride(2), v.stride(0), v.stride(1), v.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0), core.block, ctx.scale, _lib.ptr(lut), ctx.maxlut,
-                _lib.ptr(ctx.tiles), _lib.stream_ptr(q.device))
-            _lib.check(rc, 'bsp_attention_bwd')
-            if ctx.needs_input_grad[1]:
+        if need_k and FUSED_KV:
+            # two launches: rows (dq, delta), then columns (dk and dv)
+            delta = torch.empty((q.size(0), q.size(1), ctx.rows * 64), dtype=torch.float32, device=q.device)
+            dq = _attention_core.rows_kernel(ctx, do, None, delta)
+            dk, dv = _attention_core.columns_kernel(ctx, do, delta)
+        else:
+            if need_v:
+                dv = core.dsd_tn(p, do)                    # p^T . do, as the dsd operator's backward does (matmul.py:598-601)
+            if need_k:
+                ds = torch.empty_like(p)
+                dq = _attention_core.rows_kernel(ctx, do, ds, None)
                 dk = core.dsd_tn(ds, q)                    # ds^T . q (matmul.py:598-601 of the sdd operator)
-            if not ctx.needs_input_grad[0]:
-                dq = None
-        return (dq, dk, dv) + (None,) * 11
+            elif need_q:
+                dq = _attention_core.rows_kernel(ctx, do, None, None)
+        return (dq if need_q else None, dk, dv if need_v else None) + (None,) * 11
 
 
 def _core_for(sdd_nt, softmax, dsd_nn):
