@@ -54,9 +54,18 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   const int64_t wg = xcd_remap(blockIdx.x, n_wg);
   // block-rows from the last one down (the longest rows of a causal layout first), all rows of a (batch, head) in a
   // row: its k and v tiles stay in the L2 of the XCD that works on it
-  const int br = a.R - 1 - (int)(wg % a.R);
-  const int zh = (int)(wg / a.R);
-  const int h = zh % a.H, z = zh / a.H;
+  // (with per-element masks, which the batches share: the batches of a block-row next to each other, so that the second
+  // one finds the row's mask values in L2)
+  int br, h, z;
+  if constexpr (EXTRA) {
+    z = (int)(wg % a.Z);
+    br = a.R - 1 - (int)((wg / a.Z) % a.R);
+    h = (int)(wg / a.Z / a.R);
+  } else {
+    br = a.R - 1 - (int)(wg % a.R);
+    const int zh = (int)(wg / a.R);
+    h = zh % a.H, z = zh / a.H;
+  }
   const table_ptr lut = as_table(a.lut);
   const int size = lut[2 * (h * a.R + br) + 0];   // header (size, offset), softmax.py:30-32
   const int offset = lut[2 * (h * a.R + br) + 1];
