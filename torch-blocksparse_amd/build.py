@@ -24,13 +24,36 @@ def lib_path():
     return os.path.join(LIBDIR, LIBNAME)
 
 
+# Kernels that count their own outstanding vector-memory operations (s_waitcnt vmcnt(n) in front of the barriers of an
+# LDS ring of direct global -> LDS loads).  A register spill adds scratch loads and stores to that count and the waits
+# would then let a tile be read before it has landed: the build refuses such a kernel.
+COUNTED_WAITS = {'attention_core.hip': 'k_attn64', 'attention_long.hip': 'k_attn64', 'attention_kv.hip': 'k_attn64', 'matmul_dl.hip': 'k_'}
+
+
+def _spilled_kernels(remarks, prefix):
+    bad, name = [], None
+    for line in remarks.splitlines():
+        if 'Function Name:' in line:
+            name = line.split('Function Name:')[1].split()[0]
+        elif 'ScratchSize [bytes/lane]:' in line and name and prefix in name:
+            if int(line.split('ScratchSize [bytes/lane]:')[1].split()[0]) > 0:
+                bad.append(name)
+    return bad
+
+
 def _compile(src):
     obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + '.o')
-    cmd = ['hipcc'] + FLAGS + ['-c', os.path.join(CSRC, src), '-o', obj]
+    check = COUNTED_WAITS.get(src)
+    cmd = ['hipcc'] + FLAGS + (['-Rpass-analysis=kernel-resource-usage'] if check else []) + ['-c', os.path.join(CSRC, src), '-o', obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = '\n'.join(l for l in r.stderr.splitlines() if 'packed-fp32-ops' not in l)
     if r.returncode != 0:
         raise RuntimeError('hipcc failed on %s:\n%s' % (src, err))
+    if check:
+        bad = _spilled_kernels(err, check)
+        if bad:
+            raise RuntimeError('%s: kernels with counted waits use scratch memory (register spills):\n  %s' % (src, '\n  '.join(bad)))
+        err = '\n'.join(l for l in err.splitlines() if any(w in l for w in ('warning', 'error', 'note:')))   # (not the remarks and their source lines)
     return obj, err
 
 

@@ -166,6 +166,29 @@ template <int SUBS> __device__ __forceinline__ int chunk_in_block(int wave, int 
   return ((16 * wave + qrow) % B) * B + (32 * s + 8 * q) % B;
 }
 
+// wait until at most c (0 .. 16; more is treated as 16) vector-memory operations are outstanding, exactly
+__device__ __forceinline__ void wait_vm_exact(int c) {
+  switch (c < 16 ? c : 16) {
+    case 0: BSP_WAIT_VM(0); break;
+    case 1: BSP_WAIT_VM(1); break;
+    case 2: BSP_WAIT_VM(2); break;
+    case 3: BSP_WAIT_VM(3); break;
+    case 4: BSP_WAIT_VM(4); break;
+    case 5: BSP_WAIT_VM(5); break;
+    case 6: BSP_WAIT_VM(6); break;
+    case 7: BSP_WAIT_VM(7); break;
+    case 8: BSP_WAIT_VM(8); break;
+    case 9: BSP_WAIT_VM(9); break;
+    case 10: BSP_WAIT_VM(10); break;
+    case 11: BSP_WAIT_VM(11); break;
+    case 12: BSP_WAIT_VM(12); break;
+    case 13: BSP_WAIT_VM(13); break;
+    case 14: BSP_WAIT_VM(14); break;
+    case 15: BSP_WAIT_VM(15); break;
+    default: BSP_WAIT_VM(16); break;
+  }
+}
+
 // wait until at most c (0, 2, 4, 6 or 8) vector-memory operations are outstanding; the instruction takes an immediate
 __device__ __forceinline__ void wait_vm(int c) {
   if (c >= 8) BSP_WAIT_VM(8);

@@ -130,16 +130,47 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   // Before tile n is read: this wavefront's loads of it have landed (all but those of the tiles issued after it,
   // kStages - 2 of them or fewer near the end), then the barrier (everybody's have, and everybody is done reading tile n - 1), then the
   // load of tile n + kStages - 1 into the stage that tile n - 1 used.
-  auto step = [&](int n) {
-    const int rem = total - 1 - n;
-    if (rem >= kStages - 2) BSP_WAIT_VM(LW * (kStages - 2));
-    else if (kStages > 3 && rem == 1) BSP_WAIT_VM(LW);
-    else BSP_WAIT_VM(0);
+  // With per-element masks (EXTRA) the mask values of block b + 1 are fetched into registers while block b is worked on:
+  // four loads per lane and block (two masks, two chunks of eight columns; a mask that is not given is replaced by the
+  // other one, so that the count is fixed), issued right before the tile load of a step, the first ones (block 0)
+  // before the last tile of the prologue.  They share the counter of the tile loads and complete in order with them, so
+  // the wait for tile n also counts the mask loads issued after it: those of blocks max(0, n - kStages + 3) .. n, as far
+  // as they were issued (blocks 0 .. size).
+  constexpr int MASK_LOADS = 4;
+  auto arrive = [&](int n) {
+    if constexpr (EXTRA) {
+      int tiles = total - 1 - n;
+      tiles = tiles < kStages - 2 ? (tiles < 0 ? 0 : tiles) : kStages - 2;
+      const int first = n - kStages + 3 > 0 ? n - kStages + 3 : 0, last = n < size ? n : size;
+      wait_vm_exact(LW * tiles + MASK_LOADS * (last >= first ? last - first + 1 : 0));
+    } else {
+      const int rem = total - 1 - n;
+      if (rem >= kStages - 2) BSP_WAIT_VM(LW * (kStages - 2));
+      else if (kStages > 3 && rem == 1) BSP_WAIT_VM(LW);
+      else BSP_WAIT_VM(0);
+    }
     asm volatile("" ::: "memory");                     // (the compiler must not move LDS accesses across the barrier)
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+  };
+  auto advance = [&](int n) {
     if (n + kStages - 1 < total) issue(n + kStages - 1, next_col);
     next_col = tile_col(n + kStages);                  // the table runs one step ahead of the load that uses it
+  };
+  auto step = [&](int n) {
+    arrive(n);
+    advance(n);
+  };
+  // the mask values of the lane's two chunks of block b (address: softmax.py:50-55, 67-70)
+  auto load_masks = [&](int b, P8 (&pr)[2], P8 (&pa)[2]) {
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      const int64_t gcol = (int64_t)bcol[b < NB ? b : NB - 1] * 64 + 32 * s + 8 * q;
+      const T *attn = reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol;
+      const T *rpe = reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol;
+      pr[s].load(a.rpe ? rpe : attn);
+      pa[s].load(a.attn ? attn : rpe);
+    }
   };
   // The key-padding term of every column of the block-row (softmax.py:104-106, 122-124), fetched once per workgroup
   // and kept in LDS as the value that is added to the logits; the first barrier below orders it before its readers.
@@ -173,6 +204,8 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
       }
     }
   }
+  P8 pr[EXTRA ? NB + 1 : 1][2], pa[EXTRA ? NB + 1 : 1][2];
+  if constexpr (EXTRA) load_masks(0, pr[0], pa[0]);
 #pragma unroll
   for (int n = 2; n < kStages - 1; n++)
     if (n < total) issue(n, tile_col(n));
@@ -182,10 +215,18 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   f32x4 acc[NB][4];
   // the k row that supplies result row m of sub-tile jt (see the file comment)
   const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
+  float mx = -INFINITY;
+  int any_block = SUBS == 1;                           // small blocks: does the lane's row of small blocks hold any block?
 #pragma unroll
   for (int b = 0; b < NB; b++)
     if (b < size) {
-      step(b);
+      if constexpr (EXTRA) {
+        arrive(b);
+        load_masks(b + 1, pr[b + 1], pa[b + 1]);       // (past the row's end: the last block's again, never used)
+        advance(b);
+      } else {
+        step(b);
+      }
       const unsigned char *tile = ring + (b % kStages) * TB;
       frag_t kf[4][NK];
 #pragma unroll
@@ -199,6 +240,41 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
 #pragma unroll
         for (int s2 = 0; s2 < NK; s2++) acc[b][jt] = M::run(kf[jt][s2], xq[s2], acc[b][jt]);
       }
+      if constexpr (EXTRA) {
+        // the block's logits right away, with the mask values that were fetched during the previous block
+        const float unit = logit_unit<T>(), sc = a.scale * unit;
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+          float add[8];
+          if (a.kpm != nullptr) {
+#pragma unroll
+            for (int e4 = 0; e4 < 8; e4 += 4)
+              *reinterpret_cast<f32x4 *>(&add[e4]) = *reinterpret_cast<const f32x4 *>(&kpm_s[b * 64 + 32 * s + 8 * q + e4]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 8; i++) add[i] = 0.f;
+          }
+          if constexpr (SUBS > 1) {                    // a chunk in an absent small block takes no part in the row
+            const bool here = chunk_block_id<SUBS>(tid_[b], s, q) >= 0;
+            any_block |= here;
+            if (!here) {
+#pragma unroll
+              for (int i = 0; i < 8; i++) add[i] = -INFINITY;
+            }
+          }
+#pragma unroll
+          for (int i = 0; i < 8; i++) {
+            float fx = fmaf(to_float(from_float<T>(acc[b][2 * s + (i >> 2)][i & 3])), sc, add[i]);   // softmax.py:112-116, 122-124
+            if (a.rpe) fx = fmaf(to_float(pr[b][s].e[i]), unit, fx);                                 // :118-120
+            if (a.attn) {                                                                            // :126-128, 'mul' mode :108-110
+              const float m = to_float(pa[b][s].e[i]);
+              fx += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+            }
+            acc[b][2 * s + (i >> 2)][i & 3] = fx;
+            mx = fmaxf(mx, fx);
+          }
+        }
+      }
     }
 
   // ---- between the products: the softmax on the wavefront's 16 rows.  A lane's
@@ -209,27 +285,9 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   {
     const float unit = logit_unit<T>(), sc = a.scale * unit;
     const bool has_kpm = a.kpm != nullptr;
-    float mx = -INFINITY;
-    int any_block = SUBS == 1;                           // small blocks: does the lane's row of small blocks hold any block?
-    constexpr int GS = EXTRA ? (NB < 4 ? NB : 4) : NB;   // blocks whose mask values are in flight together
+    if constexpr (!EXTRA) {
 #pragma unroll
-    for (int g = 0; g < NB; g += GS) {
-      P8 pr[EXTRA ? GS : 1][2], pa[EXTRA ? GS : 1][2];
-      if constexpr (EXTRA) {
-#pragma unroll
-        for (int b = g; b < g + GS; b++)
-          if (b < size) {
-#pragma unroll
-            for (int s = 0; s < 2; s++) {
-              const int64_t gcol = (int64_t)bcol[b] * 64 + 32 * s + 8 * q;
-              if (a.rpe)                                                // address: softmax.py:50-55
-                pr[b - g][s].load(reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol);
-              if (a.attn) pa[b - g][s].load(reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol);   // :67-70
-            }
-          }
-      }
-#pragma unroll
-      for (int b = g; b < g + GS; b++)
+      for (int b = 0; b < NB; b++)
         if (b < size) {
 #pragma unroll
           for (int s = 0; s < 2; s++) {
@@ -252,14 +310,7 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
             }
 #pragma unroll
             for (int i = 0; i < 8; i++) {
-              float fx = fmaf(to_float(from_float<T>(acc[b][2 * s + (i >> 2)][i & 3])), sc, add[i]);   // softmax.py:112-116, 122-124
-              if constexpr (EXTRA) {
-                if (a.rpe) fx = fmaf(to_float(pr[b - g][s].e[i]), unit, fx);   // :118-120
-                if (a.attn) {                                                  // :126-128, 'mul' mode :108-110
-                  const float m = to_float(pa[b - g][s].e[i]);
-                  fx += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
-                }
-              }
+              const float fx = fmaf(to_float(from_float<T>(acc[b][2 * s + (i >> 2)][i & 3])), sc, add[i]);   // softmax.py:112-116, 122-124
               acc[b][2 * s + (i >> 2)][i & 3] = fx;
               mx = fmaxf(mx, fx);
             }
