@@ -499,6 +499,49 @@ def test_backward_through_the_column_kernel_and_through_the_two_operators(block,
             assert_close(g, r, dtype, name)
 
 
+class _FakeCtx:
+    """stand-in for the autograd context: the kernels of the backward pass called one by one"""
+    needs_input_grad = (True, True, True)
+
+    def save_for_backward(self, *t):
+        self.saved_tensors = t
+
+
+@pytest.mark.parametrize('R,block', [(6, 64), (12, 64), (8, 32)])
+def test_rows_kernel_outputs_in_every_combination(R, block):
+    """bsp_attention_bwd writes dq always, ds and the rows' delta each only when asked: the same bits in every
+    combination, delta = sum_d do . o, and the column kernel fed with that delta reproduces ds^T . q and p^T . do.
+    R = 12 block-rows of 64: rows of up to 12 tiles, the streaming kernels."""
+    torch.manual_seed(R)
+    Z, H, dh = 2, 2, 64
+    lay = torch.tril(torch.ones(H, R, R, dtype=torch.int64))
+    lay[1, :, 1] = 0
+    core = ac.AttentionCore(lay, block)
+    L = R * block
+    q, k, v, do = [torch.randn(Z, H, L, dh, device=DEV).half() for _ in range(4)]
+    ctx = _FakeCtx()
+    with torch.no_grad():
+        o = ac._attention_core.forward(ctx, q, k, v, 0.125, None, None, None, 'add', 'add', core, *core.tables(q.device)[:4])
+        p = ctx.saved_tensors[3]
+        outs = {}
+        for want_ds in (False, True):
+            for want_delta in (False, True):
+                ds = torch.full_like(p, 7.0) if want_ds else None
+                delta = torch.full((Z, H, ctx.rows * 64), 7.0, device=DEV) if want_delta else None
+                outs[(want_ds, want_delta)] = (ac._attention_core.rows_kernel(ctx, do, ds, delta), ds, delta)
+        dq, ds, delta = outs[(True, True)]
+        for key, (dq2, ds2, delta2) in outs.items():
+            assert torch.equal(dq2, dq), key
+            assert ds2 is None or torch.equal(ds2, ds), key
+            assert delta2 is None or torch.equal(delta2, delta), key
+        ref_delta = (do.float() * o.float()).sum(-1)
+        assert float((delta - ref_delta).abs().max()) <= 1e-3 * float(ref_delta.abs().max())
+        dk, dv = ac._attention_core.columns_kernel(ctx, do, delta)
+        dk_ops, dv_ops = core.dsd_tn(ds, q), core.dsd_tn(p, do)
+    for name, g, c in (('dk', dk, dk_ops), ('dv', dv, dv_ops)):
+        assert float((g.float() - c.float()).abs().max()) <= 1.5e-3 * float(c.float().abs().max()), name
+
+
 def test_c_abi_argument_checks():
     lib = _lib.load()
     t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
