@@ -135,7 +135,7 @@ def main():
         print(json.dumps({'metric': 'per-launch effective throughput (nonzero blocks), not the headline metric', 'n_gpus': 1,
                           'steps': args.steps, 'warmup': args.warmup, 'data': 'synthetic',
                           'config': {'workload': res['workload'], 'config': args.config, 'kernel_flags': args.kernel_flags},
-                          'launches': res['launches']}))
+                          'launches': res['launches'], **({'ms_per_step': res['ms_per_step']} if 'ms_per_step' in res else {})}))
         return
 
     import torch
@@ -634,8 +634,24 @@ def other_config(config, steps, warmup):
                 out.append(ent)
         out.extend(fused_chain_launches(lay, q, k, v, do, 0.125, timeit,
                                         [('scale only', {}), ('rpe + causal mask', dict(rpe=rpe, attn_mask=causal, attn_mask_mode='mul'))]))
+        # the whole step, forward + backward through autograd: the three operators against attention_chain (what the modules call)
+        from torch_blocksparse import attention_core as ac
+        qg, kg, vg = [t.detach().requires_grad_(True) for t in (q, k, v)]
+        steps_ms = {}
+        for label, kw in (('scale only', {}), ('rpe + causal mask', dict(rpe=rpe, attn_mask=causal, attn_mask_mode='mul'))):
+            for fused in (False, True):
+                def step():
+                    qg.grad = kg.grad = vg.grad = None
+                    ac.attention_chain(sdd, sm, dsd, qg, kg, vg, scale=0.125, **kw).backward(do)
+                old_fused, ac.FUSED = ac.FUSED, fused
+                try:
+                    steps_ms.setdefault(label, {})['fused chain' if fused else 'three operators'] = round(timeit(step), 4)
+                finally:
+                    ac.FUSED = old_fused
         workload = ('BigBird layout (3 window + 2 global + 3 random blocks, causal), batch 2, 12 heads, seq 16384, head_dim 64, block 64, fp16, '
                     'forward and backward launches; bound: HBM (softmax bytes: 2|x| + the mask and rpe bytes the layout touches)')
+        torch.cuda.empty_cache()
+        return {'workload': workload, 'launches': out, 'ms_per_step': steps_ms}
     torch.cuda.empty_cache()
     return {'workload': workload, 'launches': out}
 
