@@ -273,8 +273,7 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  * D = 64 or 128, blocks of 64, 32 or 16; BSP_ERR_UNSUPPORTED / BSP_ERR_ROW_TOO_LONG otherwise, and the caller runs
  * the three operators.  Rows of at most BSP_ATTENTION_MAX_ROW_BLOCKS tiles of 64 x 64 are held in registers; longer
  * rows (up to the softmax operator's 32768 elements) are streamed: forward in two sweeps over the row (running maximum
- * and sum first, then p and p . v), backward with dq accumulated block by block.  The streamed kernels take the
- * key-padding mask but neither rpe nor attn (BSP_ERR_ROW_TOO_LONG with either).
+ * and sum first, then p and p . v), backward with dq accumulated block by block.
  *   block 64: d_lut / maxlut from bsp_softmax_lut_build on the layout, R = its block-rows, d_tiles = NULL.
  *   blocks 16 and 32 (S = 64 / block, layout sides divisible by S): the kernels work on 64 x 64 tiles.  d_lut / maxlut
  *             from bsp_softmax_lut_build on the layout coarsened to tiles ([H, R_blocks / S, C_blocks / S], a tile

@@ -223,20 +223,8 @@ def test_modules_take_the_fused_kernels_and_agree_with_the_operators():
 def test_cases_left_to_the_three_operators():
     torch.manual_seed(7)
     Z, H, dh = 1, 2, 64
-    # a row of nine blocks is streamed by the fused kernels, which then take no per-element mask: with an attention mask
-    # or a relative position embedding such a layout goes to the operators
-    layout = torch.zeros(H, 10, 10, dtype=torch.int64)
-    layout[:, :, 0] = 1
-    layout[:, 9, :9] = 1
-    ops = _ops(layout)
-    q, k, v = [torch.randn(Z, H, 640, dh, device=DEV).half() for _ in range(3)]
-    am = (0.5 * torch.randn(640, 640, device=DEV)).half()
+    q = torch.randn(Z, H, 640, dh, device=DEV).half()
     n0 = ac.fused_calls
-    o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, attn_mask=am)
-    assert ac.fused_calls == n0
-    assert_close(o, D.attention(q, k, v, layout, 64, 0.125, attn_mask=am, attn_mask_mode='add'), torch.float16, 'o')
-    ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, rpe=am)
-    assert ac.fused_calls == n0
     # a row of 32768 elements: the softmax operator's own bound (softmax.py:225-227)
     layout = torch.ones(1, 1, 512, dtype=torch.int64)
     ops = _ops(layout)
@@ -358,16 +346,22 @@ def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
     assert ac.fused_calls == n0 + 1
 
 
-@pytest.mark.parametrize('block,dtype,dh,R,C,kpm', [
-    (64, torch.float16, 64, 12, 20, None),
-    (64, torch.float16, 64, 16, 16, 'add'),
-    (64, torch.bfloat16, 128, 10, 24, 'mul'),
-    (64, torch.float16, 128, 9, 9, None),
-    (32, torch.float16, 64, 16, 40, 'add'),
-    (16, torch.bfloat16, 64, 24, 80, 'mul'),
-    (16, torch.float16, 128, 16, 48, None),
+@pytest.mark.parametrize('block,dtype,dh,R,C,kpm,extra', [
+    (64, torch.float16, 64, 12, 20, None, ()),
+    (64, torch.float16, 64, 16, 16, 'add', ()),
+    (64, torch.bfloat16, 128, 10, 24, 'mul', ()),
+    (64, torch.float16, 128, 9, 9, None, ()),
+    (32, torch.float16, 64, 16, 40, 'add', ()),
+    (16, torch.bfloat16, 64, 24, 80, 'mul', ()),
+    (16, torch.float16, 128, 16, 48, None, ()),
+    (64, torch.float16, 64, 12, 20, None, ('rpe',)),
+    (64, torch.float16, 64, 16, 16, 'add', ('attn_mul',)),
+    (64, torch.bfloat16, 128, 10, 24, 'mul', ('rpe', 'attn_add')),
+    (64, torch.float16, 128, 12, 12, 'add', ('rpe', 'attn_mul')),
+    (32, torch.float16, 64, 16, 40, None, ('attn_add',)),
+    (16, torch.bfloat16, 64, 24, 80, 'add', ('rpe', 'attn_mul')),
 ])
-def test_rows_longer_than_eight_tiles_are_streamed(block, dtype, dh, R, C, kpm):
+def test_rows_longer_than_eight_tiles_are_streamed(block, dtype, dh, R, C, kpm, extra):
     """Rows of 9 .. 24 tiles beside short and empty ones: two-sweep forward, block-by-block backward; key-padding masks
     in both modes, among them a whole masked tile in the middle of a row (its maximum so far stays where it was) and
     one at the start (the running maximum starts at -inf)."""
@@ -394,6 +388,15 @@ def test_rows_longer_than_eight_tiles_are_streamed(block, dtype, dh, R, C, kpm):
         m[0, :64] = 0
         m[1, 190:330] = 0
         kw.update(key_padding_mask=m.to(DEV).to(dtype), key_padding_mask_mode='mul')
+    Lq, Lk = R * block, C * block
+    if 'rpe' in extra:
+        kw['rpe'] = (0.3 * torch.randn(H, Lq, Lk)).to(DEV).to(dtype)
+    if 'attn_add' in extra:
+        kw.update(attn_mask=(0.5 * torch.randn(Lq, Lk)).to(DEV).to(dtype), attn_mask_mode='add')
+    if 'attn_mul' in extra:
+        m = (torch.rand(Lq, Lk) < 0.7).float()
+        m[:, Lk - block:] = 1              # (no row loses all its columns: the last block-column is in every row with a block)
+        kw.update(attn_mask=m.to(DEV).to(dtype), attn_mask_mode='mul')
     with guard_allocations('fused attention, long rows'):
         got = _run(ops, q, k, v, do, True, **kw)
     chain = _run(ops, q, k, v, do, False, **kw)
@@ -404,7 +407,11 @@ def test_rows_longer_than_eight_tiles_are_streamed(block, dtype, dh, R, C, kpm):
     live = lay.sum(2).ne(0).all(0)
     rows = live.repeat_interleave(block).to(DEV)
     okw = {n: kw[n] for n in ('key_padding_mask', 'key_padding_mask_mode') if n in kw}
-    ref = D.attention(q[:, :, rows], k, v, lay[:, live], block, kw['scale'], do=do[:, :, rows], attn_mask_mode='add', **okw)
+    if 'rpe' in kw:
+        okw['rpe'] = kw['rpe'][:, rows]
+    if 'attn_mask' in kw:
+        okw['attn_mask'] = kw['attn_mask'][rows]
+    ref = D.attention(q[:, :, rows], k, v, lay[:, live], block, kw['scale'], do=do[:, :, rows], attn_mask_mode=kw.get('attn_mask_mode', 'add'), **okw)
     assert_close(got[0][:, :, rows], ref[0], dtype, 'o')
     assert_close(got[1][:, :, rows], ref[1], dtype, 'dq')
 
@@ -561,7 +568,7 @@ def test_c_abi_argument_checks():
     assert fwd(tiles=_lib.ptr(lut)) != _lib.OK          # ... and blocks of 64 take none
     assert fwd(D=96) == _lib.ERR_UNSUPPORTED
     assert fwd(maxlut=9) == _lib.OK                     # (the streaming kernels; the table's rows hold one block)
-    assert fwd(maxlut=9, rpe=_lib.ptr(t)) == _lib.ERR_ROW_TOO_LONG
+    assert fwd(maxlut=9, rpe=_lib.ptr(t)) == _lib.OK
     assert fwd(maxlut=512) == _lib.ERR_ROW_TOO_LONG
     assert fwd(ldq=60) != _lib.OK                       # a row stride that is not a multiple of 8 elements
     assert fwd(q=None) != _lib.OK

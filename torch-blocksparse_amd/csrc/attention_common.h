@@ -229,7 +229,7 @@ template <int D> __device__ __forceinline__ int dual_offset(int r, int col) {   
 }
 
 }  // namespace
-// rows of more than BSP_ATTENTION_MAX_ROW_BLOCKS tiles (attention_long.hip); no relative position embedding, no attention mask
+// rows of more than BSP_ATTENTION_MAX_ROW_BLOCKS tiles (attention_long.hip)
 int attention_long(int dtype, const AttnArgs &a, int D, int block, bool bwd, hipStream_t st);
 // dk and dv, one workgroup per column of tiles (attention_kv.hip)
 int attention_kv(int dtype, const AttnArgs &a, int D, int block, hipStream_t st);

@@ -678,8 +678,7 @@ int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *st
   if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
   if ((block != 64) != (a.tiles != nullptr)) return BSP_ERR_ARG;   // the tile table goes with the small blocks, and only with them
   if ((int64_t)maxlut * 64 >= 32768) return BSP_ERR_ROW_TOO_LONG;   // the softmax operator's bound on a row (softmax.py:225-227)
-  const bool is_long = maxlut > BSP_ATTENTION_MAX_ROW_BLOCKS;         // longer rows: streamed, without the two per-element masks
-  if (is_long && (a.rpe || a.attn)) return BSP_ERR_ROW_TOO_LONG;
+  const bool is_long = maxlut > BSP_ATTENTION_MAX_ROW_BLOCKS;         // longer rows: streamed
   // 16-byte vector accesses everywhere: every pointer and every stride a multiple of 8 elements
   const void *ptrs[] = {a.x, a.y1, a.y2, a.p_in, a.o_in, a.p_out, a.o, a.rpe, a.kpm, a.attn};
   for (const void *p : ptrs)

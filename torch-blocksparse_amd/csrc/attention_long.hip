@@ -9,8 +9,8 @@
 //             running sum of exponentials of each row (rescaled when the maximum grows); the second computes the
 //             scores again (the k tiles come from L2 a second time, the matrix instructions are cheap), writes
 //             p = exp(s - max) / sum and accumulates p . v.  Twice the exponentials of the kernel that holds the row.
-// No relative position embedding and no attention mask here (their values would have to travel through the ring
-// too); the key-padding mask of a block is one more 128-byte load of a k tile's stage.
+// The key-padding mask of a block is one more 128-byte load of a k tile's stage; the values of a relative position
+// embedding and of an attention mask are fetched into registers in the step of the block's k tile (in both sweeps).
 #include "attention_common.h"
 
 namespace bsp {
@@ -217,7 +217,7 @@ if (a.p_out == nullptr) continue;   // ds is not asked for
   store_rows<T, D>(cs, po, a.o_ld, o, lane);
 }
 
-template <typename T, int D, int SUBS>
+template <typename T, int D, int SUBS, bool EXTRA>
 __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   typedef Mma16<T> M;
   typedef typename M::frag_t frag_t;
@@ -299,13 +299,42 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
       }
     }
   };
-  auto step = [&](int n) {   // stores of p issued in between are not counted: see k_attn64_bwd_long
-    wait_vm(loads_of(n + 1) + (kStages > 3 ? loads_of(n + 2) : 0));
+  // With per-element masks (EXTRA) the step of a k tile fetches the block's mask values into registers between the
+  // barrier and the next tile load: four loads per lane (two masks, two chunks of eight columns; a mask that is not
+  // given is replaced by the other, so that the count is fixed).  They share the counter of the tile loads and complete
+  // in order with them: the wait for tile n also counts the mask loads of the k-tile steps n - kStages + 2 .. n - 1,
+  // and using the values makes the tiles issued before them land one or two steps early.
+  constexpr int MASK_LOADS = 4;
+  auto is_k_step = [&](int m) { return m >= 0 && m < total && !is_v(m); };
+  auto arrive = [&](int n) {   // stores of p issued in between are not counted: see k_attn64_bwd_long
+    if constexpr (EXTRA) {
+      wait_vm_exact(loads_of(n + 1) + (kStages > 3 ? loads_of(n + 2) : 0) +
+                    MASK_LOADS * ((is_k_step(n - 1) ? 1 : 0) + (kStages > 3 && is_k_step(n - 2) ? 1 : 0)));
+    } else {
+      wait_vm(loads_of(n + 1) + (kStages > 3 ? loads_of(n + 2) : 0));
+    }
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+  };
+  auto advance = [&](int n) {
     if (n + kStages - 1 < total) issue(n + kStages - 1, next_col);
     next_col = tile_col(n + kStages);
+  };
+  auto step = [&](int n) {
+    arrive(n);
+    advance(n);
+  };
+  // the mask values of the lane's two chunks of the block in block-column col (address: softmax.py:50-55, 67-70)
+  auto load_masks = [&](int col, P8 (&pr)[2], P8 (&pa)[2]) {
+#pragma unroll
+    for (int s = 0; s < 2; s++) {
+      const int64_t gcol = (int64_t)col * 64 + 32 * s + 8 * q;
+      const T *attn = reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol;
+      const T *rpe = reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol;
+      pr[s].load(a.rpe ? rpe : attn);
+      pa[s].load(a.attn ? attn : rpe);
+    }
   };
 #pragma unroll
   for (int n = 0; n < kStages - 1; n++) issue(n, tile_col(n));   // (three tiles at least)
@@ -314,7 +343,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
   const float unit = logit_unit<T>(), sc = a.scale * unit;
   // the logits of the lane's 16 values of the tile in stage n % kStages: fx[2s + t][e], columns 32s + 8q + 4t + e
-  auto logits = [&](int n, const i32x4 &ids, f32x4 (&fx)[4]) {
+  auto logits = [&](int n, const i32x4 &ids, f32x4 (&fx)[4], const P8 (&pr)[2], const P8 (&pa)[2]) {
     const unsigned char *tile = ring + (n % kStages) * TB;
     frag_t kf[4][NK];
 #pragma unroll
@@ -350,8 +379,17 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
         }
       }
 #pragma unroll
-      for (int i = 0; i < 8; i++)                        // :112-116
-        fx[2 * s + (i >> 2)][i & 3] = fmaf(to_float(from_float<T>(fx[2 * s + (i >> 2)][i & 3])), sc, add[i]);
+      for (int i = 0; i < 8; i++) {                      // :112-116
+        float f = fmaf(to_float(from_float<T>(fx[2 * s + (i >> 2)][i & 3])), sc, add[i]);
+        if constexpr (EXTRA) {
+          if (a.rpe) f = fmaf(to_float(pr[s].e[i]), unit, f);                                       // :118-120
+          if (a.attn) {                                                                            // :126-128, 'mul' mode :108-110
+            const float m = to_float(pa[s].e[i]);
+            f += a.attn_mul ? (m == 0.f ? -INFINITY : 0.f) : m * unit;
+          }
+        }
+        fx[2 * s + (i >> 2)][i & 3] = f;
+      }
     }
   };
 
@@ -361,9 +399,16 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   for (int b = 0; b < size; b++) {
     const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), core[4 * b], rs);
     if constexpr (SUBS > 1) any_block |= int(chunk_block_id<SUBS>(ids, 0, q) >= 0 || chunk_block_id<SUBS>(ids, 1, q) >= 0);
-    step(b);
+    P8 pr[2], pa[2];
+    if constexpr (EXTRA) {
+      arrive(b);
+      load_masks(core[4 * b + 1], pr, pa);
+      advance(b);
+    } else {
+      step(b);
+    }
     f32x4 fx[4];
-    logits(b, ids, fx);
+    logits(b, ids, fx, pr, pa);
     float mb = m_run;
 #pragma unroll
     for (int jt = 0; jt < 4; jt++)
@@ -402,9 +447,16 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
     const int tile_id = core[4 * b];
     const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), tile_id, rs);
     const int n = size + 2 * b;
-    step(n);
+    P8 pr[2], pa[2];
+    if constexpr (EXTRA) {
+      arrive(n);
+      load_masks(core[4 * b + 1], pr, pa);
+      advance(n);
+    } else {
+      step(n);
+    }
     f32x4 fx[4];
-    logits(n, ids, fx);
+    logits(n, ids, fx, pr, pa);
     frag_t pf[2];
 #pragma unroll
     for (int s = 0; s < 2; s++) {
@@ -450,7 +502,8 @@ template <typename T, int D, int SUBS> void launch_long(const AttnArgs &a, bool 
   constexpr int LDS = ring_stages<D>() * 64 * D * 2 + 4 * 16 * 72 * 2 + ring_stages<D>() * 128;
   static_assert(LDS <= 64 * 1024, "within what a launch may ask for without raising the kernel's limit");
   if (bwd) hipLaunchKernelGGL((k_attn64_bwd_long<T, D, SUBS>), grid, wg, LDS, st, a);
-  else hipLaunchKernelGGL((k_attn64_fwd_long<T, D, SUBS>), grid, wg, LDS, st, a);
+  else if (a.rpe || a.attn) hipLaunchKernelGGL((k_attn64_fwd_long<T, D, SUBS, true>), grid, wg, LDS, st, a);
+  else hipLaunchKernelGGL((k_attn64_fwd_long<T, D, SUBS, false>), grid, wg, LDS, st, a);
 }
 
 template <typename T, int SUBS> int launch_long_d(const AttnArgs &a, int D, bool bwd, hipStream_t st) {
@@ -470,7 +523,6 @@ template <typename T> int launch_long_t(const AttnArgs &a, int D, int block, boo
 }  // namespace
 
 int attention_long(int dtype, const AttnArgs &a, int D, int block, bool bwd, hipStream_t st) {
-  if (a.rpe || a.attn) return BSP_ERR_ROW_TOO_LONG;
   if (dtype == BSP_F16) return launch_long_t<f16>(a, D, block, bwd, st);
   if (dtype == BSP_BF16) return launch_long_t<bf16>(a, D, block, bwd, st);
   return BSP_ERR_UNSUPPORTED;

@@ -17,7 +17,7 @@ from .matmul import MatMul, _LayoutOnDevice
 from .softmax import Softmax, _sparse_softmax
 
 FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
-MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS: longer rows are streamed
+MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS: longer rows are streamed (the library decides)
 fused_calls = 0             # forward calls that took the fused kernels; tests read it
 # Blocks of 16 and 32 are computed as whole 64 x 64 tiles: a tile costs the same however few of its blocks exist, so
 # below this share of present blocks per present tile the three operators (whose work follows the blocks) are faster.
@@ -121,10 +121,9 @@ class AttentionCore:
                                      _ColumnTable(cctx.lay, device))
         return self._tables[key]
 
-    def usable(self, q, k, v, dropout_p=0., per_element_masks=False):
+    def usable(self, q, k, v, dropout_p=0.):
         """Can this call take the fused kernels?  (Shapes that do not fit the layout are left to the operators, which
-        raise the reference's errors.)  Rows of more than MAX_ROW_BLOCKS tiles go to the streaming kernels, which take
-        neither a relative position embedding nor an attention mask (`per_element_masks`)."""
+        raise the reference's errors.)"""
         if not FUSED or self.block not in (16, 32, 64) or dropout_p:
             return False
         if not (q.is_cuda and q.dtype in (torch.float16, torch.bfloat16) and k.dtype == q.dtype and v.dtype == q.dtype):
@@ -138,7 +137,7 @@ class AttentionCore:
         t = self.tables(q.device)
         if t is None or t[1] <= 0 or t[4] < MIN_TILE_FILL.get(b, 0.):
             return False
-        return t[1] <= MAX_ROW_BLOCKS or (not per_element_masks and t[1] * 64 < 32768)
+        return t[1] * 64 < 32768                           # the softmax operator's bound on a row (softmax.py:225-227)
 
     def __call__(self, q, k, v, scale=1., rpe=None, key_padding_mask=None, attn_mask=None,
                  key_padding_mask_mode='add', attn_mask_mode='add'):
@@ -270,7 +269,7 @@ def attention_chain(sdd_nt, softmax, dsd_nn, q, k, v, scale=1., rpe=None, key_pa
                     key_padding_mask_mode='add', attn_mask_mode='add', dropout_p=0.):
     """dsd_nn(softmax(sdd_nt(q, k), ...), v): fused when the operators and tensors allow it, else the three calls."""
     core = _core_for(sdd_nt, softmax, dsd_nn)
-    if core is not None and core.usable(q, k, v, dropout_p, rpe is not None or attn_mask is not None):
+    if core is not None and core.usable(q, k, v, dropout_p):
         return core(q, k, v, scale, rpe, key_padding_mask, attn_mask, key_padding_mask_mode, attn_mask_mode)
     w = sdd_nt(q, k)
     kwargs = dict(dropout_p=dropout_p) if dropout_p else {}
