@@ -549,6 +549,49 @@ def test_rows_kernel_outputs_in_every_combination(R, block):
         assert float((g.float() - c.float()).abs().max()) <= 1.5e-3 * float(c.float().abs().max()), name
 
 
+@pytest.mark.parametrize('seed', range(32))
+def test_seeded_random_sweep_against_the_three_operators(seed):
+    """Random layouts (square and rectangular, rows and columns from empty to long, tiles from full to mostly holes),
+    block sizes, head dimensions, types and mask combinations: every kernel variant (rows in registers / streamed, with
+    and without per-element masks, columns whole / in parts) against the three-operator chain."""
+    g = torch.Generator().manual_seed(1000 + seed)
+    rnd = lambda n: int(torch.randint(0, n, (1,), generator=g))
+    block = (64, 32, 16)[rnd(3)]
+    S = 64 // block
+    dh = (64, 128)[rnd(2)]
+    dtype = (torch.float16, torch.bfloat16)[rnd(2)]
+    Z, H = 1 + rnd(2), 1 + rnd(3)
+    Rt, Ct = 1 + rnd(20), 1 + rnd(20)                     # tiles of 64
+    if seed % 4 == 0:
+        Rt, Ct = 9 + rnd(12), 9 + rnd(12)                  # long rows more often
+    R, C = Rt * S, Ct * S
+    density = (0.15, 0.4, 0.7, 1.0)[rnd(4)]
+    lay = (torch.rand(H, R, C, generator=g) < density).long()
+    lay[:, :, rnd(C)] = 1                                  # a full column (long when R is), so no row is empty ...
+    if R > 2:
+        lay[rnd(H), rnd(R), :] = 0                         # ... except one
+    torch.manual_seed(seed)
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.Softmax(lay, block), tb.MatMul(lay, block, 'dsd'))
+    Lq, Lk = R * block, C * block
+    q, do = [torch.randn(Z, H, Lq, dh, device=DEV).to(dtype) for _ in range(2)]
+    k, v = [torch.randn(Z, H, Lk, dh, device=DEV).to(dtype) for _ in range(2)]
+    kw = dict(scale=dh ** -0.5)
+    choice = rnd(8)
+    if choice & 1:
+        kw['key_padding_mask'] = (0.5 * torch.randn(Z, Lk, generator=g)).to(DEV).to(dtype)
+    if choice & 2:
+        kw['rpe'] = (0.3 * torch.randn(H, Lq, Lk, generator=g)).to(DEV).to(dtype)
+    if choice & 4:
+        kw.update(attn_mask=(0.5 * torch.randn(Lq, Lk, generator=g)).to(DEV).to(dtype), attn_mask_mode='add')
+    got = _run(ops, q, k, v, do, True, **kw)
+    chain = _run(ops, q, k, v, do, False, **kw)
+    tol = CHAIN_TOL[dtype]
+    for name, a, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
+        assert not bool(torch.isnan(a).any()), name
+        ref = float(c.float().abs().max())
+        assert float((a.float() - c.float()).abs().max()) <= tol[0 if name in ('o', 'dv') else 1] * ref, (name, block, dh, dtype, Rt, Ct, density, choice)
+
+
 def test_c_abi_argument_checks():
     lib = _lib.load()
     t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
