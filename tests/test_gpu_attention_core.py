@@ -329,7 +329,7 @@ def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
     lay[:, torch.arange(16), torch.arange(16)] = 1            # one block of 16 per tile of 4 x 4
     ops = (tb.MatMul(lay, 16, 'sdd', trans_b=True), tb.Softmax(lay, 16), tb.MatMul(lay, 16, 'dsd'))
     q, k, v = [torch.randn(Z, H, 256, dh, device=DEV).half() for _ in range(3)]
-    ac.MIN_TILE_FILL.update({16: 0.3, 32: 0.5})
+    ac.MIN_TILE_FILL.update({16: 0.25, 32: 0.5})
     n0 = ac.fused_calls
     o = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0
@@ -337,7 +337,7 @@ def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
     o2 = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125)
     assert ac.fused_calls == n0 + 1
     assert float((o.float() - o2.float()).abs().max()) <= 4e-3 * float(o.float().abs().max())
-    ac.MIN_TILE_FILL.update({16: 0.3, 32: 0.5})
+    ac.MIN_TILE_FILL.update({16: 0.25, 32: 0.5})
     # the default block of the sparse self-attention module is 16: it takes the fused kernels
     mod = tb.SparseSelfAttention(tb.SparsityConfig(mode='fixed', block=16, stride=64, attention='unidirectional'))
     q, k, v = [torch.randn(2, 4, 512, dh, device=DEV).half() for _ in range(3)]

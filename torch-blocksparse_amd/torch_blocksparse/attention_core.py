@@ -21,8 +21,10 @@ MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS: longer rows are stre
 fused_calls = 0             # forward calls that took the fused kernels; tests read it
 # Blocks of 16 and 32 are computed as whole 64 x 64 tiles: a tile costs the same however few of its blocks exist, so
 # below this share of present blocks per present tile the three operators (whose work follows the blocks) are faster.
-# Measured break-even points on MI355X, fwd + bwd, head dimension 64, rows of 8 tiles and of 30+ tiles.
-MIN_TILE_FILL = {16: 0.3, 32: 0.5}
+# Measured on MI355X, fwd + bwd, head dimension 64, rows of 8 tiles and of 30+ tiles: break-even at 0.5 for blocks of 32;
+# for blocks of 16 the two paths stay within 8 % of each other between 0.15 and 0.3, which way depends on the layout
+# (the 'fixed' layout of the sparse self-attention module's default configuration, 0.26, is 8 % faster fused).
+MIN_TILE_FILL = {16: 0.25, 32: 0.5}
 # dk and dv from the column kernel (bsp_attention_bwd_kv), which computes the softmax gradient again instead of reading it;
 # False: the row kernel stores the gradient and the two products are ordinary dsd operators
 FUSED_KV = os.environ.get('BSP_FUSED_ATTENTION_KV', '1') != '0'
