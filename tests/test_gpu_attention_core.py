@@ -326,7 +326,7 @@ def test_small_blocks_that_the_tiles_do_not_fit_go_to_the_operators():
     assert_close(o, D.attention(q, k, v, lay, 16, 0.125, attn_mask_mode='add'), torch.float16, 'o')
     # tiles that are mostly holes: the kernels would compute them whole, the operators are chosen
     lay = torch.zeros(H, 16, 16, dtype=torch.int64)
-    lay[:, torch.arange(16), torch.arange(16)] = 1            # one block of 16 per tile of 4 x 4
+    lay[:, torch.arange(0, 16, 2), torch.arange(0, 16, 2)] = 1   # two blocks of 16 per tile of 4 x 4 on the diagonal
     ops = (tb.MatMul(lay, 16, 'sdd', trans_b=True), tb.Softmax(lay, 16), tb.MatMul(lay, 16, 'dsd'))
     q, k, v = [torch.randn(Z, H, 256, dh, device=DEV).half() for _ in range(3)]
     ac.MIN_TILE_FILL.update({16: 0.25, 32: 0.5})
