@@ -275,11 +275,15 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  * rows (up to the softmax operator's 32768 elements) are streamed: forward in two sweeps over the row (running maximum
  * and sum first, then p and p . v), backward with dq accumulated block by block.
  *   block 64: d_lut / maxlut from bsp_softmax_lut_build on the layout, R = its block-rows, d_tiles = NULL.
- *   blocks 16 and 32 (S = 64 / block, layout sides divisible by S): the kernels work on 64 x 64 tiles.  d_lut / maxlut
- *             from bsp_softmax_lut_build on the layout coarsened to tiles ([H, R_blocks / S, C_blocks / S], a tile
- *             present if any of its S x S blocks is), R = its rows; d_tiles: per present tile, in the order of that table's block ids (row-major over head, tile-row,
- *             tile-column), S * S ints: the ids of its blocks in the [Z, nnz, block, block] tensor, row by row, -1
- *             where absent.
+ *   blocks 16 and 32 (S = 64 / block, layout sides divisible by S): the kernels work on 64 x 64 tiles that the caller
+ *             forms: a line of tiles is S consecutive block-rows, and a tile takes S block-columns gathered from
+ *             anywhere in the line (in practice: the columns in which any of the line's block-rows holds a block,
+ *             ascending, S per tile, so that single block-columns do not cost whole tiles).  R = lines.  d_lut: per
+ *             (head, line) two ints (tiles, offset of the first entry in ints from the start), then per tile eight
+ *             ints (tile index, ., ., ., then its S block-columns; unused slots repeat a valid column).  d_tiles: per
+ *             tile, by tile index, S * S ints: the ids of its blocks in the [Z, nnz, block, block] tensor,
+ *             [block-row of the line][gathered block-column], -1 where the layout has none.  maxlut = the most
+ *             tiles of a line.
  *   forward : p = softmax(round(q . k^T) * scale + rpe + kpm + attn) over each row's nonzero blocks, o = p . v.
  *             q, o: [Z, H, rows, D]; k, v: [Z, H, columns, D], unit stride along D; p: [Z, nnz, block, block] (every
  *             block is written); rows of o without any block are set to zero.  Masks as for bsp_softmax_fwd.
@@ -313,14 +317,19 @@ int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, 
  * dk = ds^T . q with ds computed again from p (the formula above), delta = the row sums that bsp_attention_bwd wrote
  * ([Z][H][delta_stride_h], fp32).  Call bsp_attention_bwd with ds = NULL and delta given first: the sparse gradient
  * is then neither written nor read.  Replaces the two transposed dsd products of the operators' backward pass
- * (matmul.py:598-601).  d_col_lut: the layout (coarsened to tiles for blocks of 16 / 32, as d_lut) read along columns:
- * n_items work items of eight ints (number of blocks, offset of the first entry in ints from the start, head, column,
- * slot, 0, 0, 0), then per block four ints (id, row, column, head), the blocks of a column by row.  A work item is a
+ * (matmul.py:598-601).  d_col_lut: the layout read along columns: n_items work items of twelve ints (number of entries,
+ * offset of the first entry in ints from the start, head, column, slot, 0, 0, 0, then the column's S block-columns,
+ * the last repeated up to four), then the entries, a column's by row.  Block 64: a column is a block-column, an entry
+ * four ints (id, row, column, head).  Blocks 16 / 32: a column is any S block-columns of a head (every block-column
+ * in exactly one; the kernel takes the wavefronts' keys from them), an entry a tile of eight ints (tile index, ., ., .,
+ * then the S block-rows gathered into it), and d_tiles gives per tile the ids [gathered block-row][block-column of the
+ * column] (tiles of this call's own numbering, not those of bsp_attention_fwd / _bwd).  A work item is a
  * whole column (slot -1; also every column without blocks, whose rows of dk and dv are set to zero) or one part of a
  * long column: columns differ in length far more than rows do, so the caller cuts the long ones into parts, whose
  * partial sums go to fp32 slots (partial: [Z][n_slots][2][64][D] floats, slot = the item's) and are added in order by a
- * second kernel of the same call, per d_split_lut: n_split entries of four ints (head, column, first slot, parts; a
- * column's slots are consecutive).  No atomics.  C = columns; dk, dv: [Z, H, columns, D]. */
+ * second kernel of the same call, per d_split_lut: n_split entries of eight ints (head, column, first slot, parts, then
+ * the column's block-columns as in the work items; a column's slots are consecutive).  No atomics.  C = columns of
+ * tiles; dk, dv: [Z, H, keys, D]. */
 int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, const void *v, const void *p, const float *delta, void *dk,
                          void *dv, int Z, int H, int C, int D, int64_t do_stride_z, int64_t do_stride_h, int64_t lddo,
                          int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t v_stride_z, int64_t v_stride_h,

@@ -160,6 +160,35 @@ template <int SUBS> __device__ __forceinline__ i32x4 load_block_ids(table_ptr ti
   }
   return t;
 }
+// Table entries.  Blocks of 64: four ints (block id, block-column [the column kernel: block-row], ., .).  Smaller
+// blocks: eight ints (tile, ., ., ., then the S block-columns [block-rows] gathered into the tile, S = SUBS): the tile's
+// 64 columns [rows] are S groups of 64 / S consecutive ones, each group anywhere in the matrix.
+template <int SUBS> constexpr int entry_ints() { return SUBS == 1 ? 4 : 8; }
+template <int SUBS> __device__ __forceinline__ int entry_group(table_ptr e, int g) { return SUBS == 1 ? e[1] : e[4 + g]; }
+template <int SUBS> __device__ __forceinline__ i32x4 entry_groups(table_ptr e) {
+  i32x4 t = i32x4{0, 0, 0, 0};
+  if constexpr (SUBS == 1) {
+    t[0] = e[1];
+  } else {
+#pragma unroll
+    for (int g = 0; g < SUBS; g++) t[g] = e[4 + g];
+  }
+  return t;
+}
+// position (in elements) of the lane's chunk (columns 32s + 8q .. + 7 of the tile) in the matrix, from the tile's groups
+template <int SUBS> __device__ __forceinline__ int64_t chunk_position(const i32x4 &groups, int s, int q) {
+  constexpr int B = 64 / SUBS;
+  if constexpr (SUBS == 1) return (int64_t)groups[0] * 64 + 32 * s + 8 * q;
+  else return (int64_t)chunk_block_id<SUBS>(groups, s, q) * B + (32 * s + 8 * q) % B;
+}
+// position of element j (0 .. 63, any lane) of the tile
+template <int SUBS> __device__ __forceinline__ int64_t element_position(const i32x4 &groups, int j) {
+  constexpr int B = 64 / SUBS;
+  int grp = groups[0];
+#pragma unroll
+  for (int g = 1; g < SUBS; g++) grp = (j / B == g) ? groups[g] : grp;
+  return (int64_t)grp * B + j % B;
+}
 // the lane's chunk (row 16 * wave + lane % 16 of the tile, columns 32s + 8q ..) inside its small block, in elements
 template <int SUBS> __device__ __forceinline__ int chunk_in_block(int wave, int qrow, int s, int q) {
   constexpr int B = 64 / SUBS;

@@ -82,16 +82,19 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
     return;
   }
   const table_ptr core = lut + offset;
-  int32_t bid[NB], bcol[NB];
+  constexpr int ES = entry_ints<SUBS>();
+  const int wgroup = (16 * wave) / (64 / SUBS);   // the group of the tile's rows (k, v: of the gathered columns) that the wavefront's 16 lie in
+  int32_t bid[NB];
+  i32x4 bcol[NB];    // the block-column(s) of each tile
 #pragma unroll
   for (int b = 0; b < NB; b++) {
     const int bb = b < size ? b : 0;    // blocks past the end repeat the first one (valid to read, never used)
-    bid[b] = core[4 * bb + 0];
-    bcol[b] = core[4 * bb + 1];
+    bid[b] = core[ES * bb + 0];
+    bcol[b] = entry_groups<SUBS>(core + ES * bb);
   }
   i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
 #pragma unroll
-  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], (16 * wave) / (64 / SUBS));
+  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   frag_t xq[NK];
 #pragma unroll
@@ -111,18 +114,19 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   const int total = 2 * size;
   int next_col;
   // the block-column of tile n, from the table (a scalar load; clamped past the end)
+  // (small blocks: the block-column of the group that this wavefront loads; off1 / off2 count rows from the tile's first)
   auto tile_col = [&](int n) {
     const int m = n < size ? n : n - size;
-    return core[4 * (m < size ? m : size - 1) + 1];
+    return entry_group<SUBS>(core + ES * (m < size ? m : size - 1), wgroup) - wgroup;
   };
   auto issue = [&](int n, int col) {
     unsigned char *st = ring + (n % kStages) * TB + wave * LW * 1024;
     if (n < size) {
-      const T *base = py1 + (int64_t)col * 64 * a.y1_ld;
+      const T *base = py1 + (int64_t)col * (64 / SUBS) * a.y1_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++) __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + i * 1024), 16, 0, 0);
     } else {
-      const T *base = py2 + (int64_t)col * 64 * a.y2_ld;
+      const T *base = py2 + (int64_t)col * (64 / SUBS) * a.y2_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++) __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + i * 1024), 16, 0, 0);
     }
@@ -165,7 +169,7 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   auto load_masks = [&](int b, P8 (&pr)[2], P8 (&pa)[2]) {
 #pragma unroll
     for (int s = 0; s < 2; s++) {
-      const int64_t gcol = (int64_t)bcol[b < NB ? b : NB - 1] * 64 + 32 * s + 8 * q;
+      const int64_t gcol = chunk_position<SUBS>(bcol[b < NB ? b : NB - 1], s, q);
       const T *attn = reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol;
       const T *rpe = reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol;
       pr[s].load(a.rpe ? rpe : attn);
@@ -179,10 +183,10 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   {
     if (kpm_lane) {
       const int b = tid >> 3;
-      int col = bcol[0];
+      i32x4 col = bcol[0];
 #pragma unroll
       for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
-      kp.load(reinterpret_cast<const T *>(a.kpm) + z * a.kpm_sz + (int64_t)col * 64 + (tid & 7) * 8);
+      kp.load(reinterpret_cast<const T *>(a.kpm) + z * a.kpm_sz + element_position<SUBS>(col, (tid & 7) * 8));
     }
   }
   // the first two tiles always exist (a row has at least one block); in a straight line, so that the wait for the
@@ -446,12 +450,13 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
     return;
   }
   const table_ptr core = lut + offset;
+  constexpr int ES = entry_ints<SUBS>();
+  const int wgroup = (16 * wave) / (64 / SUBS);   // as in the forward kernel
   int32_t bid[NB];
 #pragma unroll
-  for (int b = 0; b < NB; b++) bid[b] = core[4 * (b < size ? b : 0)];
-  i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
-#pragma unroll
-  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], (16 * wave) / (64 / SUBS));
+  for (int b = 0; b < NB; b++) bid[b] = core[ES * (b < size ? b : 0)];
+  // (small blocks: the ids of the wavefront's row of small blocks in a tile are read from the tile table where they are
+  // needed; kept for all tiles of the row, they and the arguments do not fit into the scalar registers)
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   const T *pof = reinterpret_cast<const T *>(a.o_in) + z * a.oin_sz + h * a.oin_sh + row * a.oin_ld + 8 * q;
   frag_t xq[NK], oq[NK];
@@ -493,7 +498,8 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   // block-column (v and k tiles) or block id (p) of tile n, from the table (a scalar load; clamped past the end)
   auto tile_key = [&](int n) {
     const int m = n < 2 * size ? (n >> 1) : n - 2 * size;
-    return core[4 * (m < size ? m : size - 1) + ((n < 2 * size && (n & 1)) ? 0 : 1)];
+    const table_ptr e = core + ES * (m < size ? m : size - 1);
+    return (n < 2 * size && (n & 1)) ? e[0] : entry_group<SUBS>(e, wgroup) - wgroup;
   };
   int next_key;
   auto issue = [&](int n, int key) {
@@ -507,10 +513,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
       } else {
         // the tile of p gathered from its small blocks; chunks of absent blocks fetch the start of the tensor instead
         // (every load is issued: the waits count them) and are replaced by zeros when they are read
-        const int m = n >> 1;
-        i32x4 ids = tid_[0];
-#pragma unroll
-        for (int b2 = 1; b2 < NB; b2++) ids = (m == b2) ? tid_[b2] : ids;
+        const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), key, wgroup);
 #pragma unroll
         for (int i = 0; i < LWP; i++) {
           int id = ids[0];
@@ -521,12 +524,12 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         }
       }
     } else if (n < 2 * size) {
-      const T *base = py1 + (int64_t)key * 64 * a.y1_ld;
+      const T *base = py1 + (int64_t)key * (64 / SUBS) * a.y1_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
     } else {
-      const T *base = py2 + (int64_t)key * 64 * a.y2_ld;
+      const T *base = py2 + (int64_t)key * (64 / SUBS) * a.y2_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
@@ -560,6 +563,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
 #pragma unroll
   for (int b = 0; b < NB; b++)
     if (b < size) {
+      const i32x4 ids_b = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
       step(2 * b);
       const unsigned char *tile = ring + ((2 * b) % kStages) * TB;
       frag_t kf[4][NK];
@@ -582,7 +586,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         P8 y, d;
         y.raw = *reinterpret_cast<const u32x4 *>(pt + (((q + 4 * s) ^ pswz) << 4));
         bool here = true;
-        if constexpr (SUBS > 1) here = chunk_block_id<SUBS>(tid_[b], s, q) >= 0;
+        if constexpr (SUBS > 1) here = chunk_block_id<SUBS>(ids_b, s, q) >= 0;
 #pragma unroll
         for (int i = 0; i < 8; i++) {
           const float dp = to_float(from_float<T>(acc[2 * s + (i >> 2)][i & 3]));   // dp as the sdd operator would have stored it
@@ -629,9 +633,10 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
       } else {
         T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
+        const i32x4 ids_b = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-          const int id = chunk_block_id<SUBS>(tid_[b], s, q);
+          const int id = chunk_block_id<SUBS>(ids_b, s, q);
           if (id >= 0)
             *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[b][s]);
         }

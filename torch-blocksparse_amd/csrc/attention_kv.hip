@@ -38,15 +38,18 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   const int64_t n_wg = (int64_t)a.Z * a.R;             // R: work items (columns of tiles, the long ones in parts)
   const int64_t wg = xcd_remap(blockIdx.x, n_wg);
   const int item = (int)(wg % a.R), z = (int)(wg / a.R);
-  const table_ptr lut = as_table(a.lut);                // per item (blocks, offset, head, column, slot of partial results or -1)
-  const int size = lut[8 * item + 0];
-  const int offset = lut[8 * item + 1];
-  const int h = lut[8 * item + 2], bc = lut[8 * item + 3], slot = lut[8 * item + 4];
+  const table_ptr lut = as_table(a.lut);                // per item twelve ints (entries, offset, head, column, slot of partial results or -1, ., ., ., its S block-columns)
+  const int size = lut[12 * item + 0];
+  const int offset = lut[12 * item + 1];
+  const int h = lut[12 * item + 2], slot = lut[12 * item + 4];
   const int qrow = lane & 15, q = lane >> 4;
-  const int64_t key = (int64_t)bc * 64 + wave * 16 + qrow;
+  // the column's 64 keys: S groups of 64 / S consecutive ones (S = SUBS block-columns, anywhere in the matrix); the first
+  // key of the wavefront's 16
+  const int64_t key0 = (int64_t)lut[12 * item + 8 + (16 * wave) / (64 / SUBS)] * (64 / SUBS) + (16 * wave) % (64 / SUBS);
+  const int64_t key = key0 + qrow;
   T *cs = reinterpret_cast<T *>(smem) + wave * 16 * LDK;
-  T *pdk = reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + ((int64_t)bc * 64 + wave * 16) * a.o_ld;
-  T *pdv = reinterpret_cast<T *>(a.o2) + z * a.o2_sz + h * a.o2_sh + ((int64_t)bc * 64 + wave * 16) * a.o2_ld;
+  T *pdk = reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + key0 * a.o_ld;
+  T *pdv = reinterpret_cast<T *>(a.o2) + z * a.o2_sz + h * a.o2_sh + key0 * a.o2_ld;
   f32x4 dk[ND], dv[ND];
 #pragma unroll
   for (int j = 0; j < ND; j++) dk[j] = dv[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -63,7 +66,8 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   const T *py1 = reinterpret_cast<const T *>(a.y1) + z * a.y1_sz + h * a.y1_sh;   // do
   const T *py2 = reinterpret_cast<const T *>(a.y2) + z * a.y2_sz + h * a.y2_sh;   // q
   const T *pin = reinterpret_cast<const T *>(a.p_in) + z * a.pin_sz;
-  const float *pdelta = a.delta + ((int64_t)z * a.H + h) * a.delta_sh + lane;
+  const float *pdelta = a.delta + ((int64_t)z * a.H + h) * a.delta_sh;
+  constexpr int ES = entry_ints<SUBS>();
   int64_t off1[LW], off2[LW];
   int offp[LWP], colp[LWP];
 #pragma unroll
@@ -90,9 +94,12 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   // tile n: block n / 3; its tile of p, its do tile (with delta), its q tile
   const int total = 3 * size;
   auto loads_of = [&](int n) { return n >= total ? 0 : (n % 3 == 0) ? LWP : (n % 3 == 1) ? LW + 1 : LW; };
-  auto tile_key = [&](int n) {   // tile id (p) or row of tiles (do, q), from the table; clamped past the end
+  // tile id (p) or block-row (do, q; small blocks: of the group of rows that this wavefront loads), from the table;
+  // clamped past the end
+  auto tile_key = [&](int n) {
     const int m = n / 3;
-    return core[4 * (m < size ? m : size - 1) + (n % 3 == 0 ? 0 : 1)];
+    const table_ptr e = core + ES * (m < size ? m : size - 1);
+    return n % 3 == 0 ? e[0] : entry_group<SUBS>(e, rs) - rs;
   };
   int next_key;
   auto issue = [&](int n, int key_) {
@@ -118,14 +125,15 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
         }
       }
     } else if (kind == 1) {
-      const T *base = py1 + (int64_t)key_ * 64 * a.y1_ld;
+      const T *base = py1 + (int64_t)key_ * (64 / SUBS) * a.y1_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
       // the 64 delta of the tile's rows: every wavefront loads the same 256 bytes, so that all count the same loads
-      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pdelta + (int64_t)key_ * 64), BSP_LDS_PTR(dring + (n % kStages) * 256), 4, 0, 0);
+      const i32x4 groups = entry_groups<SUBS>(core + ES * (n / 3));
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pdelta + element_position<SUBS>(groups, lane)), BSP_LDS_PTR(dring + (n % kStages) * 256), 4, 0, 0);
     } else {
-      const T *base = py2 + (int64_t)key_ * 64 * a.y2_ld;
+      const T *base = py2 + (int64_t)key_ * (64 / SUBS) * a.y2_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
@@ -156,7 +164,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   for (int b = 0; b < size; b++) {
     i32x4 present = i32x4{0, 0, 0, 0};   // small blocks: the ids of the wavefront's column of small blocks in the tile, by row
     if constexpr (SUBS > 1) {
-      const table_ptr src = as_table(a.tiles) + (int64_t)core[4 * b] * (SUBS * SUBS) + rs;
+      const table_ptr src = as_table(a.tiles) + (int64_t)core[ES * b] * (SUBS * SUBS) + rs;
 #pragma unroll
       for (int r2 = 0; r2 < SUBS; r2++) present[r2] = src[r2 * SUBS];
     }
@@ -253,13 +261,14 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
 }
 
 // dk and dv of the columns that were computed in parts: per (batch, such column) the sum of its parts' slots, in order.
-// a.lut here: per column (head, column, first slot, parts).
-template <typename T, int D>
+// a.lut here: per column eight ints (head, column, first slot, parts, then its S block-columns).
+template <typename T, int D, int SUBS>
 __global__ void __launch_bounds__(256) k_attn64_kv_sum(AttnArgs a) {
   // four workgroups per (batch, column), a quarter of the 2 x 64 x D sums each
   const int quarter = blockIdx.x & 3, col = (blockIdx.x >> 2) % a.R, z = (blockIdx.x >> 2) / a.R;
   const table_ptr lut = as_table(a.lut);
-  const int h = lut[4 * col + 0], bc = lut[4 * col + 1], first = lut[4 * col + 2], parts = lut[4 * col + 3];
+  const int h = lut[8 * col + 0], first = lut[8 * col + 2], parts = lut[8 * col + 3];
+  const i32x4 groups = i32x4{lut[8 * col + 4], lut[8 * col + 5], lut[8 * col + 6], lut[8 * col + 7]};
   const float *ws = a.partial + ((int64_t)z * a.n_slots + first) * (2 * 64 * D);
   constexpr int PER = 64 * D / 4;                        // groups of four values per result
 #pragma unroll
@@ -274,8 +283,9 @@ __global__ void __launch_bounds__(256) k_attn64_kv_sum(AttnArgs a) {
     union { u32x2 raw; T e[4]; } pk;
 #pragma unroll
     for (int e = 0; e < 4; e++) pk.e[e] = from_float<T>(sum[e]);
-    T *dst = which ? reinterpret_cast<T *>(a.o2) + z * a.o2_sz + h * a.o2_sh + ((int64_t)bc * 64 + key) * a.o2_ld
-                   : reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + ((int64_t)bc * 64 + key) * a.o_ld;
+    const int64_t pos = element_position<SUBS>(groups, key);
+    T *dst = which ? reinterpret_cast<T *>(a.o2) + z * a.o2_sz + h * a.o2_sh + pos * a.o2_ld
+                   : reinterpret_cast<T *>(a.o) + z * a.o_sz + h * a.o_sh + pos * a.o_ld;
     *reinterpret_cast<u32x2 *>(dst + 4 * d4) = pk.raw;
   }
 }
@@ -289,7 +299,7 @@ template <typename T, int D, int SUBS> void launch_kv(const AttnArgs &a, hipStre
     AttnArgs b = a;
     b.lut = a.split_lut;
     b.R = a.n_split;
-    hipLaunchKernelGGL((k_attn64_kv_sum<T, D>), dim3((unsigned)((int64_t)a.Z * a.n_split * 4)), wg, 0, st, b);
+    hipLaunchKernelGGL((k_attn64_kv_sum<T, D, SUBS>), dim3((unsigned)((int64_t)a.Z * a.n_split * 4)), wg, 0, st, b);
   }
 }
 

@@ -82,12 +82,16 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
     }
   }
   const int rs = (16 * wave) / (64 / SUBS);
+  constexpr int ES = entry_ints<SUBS>();
   // tile n: block n / 3; its v tile, its tile of p, its k tile
   const int total = 3 * size;
   auto loads_of = [&](int n) { return n >= total ? 0 : (n % 3 == 1) ? LWP : LW; };
-  auto tile_key = [&](int n) {   // block-column (v, k) or tile id (p), from the table; clamped past the end
+  // block-column (v, k; small blocks: of the group of rows that this wavefront loads) or tile id (p), from the table;
+  // clamped past the end
+  auto tile_key = [&](int n) {
     const int m = n / 3;
-    return core[4 * (m < size ? m : size - 1) + (n % 3 == 1 ? 0 : 1)];
+    const table_ptr e = core + ES * (m < size ? m : size - 1);
+    return n % 3 == 1 ? e[0] : entry_group<SUBS>(e, rs) - rs;
   };
   int next_key;
   auto issue = [&](int n, int key) {
@@ -111,12 +115,12 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
         }
       }
     } else if (kind == 0) {
-      const T *base = py1 + (int64_t)key * 64 * a.y1_ld;
+      const T *base = py1 + (int64_t)key * (64 / SUBS) * a.y1_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
     } else {
-      const T *base = py2 + (int64_t)key * 64 * a.y2_ld;
+      const T *base = py2 + (int64_t)key * (64 / SUBS) * a.y2_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
@@ -153,7 +157,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
   for (int j = 0; j < ND; j++) tr_off[j] = second_offset<D>(tr_row, 16 * j + tr_col);
   T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
   for (int b = 0; b < size; b++) {
-    const int tile_id = core[4 * b];
+    const int tile_id = core[ES * b];
     const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), tile_id, rs);
     step(3 * b);
     const unsigned char *tile = ring + ((3 * b) % kStages) * TB;
@@ -269,33 +273,36 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
     off2[i] = (int64_t)r * a.y2_ld + (((((slot >> 1) ^ swz_second<D>(r)) << 1) | (slot & 1)) << 3);
   }
   const int rs = (16 * wave) / (64 / SUBS);
+  constexpr int ES = entry_ints<SUBS>();
   // tile n < size: the k tile of block n (first sweep); then per block its k tile again and its v tile
   const int total = 3 * size;
   auto is_v = [&](int n) { return n >= size && ((n - size) & 1); };
   auto block_of = [&](int n) { return n < size ? n : (n - size) >> 1; };
   auto loads_of = [&](int n) { return n >= total ? 0 : is_v(n) ? LW : LW + (has_kpm ? 1 : 0); };
+  // (small blocks: the block-column of the group of rows that this wavefront loads)
   auto tile_col = [&](int n) {
     const int m = block_of(n < total ? n : total - 1);
-    return core[4 * m + 1];
+    return entry_group<SUBS>(core + ES * m, rs) - rs;
   };
   int next_col;
   auto issue = [&](int n, int col) {
     unsigned char *st = ring + (n % kStages) * TB;
     if (is_v(n)) {
-      const T *base = py2 + (int64_t)col * 64 * a.y2_ld;
+      const T *base = py2 + (int64_t)col * (64 / SUBS) * a.y2_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off2[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
     } else {
-      const T *base = py1 + (int64_t)col * 64 * a.y1_ld;
+      const T *base = py1 + (int64_t)col * (64 / SUBS) * a.y1_ld;
 #pragma unroll
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
       // the 64 key-padding values of the tile's columns: one more load of every wavefront (eight lanes of it; all four
       // write the same 128 bytes, so that all count the same number of loads)
       if (has_kpm) {
+        const i32x4 groups = entry_groups<SUBS>(core + ES * block_of(n));
         if (lane < 8)
-          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pkpm + (int64_t)col * 64 + lane * 8), BSP_LDS_PTR(kraw + (n % kStages) * 128), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pkpm + element_position<SUBS>(groups, lane * 8)), BSP_LDS_PTR(kraw + (n % kStages) * 128), 16, 0, 0);
       }
     }
   };
@@ -326,10 +333,10 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
     advance(n);
   };
   // the mask values of the lane's two chunks of the block in block-column col (address: softmax.py:50-55, 67-70)
-  auto load_masks = [&](int col, P8 (&pr)[2], P8 (&pa)[2]) {
+  auto load_masks = [&](const i32x4 &groups, P8 (&pr)[2], P8 (&pa)[2]) {
 #pragma unroll
     for (int s = 0; s < 2; s++) {
-      const int64_t gcol = (int64_t)col * 64 + 32 * s + 8 * q;
+      const int64_t gcol = chunk_position<SUBS>(groups, s, q);
       const T *attn = reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol;
       const T *rpe = reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol;
       pr[s].load(a.rpe ? rpe : attn);
@@ -397,12 +404,12 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   float m_run = -INFINITY, l_run = 0.f;
   int any_block = SUBS == 1;
   for (int b = 0; b < size; b++) {
-    const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), core[4 * b], rs);
+    const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), core[ES * b], rs);
     if constexpr (SUBS > 1) any_block |= int(chunk_block_id<SUBS>(ids, 0, q) >= 0 || chunk_block_id<SUBS>(ids, 1, q) >= 0);
     P8 pr[2], pa[2];
     if constexpr (EXTRA) {
       arrive(b);
-      load_masks(core[4 * b + 1], pr, pa);
+      load_masks(entry_groups<SUBS>(core + ES * b), pr, pa);
       advance(b);
     } else {
       step(b);
@@ -444,13 +451,13 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   for (int j = 0; j < ND; j++) tr_off[j] = second_offset<D>(tr_row, 16 * j + tr_col);
   T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
   for (int b = 0; b < size; b++) {
-    const int tile_id = core[4 * b];
+    const int tile_id = core[ES * b];
     const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), tile_id, rs);
     const int n = size + 2 * b;
     P8 pr[2], pa[2];
     if constexpr (EXTRA) {
       arrive(n);
-      load_masks(core[4 * b + 1], pr, pa);
+      load_masks(entry_groups<SUBS>(core + ES * b), pr, pa);
       advance(n);
     } else {
       step(n);

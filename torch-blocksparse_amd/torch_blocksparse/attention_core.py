@@ -19,15 +19,49 @@ from .softmax import Softmax, _sparse_softmax
 FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
 MAX_ROW_BLOCKS = 8          # BSP_ATTENTION_MAX_ROW_BLOCKS: longer rows are streamed (the library decides)
 fused_calls = 0             # forward calls that took the fused kernels; tests read it
-# Blocks of 16 and 32 are computed as whole 64 x 64 tiles: a tile costs the same however few of its blocks exist, so
-# below this share of present blocks per present tile the three operators (whose work follows the blocks) are faster.
-# Measured on MI355X, fwd + bwd, head dimension 64, rows of 8 tiles and of 30+ tiles: break-even at 0.5 for blocks of 32;
-# for blocks of 16 the two paths stay within 8 % of each other between 0.15 and 0.3, which way depends on the layout
-# (the 'fixed' layout of the sparse self-attention module's default configuration, 0.26, is 8 % faster fused).
-MIN_TILE_FILL = {16: 0.25, 32: 0.5}
 # dk and dv from the column kernel (bsp_attention_bwd_kv), which computes the softmax gradient again instead of reading it;
 # False: the row kernel stores the gradient and the two products are ordinary dsd operators
 FUSED_KV = os.environ.get('BSP_FUSED_ATTENTION_KV', '1') != '0'
+
+
+
+
+class _GatheredTiles:
+    """64 x 64 tiles over a layout of small blocks (S = 64 / block a side).  A *line* of tiles is S consecutive block-rows;
+    a tile takes the line's S block-rows and S block-columns gathered from anywhere in the line: the columns in which
+    any of the line's block-rows holds a block, in ascending order, S per tile.  (Tiles cut from a fixed grid would be
+    mostly holes wherever the layout has single block-columns, like the global columns of the 'fixed' layouts: a
+    kernel that works on whole tiles then does S times the work.)
+    sizes / starts: tiles per line and the line's first tile, lines in (head, line) order; cols [tiles, S]: the
+    block-columns of a tile (slots past the end of a line repeat the tile's first column); ids [tiles, S, S]: the id of
+    the block at (block-row i of the line, gathered column g), -1 where the layout has none or the slot is padding."""
+
+    def __init__(self, lay, ids, S):
+        H, R, C = lay.shape
+        L = R // S
+        pres = lay.reshape(H, L, S, C).any(2)
+        n = pres.sum(-1).flatten()
+        self.sizes = (n + S - 1) // S
+        self.starts = torch.cumsum(self.sizes, 0) - self.sizes
+        self.n_tiles = int(self.sizes.sum())
+        h, t, c = pres.nonzero().unbind(1)
+        line = h * L + t
+        rank = torch.arange(c.numel()) - (torch.cumsum(n, 0) - n)[line]
+        tile, slot = self.starts[line] + rank // S, rank % S
+        cols = torch.full((self.n_tiles, S), -1, dtype=torch.int64)
+        cols[tile, slot] = c
+        self.cols = torch.where(cols < 0, cols[:, :1], cols)
+        self.ids = torch.full((self.n_tiles, S, S), -1, dtype=torch.int64)
+        for i in range(S):
+            self.ids[tile, i, slot] = ids[h, t * S + i, c]
+        self.lines, self.heads = L, H
+
+    def entries(self):
+        """per tile eight ints: (tile, 0, line, head, then the tile's block-columns, the last repeated up to four)"""
+        t = torch.arange(self.n_tiles)
+        line = torch.repeat_interleave(torch.arange(self.heads * self.lines), self.sizes)
+        cols = self.cols if self.cols.size(1) == 4 else torch.cat((self.cols, self.cols[:, -1:].expand(-1, 4 - self.cols.size(1))), 1)
+        return torch.cat((torch.stack((t, torch.zeros_like(t), line % self.lines, line // self.lines), 1), cols), 1)
 
 
 KV_PART_BLOCKS = 16         # columns of more blocks than this (and than twice the average column) are computed in parts of about this size
@@ -35,23 +69,43 @@ KV_PART_BLOCKS = 16         # columns of more blocks than this (and than twice t
 
 class _ColumnTable:
     """The tables of the column kernel: the layout read along columns, cut into work items.
-    items: per item (blocks, offset of its entries, head, column, slot of its partial sums or -1, 0, 0, 0), then per block
-    (id, row, column, head), a column's blocks by row; the ids are the positions in the row-major order of the nonzero
-    blocks, as everywhere.  A column of more than `part` blocks is cut into parts of near-equal size, each with
-    a slot; split: per such column (head, column, first slot, parts)."""
+    items: per item twelve ints (entries, offset of its entries, head, column, slot of its partial sums or -1, 0, 0, 0, then
+    the column's block-columns, the last repeated up to four), then the entries, a column's by row.  Blocks of 64: a
+    column is a block-column, an entry (id, row, column, head); the ids are the positions in the row-major order of the
+    nonzero blocks, as everywhere.  Smaller blocks: a column is S block-columns of similar length, its entries the tiles
+    of _GatheredTiles over the transposed layout (S block-rows gathered per tile).  A column of more than `part`
+    entries is cut into parts of near-equal size, each with a slot; split: per such column eight ints (head, column,
+    first slot, parts, then its block-columns)."""
 
-    def __init__(self, layout, device, part=None):
+    def __init__(self, layout, device, part=None, S=1, ids=None):
         lay = (layout != 0).cpu()
         H, R, C = lay.shape
-        h, r, c = lay.nonzero().unbind(1)
-        col = h * C + c
-        order = torch.argsort(col * R + r)
-        sizes = torch.bincount(col, minlength=H * C)
+        self.tiles = None
+        if S == 1:
+            h, r, c = lay.nonzero().unbind(1)
+            col = h * C + c
+            order = torch.argsort(col * R + r)
+            sizes = torch.bincount(col, minlength=H * C)
+            starts = torch.cumsum(sizes, 0) - sizes
+            entries = torch.stack((order, r[order], c[order], h[order]), 1)
+            groups = torch.arange(H * C).reshape(H * C, 1) % C
+        else:
+            # a column of tiles: S block-columns of similar length (the longest S of the head, the next S, ...: the global
+            # columns of a layout end up together, and so do neighbouring local ones), so that the block-rows gathered
+            # into a tile hold blocks in most of them
+            layT, idsT = lay.transpose(1, 2), ids.transpose(1, 2)
+            order = torch.argsort(-layT.sum(-1), dim=1, stable=True)                      # [H, C]
+            pick = order[:, :, None].expand(-1, -1, R)
+            g = _GatheredTiles(torch.gather(layT, 1, pick), torch.gather(idsT, 1, pick), S)
+            C = C // S
+            sizes, starts, entries = g.sizes, g.starts, g.entries()
+            self.tiles = g.ids.transpose(1, 2).reshape(-1).to(torch.int32).to(device)     # [tile][gathered block-row][block-column of the group]
+            groups = order.reshape(H * C, S)
+        groups = torch.cat((groups, groups[:, -1:].expand(-1, 4 - groups.size(1))), 1) if groups.size(1) < 4 else groups
         if part is None:
             # only columns that stand out are cut (every part costs a slot written and read): those of more than twice the
             # average length
             part = max(KV_PART_BLOCKS, -(-2 * int(sizes.sum()) // max(1, H * C)))
-        starts = torch.cumsum(sizes, 0) - sizes
         parts = torch.clamp((sizes + part - 1) // part, min=1)
         first_item = torch.cumsum(parts, 0) - parts
         item_col = torch.repeat_interleave(torch.arange(H * C), parts)
@@ -63,9 +117,9 @@ class _ColumnTable:
         is_part = parts[item_col] > 1
         slot = torch.where(is_part, torch.cumsum(is_part.long(), 0) - 1, torch.full_like(count, -1))
         zero = torch.zeros_like(count)
-        header = torch.stack((count, 8 * n_items + 4 * begin, item_col // C, item_col % C, slot, zero, zero, zero), 1).reshape(-1)
-        entries = torch.stack((order, r[order], c[order], h[order]), 1).reshape(-1)
-        self.items = torch.cat((header, entries)).to(torch.int32).to(device)
+        header = torch.cat((torch.stack((count, 12 * n_items + entries.size(1) * begin, item_col // C, item_col % C, slot, zero, zero, zero), 1),
+                            groups[item_col]), 1).reshape(-1)
+        self.items = torch.cat((header, entries.reshape(-1))).to(torch.int32).to(device)
         self.n_items = n_items
         self.columns = C
         self.n_slots = int(is_part.sum())
@@ -73,7 +127,8 @@ class _ColumnTable:
         self.n_split = int(long_cols.numel())
         self.split = None
         if self.n_split:
-            self.split = torch.stack((long_cols // C, long_cols % C, slot[first_item[long_cols]], parts[long_cols]), 1).reshape(-1).to(torch.int32).to(device)
+            self.split = torch.cat((torch.stack((long_cols // C, long_cols % C, slot[first_item[long_cols]], parts[long_cols]), 1),
+                                    groups[long_cols]), 1).reshape(-1).to(torch.int32).to(device)
 
 
 def _vec_ok(t):
@@ -86,9 +141,10 @@ def _vec(t):
 
 
 class AttentionCore:
-    """What the fused kernels need beside the tensors: the softmax table of the layout (of the layout coarsened to 64 x 64
-    tiles, plus the ids of each tile's blocks, when the blocks are 16 or 32) and the two products that stay ordinary
-    operators in the backward pass (dv = p^T . do and dk = ds^T . q)."""
+    """What the fused kernels need beside the tensors: the softmax table of the layout (for blocks of 16 or 32: the table
+    of its 64 x 64 tiles with gathered block-columns and the ids of each tile's blocks), the tables of the column
+    kernel, and the two products that are ordinary operators in the backward pass when the column kernel is not used
+    (dv = p^T . do and dk = ds^T . q)."""
 
     def __init__(self, layout, block, softmax=None):
         self.layout = layout
@@ -117,10 +173,18 @@ class AttentionCore:
             elif R % S or C % S:
                 self._tables[key] = None
             else:
-                cctx, ids = _LayoutOnDevice(self.layout, device).coarse(S)
-                lut, maxlut = _sparse_softmax.make_lut(cctx.lay, 64, device)
-                self._tables[key] = (lut, maxlut, ids.contiguous(), R // S, self.blocks() / max(1, ids.numel()),
-                                     _ColumnTable(cctx.lay, device))
+                # tiles of 64 x 64 with gathered block-columns (rows: forward and the row kernel of the backward pass) and with
+                # gathered block-rows (the column kernel): each view has its own tiles; p lives in the small blocks either way
+                lay = (self.layout != 0).cpu()
+                ids = torch.full(lay.shape, -1, dtype=torch.int64)
+                ids[lay] = torch.arange(int(lay.sum()))
+                g = _GatheredTiles(lay, ids, S)
+                header = torch.stack((g.sizes, 2 * g.sizes.numel() + 8 * g.starts), 1).reshape(-1)
+                lut = torch.cat((header, g.entries().reshape(-1))).to(torch.int32).to(device)
+                maxlut = int(g.sizes.max()) if g.n_tiles else 0
+                ct = _ColumnTable(self.layout, device, S=S, ids=ids)
+                self._tables[key] = (lut, maxlut, g.ids.reshape(-1).to(torch.int32).to(device), R // S,
+                                     self.blocks() / max(1, g.n_tiles * S * S), ct)
         return self._tables[key]
 
     def usable(self, q, k, v, dropout_p=0.):
@@ -137,7 +201,7 @@ class AttentionCore:
         if tuple(q.shape) != (Z, H, R * b, D) or tuple(k.shape) != (Z, H, C * b, D) or tuple(v.shape) != (Z, H, C * b, D):
             return False
         t = self.tables(q.device)
-        if t is None or t[1] <= 0 or t[4] < MIN_TILE_FILL.get(b, 0.):
+        if t is None or t[1] <= 0:
             return False
         return t[1] * 64 < 32768                           # the softmax operator's bound on a row (softmax.py:225-227)
 
@@ -221,7 +285,7 @@ class _attention_core(torch.autograd.Function):
             _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(q), _lib.ptr(v), _lib.ptr(p), _lib.ptr(delta), _lib.ptr(dk), _lib.ptr(dv), Z, H, ct.columns, D,
             do.stride(0), do.stride(1), do.stride(2), q.stride(0), q.stride(1), q.stride(2), v.stride(0), v.stride(1), v.stride(2),
             dk.stride(0), dk.stride(1), dk.stride(2), dv.stride(0), dv.stride(1), dv.stride(2), p.stride(0), delta.stride(1),
-            ctx.core.block, ctx.scale, _lib.ptr(ct.items), ct.n_items, _lib.ptr(ctx.tiles), _lib.ptr(partial), ct.n_slots, _lib.ptr(ct.split), ct.n_split,
+            ctx.core.block, ctx.scale, _lib.ptr(ct.items), ct.n_items, _lib.ptr(ct.tiles), _lib.ptr(partial), ct.n_slots, _lib.ptr(ct.split), ct.n_split,
             _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_bwd_kv')
         return dk, dv
