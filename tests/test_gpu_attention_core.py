@@ -588,6 +588,35 @@ def test_seeded_random_sweep_against_the_three_operators(seed):
         assert float((a.float() - c.float()).abs().max()) <= tol[0 if name in ('o', 'dv') else 1] * ref, (name, block, dh, dtype, Rt, Ct, density, choice)
 
 
+@pytest.mark.parametrize('cfg', [dict(), dict(attention='bidirectional'), dict(stride=128), dict(numverts=4, vertsize=1), dict(block=32, stride=128)])
+def test_fixed_layouts_of_the_module_at_small_blocks(cfg):
+    """The 'fixed' layouts of the sparse self-attention module (local windows plus single global block-columns): the tiles
+    gather the global columns, rows view and columns view; against the dense oracle and the three operators."""
+    torch.manual_seed(17)
+    conf = tb.SparsityConfig(mode='fixed', **cfg)
+    mod = tb.SparseSelfAttention(conf)
+    Z, H, L, dh = 2, 4, 1024, 64
+    q, k, v, do = [torch.randn(Z, H, L, dh, device=DEV).half() for _ in range(4)]
+    sdd, dsd, sm = mod.get_ops(H, L, q.device)
+    lay = sm.layout.cpu()
+    t = ac._core_for(sdd, sm, dsd).tables(q.device)
+    aligned = int(lay.reshape(H, L // 64, 64 // conf.block, L // 64, 64 // conf.block).sum((2, 4)).ne(0).sum(2).max())
+    assert t[1] < aligned                                   # fewer tiles a line than a fixed grid would give
+    res = {}
+    for fused in (True, False):
+        ac.FUSED = fused
+        ts = [x.clone().requires_grad_(True) for x in (q, k, v)]
+        n0 = ac.fused_calls
+        o = mod(*ts)
+        assert (ac.fused_calls - n0) == int(fused)
+        o.backward(do)
+        res[fused] = [o.detach()] + [x.grad for x in ts]
+    ref = D.attention(q, k, v, lay, conf.block, dh ** -0.5, do=do, attn_mask_mode='add')
+    for name, g, c, r in zip(('o', 'dq', 'dk', 'dv'), res[True], res[False], ref):
+        assert float((g.float() - c.float()).abs().max()) <= CHAIN_TOL[torch.float16][1] * float(c.float().abs().max()), name
+        assert_close(g, r, torch.float16, name)
+
+
 def test_c_abi_argument_checks():
     lib = _lib.load()
     t = torch.zeros(1, 1, 64, 64, device=DEV, dtype=torch.float16)
