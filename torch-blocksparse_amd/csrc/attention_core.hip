@@ -85,13 +85,8 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   constexpr int ES = entry_ints<SUBS>();
   const int wgroup = (16 * wave) / (64 / SUBS);   // the group of the tile's rows (k, v: of the gathered columns) that the wavefront's 16 lie in
   int32_t bid[NB];
-  i32x4 bcol[NB];    // the block-column(s) of each tile
 #pragma unroll
-  for (int b = 0; b < NB; b++) {
-    const int bb = b < size ? b : 0;    // blocks past the end repeat the first one (valid to read, never used)
-    bid[b] = core[ES * bb + 0];
-    bcol[b] = entry_groups<SUBS>(core + ES * bb);
-  }
+  for (int b = 0; b < NB; b++) bid[b] = core[ES * (b < size ? b : 0)];   // blocks past the end repeat the first one (valid to read, never used)
   i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
 #pragma unroll
   for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
@@ -167,9 +162,10 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   };
   // the mask values of the lane's two chunks of block b (address: softmax.py:50-55, 67-70)
   auto load_masks = [&](int b, P8 (&pr)[2], P8 (&pa)[2]) {
+    const i32x4 groups = entry_groups<SUBS>(core + ES * (b < size ? b : 0));   // the block-column(s) of the tile
 #pragma unroll
     for (int s = 0; s < 2; s++) {
-      const int64_t gcol = chunk_position<SUBS>(bcol[b < NB ? b : NB - 1], s, q);
+      const int64_t gcol = chunk_position<SUBS>(groups, s, q);
       const T *attn = reinterpret_cast<const T *>(a.attn) + row * a.attn_sr + gcol;
       const T *rpe = reinterpret_cast<const T *>(a.rpe) + z * a.rpe_sz + h * a.rpe_sh + row * a.rpe_sr + gcol;
       pr[s].load(a.rpe ? rpe : attn);
@@ -182,11 +178,11 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   const bool kpm_lane = a.kpm && tid < NB * 8;
   {
     if (kpm_lane) {
-      const int b = tid >> 3;
-      i32x4 col = bcol[0];
-#pragma unroll
-      for (int i = 1; i < NB; i++) col = (b == i) ? bcol[i] : col;
-      kp.load(reinterpret_cast<const T *>(a.kpm) + z * a.kpm_sz + element_position<SUBS>(col, (tid & 7) * 8));
+      // the lane's eight columns of tile b: in one group of the tile; its block-column from the table
+      constexpr int B = 64 / SUBS;
+      const int b = tid >> 3, j = (tid & 7) * 8;
+      const int col = core[ES * (b < size ? b : 0) + (SUBS == 1 ? 1 : 4 + j / B)];
+      kp.load(reinterpret_cast<const T *>(a.kpm) + z * a.kpm_sz + (int64_t)col * B + j % B);
     }
   }
   // the first two tiles always exist (a row has at least one block); in a straight line, so that the wait for the
@@ -455,8 +451,19 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   int32_t bid[NB];
 #pragma unroll
   for (int b = 0; b < NB; b++) bid[b] = core[ES * (b < size ? b : 0)];
-  // (small blocks: the ids of the wavefront's row of small blocks in a tile are read from the tile table where they are
-  // needed; kept for all tiles of the row, they and the arguments do not fit into the scalar registers)
+  // small blocks: the ids of the wavefront's row of small blocks in each tile.  At head dimension 128 they are read from
+  // the tile table where they are needed instead: kept for all tiles of the row, they and the arguments do not fit into
+  // the scalar registers there.
+  constexpr bool KEEP_IDS = D == 64;
+  i32x4 tid_[KEEP_IDS ? NB : 1];
+  if constexpr (KEEP_IDS) {
+#pragma unroll
+    for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+  }
+  auto ids_of = [&](int b) {
+    if constexpr (KEEP_IDS) return tid_[b];
+    else return load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+  };
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   const T *pof = reinterpret_cast<const T *>(a.o_in) + z * a.oin_sz + h * a.oin_sh + row * a.oin_ld + 8 * q;
   frag_t xq[NK], oq[NK];
@@ -513,7 +520,15 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
       } else {
         // the tile of p gathered from its small blocks; chunks of absent blocks fetch the start of the tensor instead
         // (every load is issued: the waits count them) and are replaced by zeros when they are read
-        const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), key, wgroup);
+        i32x4 ids;
+        if constexpr (KEEP_IDS) {
+          const int m = n >> 1;
+          ids = tid_[0];
+#pragma unroll
+          for (int b2 = 1; b2 < NB; b2++) ids = (m == b2) ? tid_[b2] : ids;
+        } else {
+          ids = load_block_ids<SUBS>(as_table(a.tiles), key, wgroup);
+        }
 #pragma unroll
         for (int i = 0; i < LWP; i++) {
           int id = ids[0];
@@ -563,7 +578,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
 #pragma unroll
   for (int b = 0; b < NB; b++)
     if (b < size) {
-      const i32x4 ids_b = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+      const i32x4 ids_b = ids_of(b);
       step(2 * b);
       const unsigned char *tile = ring + ((2 * b) % kStages) * TB;
       frag_t kf[4][NK];
@@ -633,7 +648,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         store_block_rows<T>(stage_p, pout + (int64_t)bid[b] * 4096, __builtin_bit_cast(u32x4, pf[b][0]), __builtin_bit_cast(u32x4, pf[b][1]), lane);
       } else {
         T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
-        const i32x4 ids_b = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+        const i32x4 ids_b = ids_of(b);
 #pragma unroll
         for (int s = 0; s < 2; s++) {
           const int id = chunk_block_id<SUBS>(ids_b, s, q);
