@@ -275,6 +275,7 @@ def main():
     torch.cuda.empty_cache()
     if not args.no_other_configs:
         out['other_configs'] = {str(c): other_config(c, 20, 3) for c in (2, 4, 5)}
+        out['other_configs']['module default'] = module_default_config(20, 5)
     if not args.no_cpu_baseline:
         out['cpu_baseline'] = cpu_baseline(lay, block, dh, scale, 4096)
     print(json.dumps(out))
@@ -482,6 +483,47 @@ def fused_chain_step(w, steps, warmup):
         step()
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def module_default_config(steps, warmup):
+    """The sparse self-attention module as its defaults configure it (deepspeedsparseselfattention.py:13: 'fixed' layout,
+    block 16, stride 64, unidirectional), same batch, heads, sequence and head dimension as the headline: forward +
+    backward through autograd, the three operators (FUSED off) against the fused chain the module calls."""
+    import torch
+    import torch_blocksparse as tb
+    from torch_blocksparse import attention_core as ac
+    dev = torch.device('cuda:0')
+    torch.manual_seed(0)
+    B, H, L, dh = 8, 16, 4096, 64
+    mod = tb.SparseSelfAttention(tb.SparsityConfig())
+    q, k, v = [torch.randn(B, H, L, dh, device=dev, dtype=torch.float16, requires_grad=True) for _ in range(3)]
+    do = torch.randn(B, H, L, dh, device=dev, dtype=torch.float16)
+
+    def step():
+        q.grad = k.grad = v.grad = None
+        mod(q, k, v).backward(do)
+    res = {}
+    old = ac.FUSED
+    try:
+        for name, fused in (('three operators', False), ('fused chain', True)):
+            ac.FUSED = fused
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            res[name] = round((time.perf_counter() - t0) * 1e3 / steps, 4)
+    finally:
+        ac.FUSED = old
+    sdd, dsd, sm = mod.get_ops(H, L, dev)
+    nnz = int((sm.layout != 0).sum())
+    t = ac._core_for(sdd, sm, dsd).tables(dev)
+    torch.cuda.empty_cache()
+    return {'workload': "SparseSelfAttention(SparsityConfig()): 'fixed' layout, block 16, stride 64, unidirectional; batch 8, 16 heads, seq 4096, head_dim 64, fp16, "
+                        'forward + backward', 'blocks_per_head': nnz // H, 'ms_per_step': res,
+            'tiles': {'longest_line': t[1], 'blocks_present_per_tile': round(t[4], 3)}}
 
 
 def other_config(config, steps, warmup):
