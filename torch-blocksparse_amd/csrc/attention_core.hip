@@ -1,4 +1,5 @@
-// The attention chain of one block-row in one kernel, block 64, fp16 / bf16, for gfx950.
+// The attention chain of one block-row in one kernel, blocks of 64 (and, on tiles of 64 x 64 formed from them, of 32
+// and 16), fp16 / bf16, for gfx950.
 //
 // The reference's attention modules run three operators per call: scores = sdd(q, k^T), softmax in place, context =
 // dsd(p, v) (deepspeedsparseselfattention.py:152-157; attention.py:190-202), and autograd adds five more launches for
@@ -10,7 +11,8 @@
 //   forward  : s = q . k^T  ->  p = softmax(s * scale + rpe + key-padding mask + attention mask)  ->  o = p . v
 //              p is written once (the backward pass needs it), o once; the scores are never stored.
 //   backward : dp = do . v^T  ->  ds = p * (dp - sum(p * dp)) * scale  ->  dq = ds . k
-//              p is read once, ds written once (dk = ds^T . q and dv = p^T . do remain ordinary dsd products).
+//              p is read once; ds is written only if the caller wants it (dk = ds^T . q and dv = p^T . do then are
+//              ordinary dsd products; otherwise the column kernel of attention_kv.hip computes both from p).
 //
 // Arithmetic mirrors the separate operators: the scores (and dp) are rounded to the storage type before the softmax
 // sees them, as they are when sdd stores them; the softmax is computed in fp32 (log2 domain) and rounded before the
@@ -23,6 +25,11 @@
 // of the block (s = 0, 1): eight consecutive keys, which is at once a 16-byte piece of a row of p (stored as it is) and
 // the B-operand fragment of the second product o^T = v^T . p^T (no shuffle, no LDS round trip).  v^T comes from the v
 // tile in LDS through the transposing LDS read.
+//
+// Blocks of 32 / 16 (SUBS = 2 / 4): a tile is SUBS consecutive block-rows by SUBS block-columns gathered from anywhere in
+// those rows (the tile's table entry names them): its 64 k / v rows are SUBS groups of consecutive rows, a wavefront
+// loads 16 rows, which lie in one group, and the lane's 8-key chunk lies in one small block, whose id (-1: absent) comes
+// from the tile table.
 #include "attention_common.h"
 
 namespace bsp {

@@ -9,6 +9,10 @@
 // row): the table's work items are columns or, for long columns, parts of them, whose sums go to fp32 slots that a
 // second small kernel adds in order (no atomics: the same bits every time).
 //
+// Blocks of 16 / 32 (SUBS = 4 / 2): a column of tiles is SUBS block-columns that need not be neighbours (the work item
+// names them), and a tile's 64 rows are SUBS groups of consecutive rows gathered from anywhere (the tile's table entry
+// names the block-row of each group); the tile of p is gathered from the small blocks by their ids.
+//
 // A wavefront owns 16 of the column's 64 keys for all rows.  Per block of the column, three tiles through the ring:
 //   p    [row][key]  read transposed (a lane: its key, 8 consecutive rows)              -> operand of dv, factor of ds
 //   do   [row][d]    read along d for dp = do . v^T (the lane's v fragment stays in registers) and transposed for
