@@ -125,6 +125,9 @@ template <typename T, int D> __device__ __forceinline__ void store_rows(T *cs, T
 // LDS (rows of 72 elements), then two stores of 1 KiB of consecutive addresses.  (Stored straight from the registers,
 // every store instruction writes sixteen separate 64-byte pieces: measured, the forward kernel then takes 170 us
 // instead of 107 without the stores.)
+// The stores are non-temporal: p is 336 MB in the benchmark configuration, more than the caches hold, and is next read
+// by the backward pass; stored the ordinary way it pushes the k and v tiles that the block-rows of a (batch, head) share
+// out of L2 (forward kernel 144 us, with non-temporal stores 114 us).
 template <typename T> __device__ __forceinline__ void store_block_rows(T *cs, T *dst, const u32x4 &c0, const u32x4 &c1, int lane) {
   T *w = cs + (lane & 15) * 72 + 8 * (lane >> 4);
   *reinterpret_cast<u32x4 *>(w) = c0;
@@ -133,15 +136,15 @@ template <typename T> __device__ __forceinline__ void store_block_rows(T *cs, T 
 #pragma unroll
   for (int i = 0; i < 2; i++) {
     const int c = lane + 64 * i;
-    *reinterpret_cast<u32x4 *>(dst + c * 8) = *reinterpret_cast<const u32x4 *>(cs + (c >> 3) * 72 + (c & 7) * 8);
+    __builtin_nontemporal_store(*reinterpret_cast<const u32x4 *>(cs + (c >> 3) * 72 + (c & 7) * 8), reinterpret_cast<u32x4 *>(dst + c * 8));
   }
   __builtin_amdgcn_wave_barrier();
 }
 
-// Blocks of 16 and 32 (SUBS = 64 / block > 1): the kernels work on 64 x 64 tiles of the layout (a tile is present if any
-// of its SUBS x SUBS blocks is); the table is the softmax table of the layout coarsened to tiles and `tiles` holds, per
-// tile in that table's order, the ids of its blocks row by row, -1 where absent.  A wavefront's 16 rows lie in one row
-// of small blocks (rs) and a lane's chunk of 8 columns in one small block: its id, or -1.
+// Blocks of 16 and 32 (SUBS = 64 / block > 1): the kernels work on 64 x 64 tiles formed from SUBS x SUBS small blocks
+// (SUBS consecutive block-rows by SUBS gathered block-columns, or the other way round in the column kernel); the table
+// lists the tiles of each line and `tiles` holds, per tile, the ids of its blocks row by row, -1 where absent.  A
+// wavefront's 16 rows lie in one row of small blocks (rs) and a lane's chunk of 8 columns in one small block: its id, or -1.
 // t = the ids of the wavefront's row of small blocks in the tile (scalars, fetched once per block of the row; kept as a
 // vector type: an array indexed in a select chain ends up in scratch memory, whose loads count as vector-memory
 // operations and stall every wait of the tile ring)

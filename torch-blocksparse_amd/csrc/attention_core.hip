@@ -403,7 +403,7 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
         for (int s = 0; s < 2; s++) {
           const int id = chunk_block_id<SUBS>(tid_[b], s, q);
           if (id >= 0)
-            *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[b][s]);
+            __builtin_nontemporal_store(__builtin_bit_cast(u32x4, pf[b][s]), reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)));
         }
       }
     }
@@ -660,7 +660,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         for (int s = 0; s < 2; s++) {
           const int id = chunk_block_id<SUBS>(ids_b, s, q);
           if (id >= 0)
-            *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[b][s]);
+            __builtin_nontemporal_store(__builtin_bit_cast(u32x4, pf[b][s]), reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)));
         }
       }
     }

@@ -211,7 +211,7 @@ if (a.p_out == nullptr) continue;   // ds is not asked for
       for (int s = 0; s < 2; s++) {
         const int id = chunk_block_id<SUBS>(ids, s, q);
         if (id >= 0)
-          *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[s]);
+          __builtin_nontemporal_store(__builtin_bit_cast(u32x4, pf[s]), reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)));
       }
     }
   }
@@ -494,7 +494,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
       for (int s = 0; s < 2; s++) {
         const int id = chunk_block_id<SUBS>(ids, s, q);
         if (id >= 0)
-          *reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)) = __builtin_bit_cast(u32x4, pf[s]);
+          __builtin_nontemporal_store(__builtin_bit_cast(u32x4, pf[s]), reinterpret_cast<u32x4 *>(pz + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + chunk_in_block<SUBS>(wave, qrow, s, q)));
       }
     }
   }

@@ -51,7 +51,7 @@ class _GatheredTiles:
         cols = torch.full((self.n_tiles, S), -1, dtype=torch.int64)
         cols[tile, slot] = c
         self.cols = torch.where(cols < 0, cols[:, :1], cols)
-        self.ids = torch.full((self.n_tiles, S, S), -1, dtype=torch.int64)
+        self.ids = torch.full((self.n_tiles, S, S), -1, dtype=ids.dtype)
         for i in range(S):
             self.ids[tile, i, slot] = ids[h, t * S + i, c]
         self.lines, self.heads = L, H
@@ -176,8 +176,8 @@ class AttentionCore:
                 # tiles of 64 x 64 with gathered block-columns (rows: forward and the row kernel of the backward pass) and with
                 # gathered block-rows (the column kernel): each view has its own tiles; p lives in the small blocks either way
                 lay = (self.layout != 0).cpu()
-                ids = torch.full(lay.shape, -1, dtype=torch.int64)
-                ids[lay] = torch.arange(int(lay.sum()))
+                ids = torch.full(lay.shape, -1, dtype=torch.int32)
+                ids[lay] = torch.arange(int(lay.sum()), dtype=torch.int32)
                 g = _GatheredTiles(lay, ids, S)
                 header = torch.stack((g.sizes, 2 * g.sizes.numel() + 8 * g.starts), 1).reshape(-1)
                 lut = torch.cat((header, g.entries().reshape(-1))).to(torch.int32).to(device)
