@@ -38,6 +38,9 @@ namespace {
 // tile is 16 KiB and a launch may ask for 64 KiB of dynamic LDS without further ado
 template <int D> constexpr int ring_stages() { return D == 64 ? 4 : 3; }
 
+// cache-policy argument of the direct-to-LDS load for data that is read once (the tiles of p in the backward kernels): the
+// non-temporal bit, so that the lines do not displace the dense tiles that the workgroups of a (batch, head) share
+#define BSP_LOAD_ONCE 2
 #define BSP_GLOBAL_PTR(p) ((const void __attribute__((address_space(1))) *)(p))
 #define BSP_LDS_PTR(p) ((void __attribute__((address_space(3))) *)(p))
 // Wait until at most n vector-memory operations of this wavefront are outstanding AND all of its LDS reads have returned.

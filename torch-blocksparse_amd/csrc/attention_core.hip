@@ -523,7 +523,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
         const T *base = pin + (int64_t)key * 4096;
 #pragma unroll
         for (int i = 0; i < LWP; i++)
-          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, BSP_LOAD_ONCE);
       } else {
         // the tile of p gathered from its small blocks; chunks of absent blocks fetch the start of the tensor instead
         // (every load is issued: the waits count them) and are replaced by zeros when they are read
@@ -542,7 +542,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
 #pragma unroll
           for (int c = 1; c < SUBS; c++) id = (colp[i] == c) ? ids[c] : id;
           const T *src = id >= 0 ? pin + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + offp[i] : pin;
-          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(src), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(src), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, BSP_LOAD_ONCE);
         }
       }
     } else if (n < 2 * size) {
