@@ -321,9 +321,9 @@ int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, 
  * offset of the first entry in ints from the start, head, column, slot, 0, 0, 0, then the column's S block-columns,
  * the last repeated up to four), then the entries, a column's by row.  Block 64: a column is a block-column, an entry
  * four ints (id, row, column, head).  Blocks 16 / 32: a column is any S block-columns of a head (every block-column
- * in exactly one; the kernel takes the wavefronts' keys from them), an entry a tile of eight ints (tile index, ., ., .,
- * then the S block-rows gathered into it), and d_tiles gives per tile the ids [gathered block-row][block-column of the
- * column] (tiles of this call's own numbering, not those of bsp_attention_fwd / _bwd).  A work item is a
+ * in exactly one; the kernel takes the wavefronts' keys from them), an entry a tile of 8 + S * S ints (., ., ., ., the S
+ * block-rows gathered into it, then the ids of its blocks, [gathered block-row][block-column of the column], -1 where
+ * the layout has none).  A work item is a
  * whole column (slot -1; also every column without blocks, whose rows of dk and dv are set to zero) or one part of a
  * long column: columns differ in length far more than rows do, so the caller cuts the long ones into parts, whose
  * partial sums go to fp32 slots (partial: [Z][n_slots][2][64][D] floats, slot = the item's) and are added in order by a
@@ -335,8 +335,8 @@ int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, const void *
                          int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t v_stride_z, int64_t v_stride_h,
                          int64_t ldv, int64_t dk_stride_z, int64_t dk_stride_h, int64_t lddk, int64_t dv_stride_z,
                          int64_t dv_stride_h, int64_t lddv, int64_t p_stride_z, int64_t delta_stride_h, int block,
-                         float scale, const int32_t *d_col_lut, int n_items, const int32_t *d_tiles, float *partial,
-                         int n_slots, const int32_t *d_split_lut, int n_split, void *stream);
+                         float scale, const int32_t *d_col_lut, int n_items, float *partial, int n_slots,
+                         const int32_t *d_split_lut, int n_split, void *stream);
 
 /* ---------------------------------------------------------------------------------------------------
  * Dense utility ops of the reference package.

@@ -106,7 +106,8 @@ def test_column_table_of_small_blocks(S, seed):
     lay[:, :, 2 * S + 1] = True                          # and another one, in another aligned group of S
     ids = _ids_of(lay)
     ct = _ColumnTable(lay.long(), 'cpu', part=3, S=S, ids=ids)
-    t, tiles = ct.items.tolist(), ct.tiles.tolist()
+    t = ct.items.tolist()
+    ES = 8 + S * S
     assert ct.columns == C // S
     seen, cols_seen = set(), {h: [] for h in range(H)}
     per_column = {}
@@ -116,12 +117,13 @@ def test_column_table_of_small_blocks(S, seed):
         per_column.setdefault((h, c), (groups, []))
         assert per_column[(h, c)][0] == groups
         for e in range(count):
-            tile, _, c2, h2 = t[offset + 8 * e:offset + 8 * e + 4]
-            rows = t[offset + 8 * e + 4:offset + 8 * e + 4 + S]
+            tile, _, c2, h2 = t[offset + ES * e:offset + ES * e + 4]
+            rows = t[offset + ES * e + 4:offset + ES * e + 4 + S]
+            tiles = t[offset + ES * e + 8:offset + ES * (e + 1)]
             assert (c2, h2) == (c, h)
             for i2, r in enumerate(rows):
                 for gidx, col in enumerate(groups):
-                    b = tiles[tile * S * S + i2 * S + gidx]
+                    b = tiles[i2 * S + gidx]
                     if b >= 0:
                         assert bool(lay[h, r, col]) and int(ids[h, r, col]) == b and b not in seen
                         seen.add(b)

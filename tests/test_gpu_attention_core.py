@@ -645,15 +645,14 @@ def test_c_abi_argument_checks():
     delta = torch.zeros(1, 1, 64, device=DEV)
     dk, dv = t.clone(), t.clone()
 
-    def kv(dtype=0, D=64, block=64, n_items=ct.n_items, lddk=64, delta=delta, n_slots=0, partial=null, tiles=null):
+    def kv(dtype=0, D=64, block=64, n_items=ct.n_items, lddk=64, delta=delta, n_slots=0, partial=null):
         return lib.bsp_attention_bwd_kv(dtype, _lib.ptr(t), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(delta), _lib.ptr(dk), _lib.ptr(dv),
                                         1, 1, 1, D, *st, *st, *st, st[0], st[1], lddk, *st, p.stride(0), 64, block, 1.0, _lib.ptr(ct.items), n_items,
-                                        tiles, partial, n_slots, null, 0, _lib.stream_ptr(torch.device(DEV)))
+                                        partial, n_slots, null, 0, _lib.stream_ptr(torch.device(DEV)))
     assert kv() == _lib.OK
     assert kv(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
     assert kv(D=96) == _lib.ERR_UNSUPPORTED
     assert kv(block=128) == _lib.ERR_UNSUPPORTED
-    assert kv(block=16) != _lib.OK                      # small blocks need the tile table
     assert kv(n_items=0) != _lib.OK                     # fewer work items than columns
     assert kv(lddk=60) != _lib.OK
     assert kv(delta=None) != _lib.OK

@@ -780,15 +780,13 @@ extern "C" int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, c
                                     int64_t v_stride_h, int64_t ldv, int64_t dk_stride_z, int64_t dk_stride_h, int64_t lddk,
                                     int64_t dv_stride_z, int64_t dv_stride_h, int64_t lddv, int64_t p_stride_z,
                                     int64_t delta_stride_h, int block, float scale, const int32_t *d_col_lut, int n_items,
-                                    const int32_t *d_tiles, float *partial, int n_slots, const int32_t *d_split_lut,
-                                    int n_split, void *stream) {
+                                    float *partial, int n_slots, const int32_t *d_split_lut, int n_split, void *stream) {
   if (!d_o || !q || !v || !p || !delta || !dk || !dv || !d_col_lut || Z <= 0 || H <= 0 || C <= 0 || delta_stride_h < 0 || n_items < H * C)
     return BSP_ERR_ARG;
   if (n_slots < 0 || n_split < 0 || (n_slots > 0) != (n_split > 0) || (n_slots > 0 && (!partial || !d_split_lut)) || n_items > H * C + n_slots)
     return BSP_ERR_ARG;
   if (reinterpret_cast<uintptr_t>(partial) & 15) return BSP_ERR_ARG;
   if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
-  if ((block != 64) != (d_tiles != nullptr)) return BSP_ERR_ARG;
   const void *ptrs[] = {d_o, q, v, p, dk, dv};
   for (const void *ptr : ptrs)
     if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0) return BSP_ERR_ARG;
@@ -809,7 +807,7 @@ extern "C" int bsp_attention_bwd_kv(int dtype, const void *d_o, const void *q, c
   a.o_sz = dk_stride_z; a.o_sh = dk_stride_h; a.o_ld = lddk;
   a.o2_sz = dv_stride_z; a.o2_sh = dv_stride_h; a.o2_ld = lddv;
   a.pin_sz = p_stride_z;
-  a.scale = scale; a.lut = d_col_lut; a.tiles = d_tiles;
+  a.scale = scale; a.lut = d_col_lut;
   a.Z = Z; a.H = H; a.R = n_items;
   const int rc = attention_kv(dtype, a, D, block, as_stream(stream));
   if (rc != BSP_OK) return rc;

@@ -11,7 +11,7 @@
 //
 // Blocks of 16 / 32 (SUBS = 4 / 2): a column of tiles is SUBS block-columns that need not be neighbours (the work item
 // names them), and a tile's 64 rows are SUBS groups of consecutive rows gathered from anywhere (the tile's table entry
-// names the block-row of each group); the tile of p is gathered from the small blocks by their ids.
+// names the block-row of each group and the ids of its blocks); the tile of p is gathered from the small blocks.
 //
 // A wavefront owns 16 of the column's 64 keys for all rows.  Per block of the column, three tiles through the ring:
 //   p    [row][key]  read transposed (a lane: its key, 8 consecutive rows)              -> operand of dv, factor of ds
@@ -71,7 +71,10 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   const T *py2 = reinterpret_cast<const T *>(a.y2) + z * a.y2_sz + h * a.y2_sh;   // q
   const T *pin = reinterpret_cast<const T *>(a.p_in) + z * a.pin_sz;
   const float *pdelta = a.delta + ((int64_t)z * a.H + h) * a.delta_sh;
-  constexpr int ES = entry_ints<SUBS>();
+  // entries of the table: blocks of 64 four ints (id, block-row, ., .); smaller blocks 8 + SUBS * SUBS ints: (., ., ., ., the
+  // block-rows of the tile's SUBS groups of rows, then the ids of its blocks, [group of rows][block-column], -1 where
+  // absent).  Everything a tile needs comes from its entry, fetched a step ahead of its use.
+  constexpr int ES = SUBS == 1 ? 4 : 8 + SUBS * SUBS;
   int64_t off1[LW], off2[LW];
   int offp[LWP], colp[LWP];
 #pragma unroll
@@ -105,8 +108,21 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
     const table_ptr e = core + ES * (m < size ? m : size - 1);
     return n % 3 == 0 ? e[0] : entry_group<SUBS>(e, rs) - rs;
   };
+  // small blocks, with the tile's key: the ids of the blocks in the wavefront's group of rows (tile of p: what it
+  // gathers) or the block-rows of all groups (do tile: where the rows' delta lie)
+  auto tile_vec = [&](int n) {
+    i32x4 t = i32x4{0, 0, 0, 0};
+    if constexpr (SUBS > 1) {
+      const int m = n / 3;
+      const table_ptr e = core + ES * (m < size ? m : size - 1) + (n % 3 == 0 ? 8 + rs * SUBS : 4);
+#pragma unroll
+      for (int c = 0; c < SUBS; c++) t[c] = e[c];
+    }
+    return t;
+  };
   int next_key;
-  auto issue = [&](int n, int key_) {
+  i32x4 next_vec;
+  auto issue = [&](int n, int key_, const i32x4 &vec) {
     unsigned char *st = ring + (n % kStages) * TB;
     const int kind = n % 3;
     if (kind == 0) {
@@ -118,12 +134,11 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
       } else {
         // gathered from the small blocks; chunks of absent blocks fetch the start of the tensor (every load is issued:
         // the waits count them) and are replaced by zeros when they are read
-        const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), key_, rs);
 #pragma unroll
         for (int i = 0; i < LWP; i++) {
-          int id = ids[0];
+          int id = vec[0];
 #pragma unroll
-          for (int c = 1; c < SUBS; c++) id = (colp[i] == c) ? ids[c] : id;
+          for (int c = 1; c < SUBS; c++) id = (colp[i] == c) ? vec[c] : id;
           const T *src = id >= 0 ? pin + (int64_t)id * ((64 / SUBS) * (64 / SUBS)) + offp[i] : pin;
           __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(src), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, BSP_LOAD_ONCE);
         }
@@ -134,8 +149,8 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
       for (int i = 0; i < LW; i++)
         __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + off1[i]), BSP_LDS_PTR(st + (wave * LW + i) * 1024), 16, 0, 0);
       // the 64 delta of the tile's rows: every wavefront loads the same 256 bytes, so that all count the same loads
-      const i32x4 groups = entry_groups<SUBS>(core + ES * (n / 3));
-      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pdelta + element_position<SUBS>(groups, lane)), BSP_LDS_PTR(dring + (n % kStages) * 256), 4, 0, 0);
+      const int64_t drow = SUBS == 1 ? (int64_t)key_ * 64 + lane : element_position<SUBS>(vec, lane);
+      __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(pdelta + drow), BSP_LDS_PTR(dring + (n % kStages) * 256), 4, 0, 0);
     } else {
       const T *base = py2 + (int64_t)key_ * (64 / SUBS) * a.y2_ld;
 #pragma unroll
@@ -148,12 +163,25 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (n + kStages - 1 < total) issue(n + kStages - 1, next_key);
+    if (n + kStages - 1 < total) issue(n + kStages - 1, next_key, next_vec);
     next_key = tile_key(n + kStages);
+    next_vec = tile_vec(n + kStages);
   };
 #pragma unroll
-  for (int n = 0; n < kStages - 1; n++) issue(n, tile_key(n));   // (a column has at least one block: three tiles)
+  for (int n = 0; n < kStages - 1; n++) issue(n, tile_key(n), tile_vec(n));   // (a column has at least one block: three tiles)
   next_key = tile_key(kStages - 1);
+  next_vec = tile_vec(kStages - 1);
+  // small blocks: the ids of the wavefront's column of small blocks in a tile, by group of rows; fetched a block ahead
+  auto column_ids = [&](int b) {
+    i32x4 t = i32x4{0, 0, 0, 0};
+    if constexpr (SUBS > 1) {
+      const table_ptr e = core + ES * (b < size ? b : size - 1) + 8 + rs;
+#pragma unroll
+      for (int r2 = 0; r2 < SUBS; r2++) t[r2] = e[r2 * SUBS];
+    }
+    return t;
+  };
+  i32x4 present_next = column_ids(0);
 
   const int krow0 = 8 * (qrow >> 2) + (qrow & 3);
   const int tr_row = q * 8 + (qrow >> 2), tr_col = (qrow & 3) * 4;
@@ -166,12 +194,8 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   }
   const uint32_t tr_p = second_offset<64>(tr_row, 16 * wave + tr_col);
   for (int b = 0; b < size; b++) {
-    i32x4 present = i32x4{0, 0, 0, 0};   // small blocks: the ids of the wavefront's column of small blocks in the tile, by row
-    if constexpr (SUBS > 1) {
-      const table_ptr src = as_table(a.tiles) + (int64_t)core[ES * b] * (SUBS * SUBS) + rs;
-#pragma unroll
-      for (int r2 = 0; r2 < SUBS; r2++) present[r2] = src[r2 * SUBS];
-    }
+    const i32x4 present = present_next;
+    present_next = column_ids(b + 1);
     step(3 * b);
     frag_t pf[2];
     {

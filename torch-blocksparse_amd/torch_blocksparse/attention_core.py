@@ -73,14 +73,14 @@ class _ColumnTable:
     the column's block-columns, the last repeated up to four), then the entries, a column's by row.  Blocks of 64: a
     column is a block-column, an entry (id, row, column, head); the ids are the positions in the row-major order of the
     nonzero blocks, as everywhere.  Smaller blocks: a column is S block-columns of similar length, its entries the tiles
-    of _GatheredTiles over the transposed layout (S block-rows gathered per tile).  A column of more than `part`
+    of _GatheredTiles over the transposed layout (S block-rows gathered per tile): 8 + S * S ints, the last S * S the ids
+    of the tile's blocks, [gathered block-row][block-column of the group].  A column of more than `part`
     entries is cut into parts of near-equal size, each with a slot; split: per such column eight ints (head, column,
     first slot, parts, then its block-columns)."""
 
     def __init__(self, layout, device, part=None, S=1, ids=None):
         lay = (layout != 0).cpu()
         H, R, C = lay.shape
-        self.tiles = None
         if S == 1:
             h, r, c = lay.nonzero().unbind(1)
             col = h * C + c
@@ -98,8 +98,9 @@ class _ColumnTable:
             pick = order[:, :, None].expand(-1, -1, R)
             g = _GatheredTiles(torch.gather(layT, 1, pick), torch.gather(idsT, 1, pick), S)
             C = C // S
-            sizes, starts, entries = g.sizes, g.starts, g.entries()
-            self.tiles = g.ids.transpose(1, 2).reshape(-1).to(torch.int32).to(device)     # [tile][gathered block-row][block-column of the group]
+            # an entry carries the ids of its tile's blocks, [gathered block-row][block-column of the group]
+            sizes, starts = g.sizes, g.starts
+            entries = torch.cat((g.entries(), g.ids.transpose(1, 2).reshape(g.n_tiles, S * S).to(torch.int64)), 1)
             groups = order.reshape(H * C, S)
         groups = torch.cat((groups, groups[:, -1:].expand(-1, 4 - groups.size(1))), 1) if groups.size(1) < 4 else groups
         if part is None:
@@ -285,7 +286,7 @@ class _attention_core(torch.autograd.Function):
             _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(q), _lib.ptr(v), _lib.ptr(p), _lib.ptr(delta), _lib.ptr(dk), _lib.ptr(dv), Z, H, ct.columns, D,
             do.stride(0), do.stride(1), do.stride(2), q.stride(0), q.stride(1), q.stride(2), v.stride(0), v.stride(1), v.stride(2),
             dk.stride(0), dk.stride(1), dk.stride(2), dv.stride(0), dv.stride(1), dv.stride(2), p.stride(0), delta.stride(1),
-            ctx.core.block, ctx.scale, _lib.ptr(ct.items), ct.n_items, _lib.ptr(ct.tiles), _lib.ptr(partial), ct.n_slots, _lib.ptr(ct.split), ct.n_split,
+            ctx.core.block, ctx.scale, _lib.ptr(ct.items), ct.n_items, _lib.ptr(partial), ct.n_slots, _lib.ptr(ct.split), ct.n_split,
             _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_bwd_kv')
         return dk, dv
