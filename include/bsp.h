@@ -274,16 +274,16 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  * the three operators.  Rows of at most BSP_ATTENTION_MAX_ROW_BLOCKS tiles of 64 x 64 are held in registers; longer
  * rows (up to the softmax operator's 32768 elements) are streamed: forward in two sweeps over the row (running maximum
  * and sum first, then p and p . v), backward with dq accumulated block by block.
- *   block 64: d_lut / maxlut from bsp_softmax_lut_build on the layout, R = its block-rows, d_tiles = NULL.
+ *   block 64: d_lut / maxlut from bsp_softmax_lut_build on the layout, R = its block-rows.
  *   blocks 16 and 32 (S = 64 / block, layout sides divisible by S): the kernels work on 64 x 64 tiles that the caller
  *             forms: a line of tiles is S consecutive block-rows, and a tile takes S block-columns gathered from
  *             anywhere in the line (in practice: the columns in which any of the line's block-rows holds a block,
  *             ascending, S per tile, so that single block-columns do not cost whole tiles).  R = lines.  d_lut: per
- *             (head, line) two ints (tiles, offset of the first entry in ints from the start), then per tile eight
- *             ints (tile index, ., ., ., then its S block-columns; unused slots repeat a valid column).  d_tiles: per
- *             tile, by tile index, S * S ints: the ids of its blocks in the [Z, nnz, block, block] tensor,
- *             [block-row of the line][gathered block-column], -1 where the layout has none.  maxlut = the most
- *             tiles of a line.
+ *             (head, line) two ints (tiles, offset of the first entry in ints from the start), then per tile
+ *             8 + S * S ints (., ., ., ., its S block-columns, the last repeated up to four; then the ids of its blocks
+ *             in the [Z, nnz, block, block] tensor, [block-row of the line][gathered block-column], -1 where the layout
+ *             has none; unused column slots repeat a valid column and hold no block).  maxlut = the most tiles of a
+ *             line.
  *   forward : p = softmax(round(q . k^T) * scale + rpe + kpm + attn) over each row's nonzero blocks, o = p . v.
  *             q, o: [Z, H, rows, D]; k, v: [Z, H, columns, D], unit stride along D; p: [Z, nnz, block, block] (every
  *             block is written); rows of o without any block are set to zero.  Masks as for bsp_softmax_fwd.
@@ -303,7 +303,7 @@ int bsp_attention_fwd(int dtype, const void *q, const void *k, const void *v, vo
                       int D, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t k_stride_z, int64_t k_stride_h,
                       int64_t ldk, int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t o_stride_z,
                       int64_t o_stride_h, int64_t ldo, int64_t p_stride_z, int block, float scale, const int32_t *d_lut,
-                      int maxlut, const int32_t *d_tiles, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h,
+                      int maxlut, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h,
                       int64_t rpe_stride_r, const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn,
                       int64_t attn_stride_r, int attn_mul, void *stream);
 int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, const void *p, const void *o, void *ds,
@@ -311,7 +311,7 @@ int bsp_attention_bwd(int dtype, const void *d_o, const void *v, const void *k, 
                       int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                       int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                       int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                      const int32_t *d_lut, int maxlut, const int32_t *d_tiles, float *delta, int64_t delta_stride_h,
+                      const int32_t *d_lut, int maxlut, float *delta, int64_t delta_stride_h,
                       void *stream);
 /* dk and dv of the same chain in one launch, one workgroup per column of 64 x 64 tiles: dv = p^T . do and
  * dk = ds^T . q with ds computed again from p (the formula above), delta = the row sums that bsp_attention_bwd wrote

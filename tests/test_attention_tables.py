@@ -67,7 +67,7 @@ def test_gathered_tiles_hold_every_block_once(S, seed, density):
     lay[1, S, :] = True                                  # a full block-row
     ids = _ids_of(lay)
     g = _GatheredTiles(lay, ids, S)
-    assert g.entries().shape == (g.n_tiles, 8)
+    assert g.entries().shape == (g.n_tiles, 8 + S * S)
     seen = set()
     for line in range(H * (R // S)):
         h, t = divmod(line, R // S)
@@ -77,7 +77,7 @@ def test_gathered_tiles_hold_every_block_once(S, seed, density):
         for k in range(int(g.sizes[line])):
             tile = int(g.starts[line]) + k
             e = g.entries()[tile].tolist()
-            assert e[:4] == [tile, 0, t, h] and e[4:4 + S] == g.cols[tile].tolist()
+            assert e[:4] == [tile, 0, t, h] and e[4:4 + S] == g.cols[tile].tolist() and e[8:] == g.ids[tile].flatten().tolist()
             for slot in range(S):
                 c = int(g.cols[tile, slot])
                 assert 0 <= c < C

@@ -625,15 +625,13 @@ def test_c_abi_argument_checks():
     null = ctypes.c_void_p(0)
     st = (t.stride(0), t.stride(1), t.stride(2))
 
-    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64, tiles=null, rpe=null):
+    def fwd(dtype=0, q=t, D=64, block=64, maxlut=maxlut, ldq=64, rpe=null):
         return lib.bsp_attention_fwd(dtype, _lib.ptr(q), _lib.ptr(t), _lib.ptr(t), _lib.ptr(p), _lib.ptr(t.clone()), 1, 1, 1, D,
-                                     st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut, tiles,
+                                     st[0], st[1], ldq, *st, *st, *st, p.stride(0), block, 1.0, _lib.ptr(lut), maxlut,
                                      rpe, 0, 0, 64, null, 0, 0, null, 0, 0, _lib.stream_ptr(torch.device(DEV)))
     assert fwd() == _lib.OK
     assert fwd(dtype=_lib.F32) == _lib.ERR_UNSUPPORTED
     assert fwd(block=128) == _lib.ERR_UNSUPPORTED
-    assert fwd(block=32) != _lib.OK                     # small blocks need the tile table
-    assert fwd(tiles=_lib.ptr(lut)) != _lib.OK          # ... and blocks of 64 take none
     assert fwd(D=96) == _lib.ERR_UNSUPPORTED
     assert fwd(maxlut=9) == _lib.OK                     # (the streaming kernels; the table's rows hold one block)
     assert fwd(maxlut=9, rpe=_lib.ptr(t)) == _lib.OK

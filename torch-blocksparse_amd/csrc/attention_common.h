@@ -21,7 +21,6 @@ struct AttnArgs {
   float *partial;            // ... the slots of the long columns' parts, [Z][n_slots][dk, dv][64][D]
   const int32_t *split_lut;  // ... per long column (head, column, first slot, parts)
   int n_slots, n_split;
-  const int32_t *tiles;      // blocks of 16 / 32: per 64 x 64 tile of the layout the ids of its blocks (-1: absent), see bsp_attention_fwd
   int64_t oin_sz, oin_sh, oin_ld;
   int64_t x_sz, x_sh, x_ld, y1_sz, y1_sh, y1_ld, y2_sz, y2_sh, y2_ld, o_sz, o_sh, o_ld, pin_sz, pout_sz;
   float scale;
@@ -146,7 +145,7 @@ template <typename T> __device__ __forceinline__ void store_block_rows(T *cs, T 
 
 // Blocks of 16 and 32 (SUBS = 64 / block > 1): the kernels work on 64 x 64 tiles formed from SUBS x SUBS small blocks
 // (SUBS consecutive block-rows by SUBS gathered block-columns, or the other way round in the column kernel); the table
-// lists the tiles of each line and `tiles` holds, per tile, the ids of its blocks row by row, -1 where absent.  A
+// lists the tiles of each line, each with the ids of its blocks row by row, -1 where absent.  A
 // wavefront's 16 rows lie in one row of small blocks (rs) and a lane's chunk of 8 columns in one small block: its id, or -1.
 // t = the ids of the wavefront's row of small blocks in the tile (scalars, fetched once per block of the row; kept as a
 // vector type: an array indexed in a select chain ends up in scratch memory, whose loads count as vector-memory
@@ -157,19 +156,21 @@ template <int SUBS> __device__ __forceinline__ int chunk_block_id(const i32x4 &t
   else if constexpr (SUBS == 4) return s ? ((q >> 1) ? t[3] : t[2]) : ((q >> 1) ? t[1] : t[0]);   // small block column 2s + q / 2
   else return 0;
 }
-template <int SUBS> __device__ __forceinline__ i32x4 load_block_ids(table_ptr tiles, int tile, int rs) {
+// the ids of the blocks of the tile's row rs of small blocks, from the tile's table entry (see entry_ints)
+template <int SUBS> __device__ __forceinline__ i32x4 entry_ids(table_ptr e, int rs) {
   i32x4 t = {0, 0, 0, 0};
   if constexpr (SUBS > 1) {
-    const table_ptr src = tiles + (int64_t)tile * (SUBS * SUBS) + rs * SUBS;
 #pragma unroll
-    for (int c = 0; c < SUBS; c++) t[c] = src[c];
+    for (int c = 0; c < SUBS; c++) t[c] = e[8 + rs * SUBS + c];
   }
   return t;
 }
 // Table entries.  Blocks of 64: four ints (block id, block-column [the column kernel: block-row], ., .).  Smaller
-// blocks: eight ints (tile, ., ., ., then the S block-columns [block-rows] gathered into the tile, S = SUBS): the tile's
-// 64 columns [rows] are S groups of 64 / S consecutive ones, each group anywhere in the matrix.
-template <int SUBS> constexpr int entry_ints() { return SUBS == 1 ? 4 : 8; }
+// blocks: 8 + S * S ints, S = SUBS: (., ., ., ., the S block-columns [block-rows] gathered into the tile, then the ids of
+// the tile's blocks, [block-row of the line][gathered block-column], -1 where absent): the tile's 64 columns [rows] are
+// S groups of 64 / S consecutive ones, each group anywhere in the matrix.  Everything a tile needs is in its entry: one
+// round of scalar loads, which the kernels issue a step ahead of the tile's loads.
+template <int SUBS> constexpr int entry_ints() { return SUBS == 1 ? 4 : 8 + SUBS * SUBS; }
 template <int SUBS> __device__ __forceinline__ int entry_group(table_ptr e, int g) { return SUBS == 1 ? e[1] : e[4 + g]; }
 template <int SUBS> __device__ __forceinline__ i32x4 entry_groups(table_ptr e) {
   i32x4 t = i32x4{0, 0, 0, 0};

@@ -96,7 +96,7 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   for (int b = 0; b < NB; b++) bid[b] = core[ES * (b < size ? b : 0)];   // blocks past the end repeat the first one (valid to read, never used)
   i32x4 tid_[NB];   // small blocks: the ids of the wavefront's row of small blocks in each tile
 #pragma unroll
-  for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+  for (int b = 0; b < NB; b++) tid_[b] = entry_ids<SUBS>(core + ES * (b < size ? b : 0), wgroup);
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   frag_t xq[NK];
 #pragma unroll
@@ -465,11 +465,11 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
   i32x4 tid_[KEEP_IDS ? NB : 1];
   if constexpr (KEEP_IDS) {
 #pragma unroll
-    for (int b = 0; b < NB; b++) tid_[b] = load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+    for (int b = 0; b < NB; b++) tid_[b] = entry_ids<SUBS>(core + ES * (b < size ? b : 0), wgroup);
   }
   auto ids_of = [&](int b) {
     if constexpr (KEEP_IDS) return tid_[b];
-    else return load_block_ids<SUBS>(as_table(a.tiles), bid[b], wgroup);
+    else return entry_ids<SUBS>(core + ES * (b < size ? b : 0), wgroup);
   };
   const T *px = reinterpret_cast<const T *>(a.x) + z * a.x_sz + h * a.x_sh + row * a.x_ld + 8 * q;
   const T *pof = reinterpret_cast<const T *>(a.o_in) + z * a.oin_sz + h * a.oin_sh + row * a.oin_ld + 8 * q;
@@ -534,7 +534,8 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd(AttnArgs a) {
 #pragma unroll
           for (int b2 = 1; b2 < NB; b2++) ids = (m == b2) ? tid_[b2] : ids;
         } else {
-          ids = load_block_ids<SUBS>(as_table(a.tiles), key, wgroup);
+          const int m = n >> 1;
+          ids = entry_ids<SUBS>(core + ES * (m < size ? m : size - 1), wgroup);
         }
 #pragma unroll
         for (int i = 0; i < LWP; i++) {
@@ -703,7 +704,6 @@ int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *st
   if (!a.x || !a.y1 || !a.y2 || (!bwd && !a.p_out) || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
     return BSP_ERR_ARG;
   if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
-  if ((block != 64) != (a.tiles != nullptr)) return BSP_ERR_ARG;   // the tile table goes with the small blocks, and only with them
   if ((int64_t)maxlut * 64 >= 32768) return BSP_ERR_ROW_TOO_LONG;   // the softmax operator's bound on a row (softmax.py:225-227)
   const bool is_long = maxlut > BSP_ATTENTION_MAX_ROW_BLOCKS;         // longer rows: streamed
   // 16-byte vector accesses everywhere: every pointer and every stride a multiple of 8 elements
@@ -735,7 +735,7 @@ extern "C" int bsp_attention_fwd(int dtype, const void *q, const void *k, const 
                                  int D, int64_t q_stride_z, int64_t q_stride_h, int64_t ldq, int64_t k_stride_z, int64_t k_stride_h,
                                  int64_t ldk, int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t o_stride_z,
                                  int64_t o_stride_h, int64_t ldo, int64_t p_stride_z, int block, float scale, const int32_t *d_lut,
-                                 int maxlut, const int32_t *d_tiles, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
+                                 int maxlut, const void *rpe, int64_t rpe_stride_z, int64_t rpe_stride_h, int64_t rpe_stride_r,
                                  const void *kpm, int64_t kpm_stride_z, int kpm_mul, const void *attn, int64_t attn_stride_r,
                                  int attn_mul, void *stream) {
   AttnArgs a{};
@@ -745,7 +745,7 @@ extern "C" int bsp_attention_fwd(int dtype, const void *q, const void *k, const 
   a.y2_sz = v_stride_z; a.y2_sh = v_stride_h; a.y2_ld = ldv;
   a.o_sz = o_stride_z; a.o_sh = o_stride_h; a.o_ld = ldo;
   a.pin_sz = 0; a.pout_sz = p_stride_z;
-  a.scale = scale; a.lut = d_lut; a.tiles = d_tiles;
+  a.scale = scale; a.lut = d_lut;
   a.rpe = rpe; a.rpe_sz = rpe_stride_z; a.rpe_sh = rpe_stride_h; a.rpe_sr = rpe_stride_r;
   a.kpm = kpm; a.kpm_sz = kpm_stride_z; a.kpm_mul = kpm_mul;
   a.attn = attn; a.attn_sr = attn_stride_r; a.attn_mul = attn_mul;
@@ -758,7 +758,7 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
                                  int64_t v_stride_z, int64_t v_stride_h, int64_t ldv, int64_t k_stride_z, int64_t k_stride_h,
                                  int64_t ldk, int64_t o_stride_z, int64_t o_stride_h, int64_t ldo, int64_t dq_stride_z,
                                  int64_t dq_stride_h, int64_t lddq, int64_t p_stride_z, int64_t ds_stride_z, int block, float scale,
-                                 const int32_t *d_lut, int maxlut, const int32_t *d_tiles, float *delta, int64_t delta_stride_h,
+                                 const int32_t *d_lut, int maxlut, float *delta, int64_t delta_stride_h,
                                  void *stream) {
   AttnArgs a{};
   a.x = d_o; a.y1 = v; a.y2 = k; a.p_in = p; a.p_out = ds; a.o = dq;
@@ -769,7 +769,7 @@ extern "C" int bsp_attention_bwd(int dtype, const void *d_o, const void *v, cons
   a.y2_sz = k_stride_z; a.y2_sh = k_stride_h; a.y2_ld = ldk;
   a.o_sz = dq_stride_z; a.o_sh = dq_stride_h; a.o_ld = lddq;
   a.pin_sz = p_stride_z; a.pout_sz = ds_stride_z;
-  a.scale = scale; a.lut = d_lut; a.tiles = d_tiles;
+  a.scale = scale; a.lut = d_lut;
   a.Z = Z; a.H = H; a.R = R;
   return run(dtype, a, D, block, maxlut, true, stream);
 }

@@ -71,10 +71,7 @@ __global__ void __launch_bounds__(256, 2) k_attn64_bwd_kv(AttnArgs a) {
   const T *py2 = reinterpret_cast<const T *>(a.y2) + z * a.y2_sz + h * a.y2_sh;   // q
   const T *pin = reinterpret_cast<const T *>(a.p_in) + z * a.pin_sz;
   const float *pdelta = a.delta + ((int64_t)z * a.H + h) * a.delta_sh;
-  // entries of the table: blocks of 64 four ints (id, block-row, ., .); smaller blocks 8 + SUBS * SUBS ints: (., ., ., ., the
-  // block-rows of the tile's SUBS groups of rows, then the ids of its blocks, [group of rows][block-column], -1 where
-  // absent).  Everything a tile needs comes from its entry, fetched a step ahead of its use.
-  constexpr int ES = SUBS == 1 ? 4 : 8 + SUBS * SUBS;
+  constexpr int ES = entry_ints<SUBS>();
   int64_t off1[LW], off2[LW];
   int offp[LWP], colp[LWP];
 #pragma unroll

@@ -93,8 +93,14 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
     const table_ptr e = core + ES * (m < size ? m : size - 1);
     return n % 3 == 1 ? e[0] : entry_group<SUBS>(e, rs) - rs;
   };
+  // (small blocks, with the key of a tile of p: the ids of the blocks it is gathered from)
+  auto tile_vec = [&](int n) {
+    const int m = n / 3;
+    return entry_ids<SUBS>(core + ES * (m < size ? m : size - 1), rs);
+  };
   int next_key;
-  auto issue = [&](int n, int key) {
+  i32x4 next_vec;
+  auto issue = [&](int n, int key, const i32x4 &ids) {
     unsigned char *st = ring + (n % kStages) * TB;
     const int kind = n % 3;
     if (kind == 1) {
@@ -104,7 +110,6 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
         for (int i = 0; i < LWP; i++)
           __builtin_amdgcn_global_load_lds(BSP_GLOBAL_PTR(base + offp[i]), BSP_LDS_PTR(st + (wave * LWP + i) * 1024), 16, 0, BSP_LOAD_ONCE);
       } else {
-        const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), key, rs);
 #pragma unroll
         for (int i = 0; i < LWP; i++) {
           int id = ids[0];
@@ -133,12 +138,14 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (n + kStages - 1 < total) issue(n + kStages - 1, next_key);
+    if (n + kStages - 1 < total) issue(n + kStages - 1, next_key, next_vec);
     next_key = tile_key(n + kStages);
+    next_vec = tile_vec(n + kStages);
   };
 #pragma unroll
-  for (int n = 0; n < kStages - 1; n++) issue(n, tile_key(n));   // (a row has at least one block: three tiles)
+  for (int n = 0; n < kStages - 1; n++) issue(n, tile_key(n), tile_vec(n));   // (a row has at least one block: three tiles)
   next_key = tile_key(kStages - 1);
+  next_vec = tile_vec(kStages - 1);
   float delta = 0.f;
 #pragma unroll
   for (int s2 = 0; s2 < NK; s2++)
@@ -158,7 +165,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
   T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
   for (int b = 0; b < size; b++) {
     const int tile_id = core[ES * b];
-    const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), tile_id, rs);
+    const i32x4 ids = entry_ids<SUBS>(core + ES * b, rs);
     step(3 * b);
     const unsigned char *tile = ring + ((3 * b) % kStages) * TB;
     frag_t kf[4][NK];
@@ -404,7 +411,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   float m_run = -INFINITY, l_run = 0.f;
   int any_block = SUBS == 1;
   for (int b = 0; b < size; b++) {
-    const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), core[ES * b], rs);
+    const i32x4 ids = entry_ids<SUBS>(core + ES * b, rs);
     if constexpr (SUBS > 1) any_block |= int(chunk_block_id<SUBS>(ids, 0, q) >= 0 || chunk_block_id<SUBS>(ids, 1, q) >= 0);
     P8 pr[2], pa[2];
     if constexpr (EXTRA) {
@@ -452,7 +459,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
   T *pz = reinterpret_cast<T *>(a.p_out) + z * a.pout_sz;
   for (int b = 0; b < size; b++) {
     const int tile_id = core[ES * b];
-    const i32x4 ids = load_block_ids<SUBS>(as_table(a.tiles), tile_id, rs);
+    const i32x4 ids = entry_ids<SUBS>(core + ES * b, rs);
     const int n = size + 2 * b;
     P8 pr[2], pa[2];
     if constexpr (EXTRA) {

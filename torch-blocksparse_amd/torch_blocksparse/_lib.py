@@ -63,9 +63,9 @@ SIGNATURES = {
     'bsp_softmax_dropout_fwd': (_i, [_i, _vp, _vp, _f, _vp, _i, _vp, _i64, _i64, _i64, _vp, _i64, _i, _vp, _i64, _i, _i, _i, _i, _i,
                                      _i64, _i64, _f, _c.c_uint64, _c.c_uint64, _vp]),
     'bsp_softmax_dropout_bwd': (_i, [_i, _vp, _vp, _f, _vp, _i, _i, _i, _i, _i, _i64, _i64, _f, _c.c_uint64, _c.c_uint64, _vp]),
-    'bsp_attention_fwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_i64] * 13 + [_i, _f, _vp, _i, _vp, _vp, _i64, _i64, _i64,
+    'bsp_attention_fwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_i64] * 13 + [_i, _f, _vp, _i, _vp, _i64, _i64, _i64,
                                 _vp, _i64, _i, _vp, _i64, _i, _vp]),
-    'bsp_attention_bwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_i64] * 17 + [_i, _f, _vp, _i, _vp, _vp, _i64, _vp]),
+    'bsp_attention_bwd': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_i64] * 17 + [_i, _f, _vp, _i, _vp, _i64, _vp]),
     'bsp_attention_bwd_kv': (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i] + [_i64] * 17 + [_i, _f, _vp, _i, _vp, _i, _vp, _i, _vp]),
     'bsp_layout_fixed': (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _i, _vp]),
     'bsp_layout_sparse_transformer': (_i, [_vp, _i, _i, _i, _i, _i, _vp]),

@@ -56,12 +56,15 @@ class _GatheredTiles:
             self.ids[tile, i, slot] = ids[h, t * S + i, c]
         self.lines, self.heads = L, H
 
-    def entries(self):
-        """per tile eight ints: (tile, 0, line, head, then the tile's block-columns, the last repeated up to four)"""
+    def entries(self, transposed_ids=False):
+        """per tile 8 + S * S ints: (tile, 0, line, head, then the tile's block-columns, the last repeated up to four, then
+        the ids of its blocks, [block-row of the line][gathered block-column], or the other way round)"""
         t = torch.arange(self.n_tiles)
         line = torch.repeat_interleave(torch.arange(self.heads * self.lines), self.sizes)
         cols = self.cols if self.cols.size(1) == 4 else torch.cat((self.cols, self.cols[:, -1:].expand(-1, 4 - self.cols.size(1))), 1)
-        return torch.cat((torch.stack((t, torch.zeros_like(t), line % self.lines, line // self.lines), 1), cols), 1)
+        ids = self.ids.transpose(1, 2) if transposed_ids else self.ids
+        return torch.cat((torch.stack((t, torch.zeros_like(t), line % self.lines, line // self.lines), 1), cols,
+                          ids.reshape(self.n_tiles, -1).to(torch.int64)), 1)
 
 
 KV_PART_BLOCKS = 16         # columns of more blocks than this (and than twice the average column) are computed in parts of about this size
@@ -99,8 +102,7 @@ class _ColumnTable:
             g = _GatheredTiles(torch.gather(layT, 1, pick), torch.gather(idsT, 1, pick), S)
             C = C // S
             # an entry carries the ids of its tile's blocks, [gathered block-row][block-column of the group]
-            sizes, starts = g.sizes, g.starts
-            entries = torch.cat((g.entries(), g.ids.transpose(1, 2).reshape(g.n_tiles, S * S).to(torch.int64)), 1)
+            sizes, starts, entries = g.sizes, g.starts, g.entries(transposed_ids=True)
             groups = order.reshape(H * C, S)
         groups = torch.cat((groups, groups[:, -1:].expand(-1, 4 - groups.size(1))), 1) if groups.size(1) < 4 else groups
         if part is None:
@@ -162,7 +164,7 @@ class AttentionCore:
         return self.nnz
 
     def tables(self, device):
-        """(table, longest row, tile table or None, rows of the table's layout, present blocks per present tile as a share,
+        """(table, longest row, None, rows of the table's layout, present blocks per present tile as a share,
         tables of the column kernel) on `device`, or None when the layout does not divide into 64 x 64 tiles."""
         key = str(device)
         if key not in self._tables:
@@ -180,12 +182,11 @@ class AttentionCore:
                 ids = torch.full(lay.shape, -1, dtype=torch.int32)
                 ids[lay] = torch.arange(int(lay.sum()), dtype=torch.int32)
                 g = _GatheredTiles(lay, ids, S)
-                header = torch.stack((g.sizes, 2 * g.sizes.numel() + 8 * g.starts), 1).reshape(-1)
+                header = torch.stack((g.sizes, 2 * g.sizes.numel() + (8 + S * S) * g.starts), 1).reshape(-1)
                 lut = torch.cat((header, g.entries().reshape(-1))).to(torch.int32).to(device)
                 maxlut = int(g.sizes.max()) if g.n_tiles else 0
                 ct = _ColumnTable(self.layout, device, S=S, ids=ids)
-                self._tables[key] = (lut, maxlut, g.ids.reshape(-1).to(torch.int32).to(device), R // S,
-                                     self.blocks() / max(1, g.n_tiles * S * S), ct)
+                self._tables[key] = (lut, maxlut, None, R // S, self.blocks() / max(1, g.n_tiles * S * S), ct)
         return self._tables[key]
 
     def usable(self, q, k, v, dropout_p=0.):
@@ -247,7 +248,7 @@ class _attention_core(torch.autograd.Function):
         rc = _lib.load().bsp_attention_fwd(
             _lib.DTYPES[q.dtype], _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(p), _lib.ptr(o), Z, H, rows, D,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
-            o.stride(0), o.stride(1), o.stride(2), p.stride(0), block, scale, _lib.ptr(lut), maxlut, _lib.ptr(tiles),
+            o.stride(0), o.stride(1), o.stride(2), p.stride(0), block, scale, _lib.ptr(lut), maxlut,
             rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3], kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
             attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'), _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_fwd')
@@ -268,7 +269,7 @@ class _attention_core(torch.autograd.Function):
             _lib.DTYPES[q.dtype], _lib.ptr(do), _lib.ptr(v), _lib.ptr(k), _lib.ptr(p), _lib.ptr(o), _lib.ptr(ds), _lib.ptr(dq), Z, H, ctx.rows, D,
             do.stride(0), do.stride(1), do.stride(2), v.stride(0), v.stride(1), v.stride(2), k.stride(0), k.stride(1), k.stride(2),
             o.stride(0), o.stride(1), o.stride(2), dq.stride(0), dq.stride(1), dq.stride(2), p.stride(0), ds.stride(0) if ds is not None else 0,
-            core.block, ctx.scale, _lib.ptr(lut), ctx.maxlut, _lib.ptr(ctx.tiles), _lib.ptr(delta), delta.stride(1) if delta is not None else 0,
+            core.block, ctx.scale, _lib.ptr(lut), ctx.maxlut, _lib.ptr(delta), delta.stride(1) if delta is not None else 0,
             _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_bwd')
         return dq
