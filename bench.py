@@ -426,7 +426,7 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants, block=64):
             with torch.no_grad():
                 state['o'] = ac._attention_core.forward(state.setdefault('ctx', _Ctx()), q, k, v, float(scale), kw.get('rpe'), kw.get('key_padding_mask'),
                                                         kw.get('attn_mask'), kw.get('key_padding_mask_mode', 'add'), kw.get('attn_mask_mode', 'add'),
-                                                        core, *core.tables(q.device)[:4])
+                                                        core, *_fwd_tables(core, q.device))
         ms = timeit(fwd)
         nbytes = 4 * dense + xb
         out.append({'launch': 'fused forward: q.k^T, softmax, p.v (%s)' % label, 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
@@ -452,6 +452,12 @@ def fused_chain_launches(lay, q, k, v, do, scale, timeit, variants, block=64):
                 'ms': round(ms, 4), 'GB/s': round(nbytes / ms * 1e-6, 1),
                 'hbm_frac': round(nbytes / ms * 1e-6 / HBM_PEAK_GBS, 4), 'roofline': launch_roofline('k_attn64_bwd_kv', 0, nbytes, ms)})
     return out
+
+
+def _fwd_tables(core, device, keep_p=True):
+    """the table arguments of _attention_core.forward: (table, longest row, keep p for a backward pass, rows)"""
+    lut, maxlut, _, rows = core.tables(device)[:4]
+    return lut, maxlut, keep_p, rows
 
 
 class _Ctx:

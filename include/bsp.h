@@ -286,7 +286,8 @@ int bsp_softmax_dropout_bwd(int dtype, const void *y, void *dy, float scale, con
  *             line.
  *   forward : p = softmax(round(q . k^T) * scale + rpe + kpm + attn) over each row's nonzero blocks, o = p . v.
  *             q, o: [Z, H, rows, D]; k, v: [Z, H, columns, D], unit stride along D; p: [Z, nnz, block, block] (every
- *             block is written); rows of o without any block are set to zero.  Masks as for bsp_softmax_fwd.
+ *             block is written), or NULL when no backward pass will follow: p is then not stored (most of the
+ *             kernel's traffic); rows of o without any block are set to zero.  Masks as for bsp_softmax_fwd.
  *   backward: ds = p * (round(do . v^T) - delta) * scale, dq = ds . k, with delta = sum_d do[row][d] * o[row][d], o
  *             the result of the forward call: in exact arithmetic this is the sum over the row of p * (do . v^T) that
  *             the softmax gradient subtracts (softmax.py:187-189), and it is known before the row's blocks are, so

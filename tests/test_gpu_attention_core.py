@@ -502,6 +502,11 @@ def test_backward_through_the_column_kernel_and_through_the_two_operators(block,
             assert_close(g, r, dtype, name)
 
 
+def _fwd_tables(core, device, keep_p=True):
+    lut, maxlut, _, rows = core.tables(device)[:4]
+    return lut, maxlut, keep_p, rows
+
+
 class _FakeCtx:
     """stand-in for the autograd context: the kernels of the backward pass called one by one"""
     needs_input_grad = (True, True, True)
@@ -524,7 +529,7 @@ def test_rows_kernel_outputs_in_every_combination(R, block):
     q, k, v, do = [torch.randn(Z, H, L, dh, device=DEV).half() for _ in range(4)]
     ctx = _FakeCtx()
     with torch.no_grad():
-        o = ac._attention_core.forward(ctx, q, k, v, 0.125, None, None, None, 'add', 'add', core, *core.tables(q.device)[:4])
+        o = ac._attention_core.forward(ctx, q, k, v, 0.125, None, None, None, 'add', 'add', core, *_fwd_tables(core, q.device))
         p = ctx.saved_tensors[3]
         outs = {}
         for want_ds in (False, True):
@@ -615,6 +620,30 @@ def test_fixed_layouts_of_the_module_at_small_blocks(cfg):
     for name, g, c, r in zip(('o', 'dq', 'dk', 'dv'), res[True], res[False], ref):
         assert float((g.float() - c.float()).abs().max()) <= CHAIN_TOL[torch.float16][1] * float(c.float().abs().max()), name
         assert_close(g, r, torch.float16, name)
+
+
+@pytest.mark.parametrize('block,R', [(64, 6), (64, 12), (16, 24)])
+def test_forward_without_a_backward_pass_does_not_store_p(block, R):
+    """Under no_grad, or when no operand asks for a gradient, the forward kernel gets no tensor for p (and allocates
+    none): the same o to the bit."""
+    torch.manual_seed(R)
+    Z, H, dh = 2, 2, 64
+    lay = torch.tril(torch.ones(H, R, R, dtype=torch.int64))
+    ops = (tb.MatMul(lay, block, 'sdd', trans_b=True), tb.Softmax(lay, block), tb.MatMul(lay, block, 'dsd'))
+    q, k, v = [torch.randn(Z, H, R * block, dh, device=DEV).half() for _ in range(3)]
+    kpm = (0.5 * torch.randn(Z, R * block, device=DEV)).half()
+    with_grad = ac.attention_chain(ops[0], ops[1], ops[2], q.clone().requires_grad_(True), k, v, scale=0.125, key_padding_mask=kpm)
+    assert with_grad.requires_grad
+    torch.cuda.synchronize()
+    nnz_bytes = Z * int(lay.sum()) * block * block * 2
+    before = torch.cuda.memory_allocated()
+    torch.cuda.reset_peak_memory_stats()
+    with torch.no_grad():
+        o1 = ac.attention_chain(ops[0], ops[1], ops[2], q.clone().requires_grad_(True), k, v, scale=0.125, key_padding_mask=kpm)
+    o2 = ac.attention_chain(ops[0], ops[1], ops[2], q, k, v, scale=0.125, key_padding_mask=kpm)       # nothing requires a gradient
+    torch.cuda.synchronize()
+    assert torch.cuda.max_memory_allocated() - before < nnz_bytes        # o and the clone of q, but no tensor of p's size
+    assert torch.equal(o1, with_grad.detach()) and torch.equal(o2, o1)
 
 
 def test_c_abi_argument_checks():

@@ -390,6 +390,7 @@ __global__ void __launch_bounds__(256, (EXTRA || D > 64) ? 2 : 3) k_attn64_fwd(A
   __builtin_amdgcn_s_barrier();                        // the ring is free: everybody is done reading the last tile
   asm volatile("" ::: "memory");
   store_rows<T, D>(cs, po, a.o_ld, o, lane);
+  if (a.p_out == nullptr) return;   // p is not asked for (a forward pass without a backward pass to follow)
 #pragma unroll
   for (int b = 0; b < NB; b++)
     if (b < size) {
@@ -701,7 +702,7 @@ template <typename T> int launch_t(const AttnArgs &a, int D, int block, int maxl
 bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
 
 int run(int dtype, AttnArgs &a, int D, int block, int maxlut, bool bwd, void *stream) {
-  if (!a.x || !a.y1 || !a.y2 || (!bwd && !a.p_out) || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
+  if (!a.x || !a.y1 || !a.y2 || !a.o || !a.lut || (bwd && (!a.p_in || !a.o_in)) || a.Z <= 0 || a.H <= 0 || a.R <= 0 || maxlut < 0)
     return BSP_ERR_ARG;
   if ((block != 64 && block != 32 && block != 16) || (dtype != BSP_F16 && dtype != BSP_BF16) || (D != 64 && D != 128)) return BSP_ERR_UNSUPPORTED;
   if ((int64_t)maxlut * 64 >= 32768) return BSP_ERR_ROW_TOO_LONG;   // the softmax operator's bound on a row (softmax.py:225-227)

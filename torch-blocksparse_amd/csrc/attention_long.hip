@@ -210,7 +210,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_bwd_long(AttnArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) o[j4 + j] = M::run(vf[j], pf[s], o[j4 + j]);
       }
-if (a.p_out == nullptr) continue;   // ds is not asked for
+    if (a.p_out == nullptr) continue;   // ds is not asked for
         if constexpr (SUBS == 1) {
       store_block_rows<T>(stage_p, pz + (int64_t)tile_id * 4096 + wave * 1024, __builtin_bit_cast(u32x4, pf[0]), __builtin_bit_cast(u32x4, pf[1]), lane);
     } else {
@@ -494,6 +494,7 @@ __global__ void __launch_bounds__(256, 3) k_attn64_fwd_long(AttnArgs a) {
 #pragma unroll
         for (int j = 0; j < 4; j++) o[j4 + j] = M::run(vf[j], pf[s], o[j4 + j]);
       }
+    if (a.p_out == nullptr) continue;   // p is not asked for
     if constexpr (SUBS == 1) {
       store_block_rows<T>(stage_p, pz + (int64_t)tile_id * 4096 + wave * 1024, __builtin_bit_cast(u32x4, pf[0]), __builtin_bit_cast(u32x4, pf[1]), lane);
     } else {

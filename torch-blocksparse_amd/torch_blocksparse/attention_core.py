@@ -212,15 +212,17 @@ class AttentionCore:
         for name, m in (('relative position embedding', rpe), ('Attention mask', attn_mask), ('Key padding mask', key_padding_mask)):
             if m is not None and m.dtype != q.dtype:      # softmax.py:348-353
                 raise ValueError('%s must be %s' % (name, q.dtype))
-        lut, maxlut, tiles, rows = self.tables(q.device)[:4]
+        lut, maxlut, _, rows = self.tables(q.device)[:4]
+        # p is kept for the backward pass; a forward pass that no backward pass can follow does not store it
+        keep_p = torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)
         return _attention_core.apply(q, k, v, float(scale), rpe, key_padding_mask, attn_mask, key_padding_mask_mode,
-                                     attn_mask_mode, self, lut, maxlut, tiles, rows)
+                                     attn_mask_mode, self, lut, maxlut, keep_p, rows)
 
 
 class _attention_core(torch.autograd.Function):
 
     @staticmethod
-    def forward(ctx, q, k, v, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode, core, lut, maxlut, tiles, rows):
+    def forward(ctx, q, k, v, scale, rpe, key_padding_mask, attn_mask, kp_mask_mode, attn_mask_mode, core, lut, maxlut, keep_p, rows):
         global fused_calls
         H, R, C = core.spdims
         Z, D, block = q.size(0), q.size(3), core.block
@@ -243,18 +245,18 @@ class _attention_core(torch.autograd.Function):
         if attn_mask is not None:                          # element (r, c), softmax.py:67-70, 283
             attn_mask = _sparse_softmax._strided16(attn_mask, 'attn_mask')
             attn_args = (_lib.ptr(attn_mask), attn_mask.stride(0))
-        p = torch.empty((Z, nnz, block, block), dtype=q.dtype, device=q.device)
+        p = torch.empty((Z, nnz, block, block), dtype=q.dtype, device=q.device) if keep_p else None
         o = torch.empty((Z, H, R * block, D), dtype=q.dtype, device=q.device)
         rc = _lib.load().bsp_attention_fwd(
             _lib.DTYPES[q.dtype], _lib.ptr(q), _lib.ptr(k), _lib.ptr(v), _lib.ptr(p), _lib.ptr(o), Z, H, rows, D,
             q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
-            o.stride(0), o.stride(1), o.stride(2), p.stride(0), block, scale, _lib.ptr(lut), maxlut,
+            o.stride(0), o.stride(1), o.stride(2), p.stride(0) if keep_p else 0, block, scale, _lib.ptr(lut), maxlut,
             rpe_args[0], rpe_args[1], rpe_args[2], rpe_args[3], kpm_args[0], kpm_args[1], int(kp_mask_mode == 'mul'),
             attn_args[0], attn_args[1], int(attn_mask_mode == 'mul'), _lib.stream_ptr(q.device))
         _lib.check(rc, 'bsp_attention_fwd')
         fused_calls += 1
         ctx.save_for_backward(q, k, v, p, o, lut)
-        ctx.core, ctx.scale, ctx.maxlut, ctx.tiles, ctx.rows = core, scale, maxlut, tiles, rows
+        ctx.core, ctx.scale, ctx.maxlut, ctx.rows = core, scale, maxlut, rows
         ctx.columns = core.tables(q.device)[5]
         return o
 
