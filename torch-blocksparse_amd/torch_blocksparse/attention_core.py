@@ -228,7 +228,8 @@ class _attention_core(torch.autograd.Function):
         Z, D, block = q.size(0), q.size(3), core.block
         nnz = core.blocks()
         # the masks against the layout, exactly as the softmax operator checks them (it takes every address from the table)
-        _sparse_softmax._check_shapes(torch.empty((Z, nnz, block, block), device='meta'), rpe, key_padding_mask, attn_mask, core.spdims, block, nnz)
+        if rpe is not None or key_padding_mask is not None or attn_mask is not None:
+            _sparse_softmax._check_shapes(torch.empty((Z, nnz, block, block), device='meta'), rpe, key_padding_mask, attn_mask, core.spdims, block, nnz)
         q, k, v = _vec(q), _vec(k), _vec(v)
         null = ctypes.c_void_p(0)
         rpe_args = (null, 0, 0, 0)
