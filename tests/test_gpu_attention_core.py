@@ -550,11 +550,13 @@ def test_rows_kernel_outputs_in_every_combination(R, block):
         assert float((g.float() - c.float()).abs().max()) <= 1.5e-3 * float(c.float().abs().max()), name
 
 
-@pytest.mark.parametrize('seed', range(32))
+@pytest.mark.parametrize('seed', list(range(32)) + [-s for s in range(1, 9)])
 def test_seeded_random_sweep_against_the_three_operators(seed):
     """Random layouts (square and rectangular, rows and columns from empty to long, tiles from full to mostly holes),
     block sizes, head dimensions, types and mask combinations: every kernel variant (rows in registers / streamed, with
     and without per-element masks, columns whole / in parts) against the three-operator chain."""
+    stored_gradient = seed < 0                             # negative seeds: dk and dv from the stored gradient and the two operators
+    seed = abs(seed) + (100 if stored_gradient else 0)
     g = torch.Generator().manual_seed(1000 + seed)
     rnd = lambda n: int(torch.randint(0, n, (1,), generator=g))
     block = (64, 32, 16)[rnd(3)]
@@ -584,7 +586,12 @@ def test_seeded_random_sweep_against_the_three_operators(seed):
         kw['rpe'] = (0.3 * torch.randn(H, Lq, Lk, generator=g)).to(DEV).to(dtype)
     if choice & 4:
         kw.update(attn_mask=(0.5 * torch.randn(Lq, Lk, generator=g)).to(DEV).to(dtype), attn_mask_mode='add')
-    got = _run(ops, q, k, v, do, True, **kw)
+    old_kv = ac.FUSED_KV
+    try:
+        ac.FUSED_KV = not stored_gradient
+        got = _run(ops, q, k, v, do, True, **kw)
+    finally:
+        ac.FUSED_KV = old_kv
     chain = _run(ops, q, k, v, do, False, **kw)
     tol = CHAIN_TOL[dtype]
     for name, a, c in zip(('o', 'dq', 'dk', 'dv'), got, chain):
