@@ -13,7 +13,7 @@ import os
 import torch
 
 from . import _lib
-from .matmul import MatMul, _LayoutOnDevice
+from .matmul import MatMul
 from .softmax import Softmax, _sparse_softmax
 
 FUSED = os.environ.get('BSP_FUSED_ATTENTION', '1') != '0'
